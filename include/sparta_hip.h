@@ -1,0 +1,219 @@
+/*
+ * sparta_hip.h - C ABI of libsparta_hip.so: the gfx950 (MI355X) device side of
+ * the block-sparse operator path.
+ *
+ * Conventions
+ *   - Every entry point returns int: 0 = ok, < 0 = argument error detected on
+ *     the host before any launch (SPX_E_*), > 0 = a hipError_t value.
+ *     spx_last_error() returns a thread-local message for the last failure.
+ *   - The library owns no device memory and never allocates any: every buffer,
+ *     workspaces included, is provided by the caller.  Work is enqueued on the
+ *     hipStream_t passed as `stream` (NULL = the default stream); no entry point
+ *     synchronises the device.
+ *   - All pointers are device pointers unless stated otherwise.  Tensors are
+ *     contiguous, row-major, with the batch as the slowest dimension.
+ *   - dtype: SPX_F32 / SPX_F16 / SPX_BF16.  Matmuls always accumulate in fp32.
+ *   - Index encodings are the reference's
+ *     (sparta/tesa/templates/block_compressed.cu.j2:138-170):
+ *       BCSR_idx int32 = (block_row << 16) | block_col, column-ascending per row
+ *       BCSC_idx int32 = (block_col << 16) | block_row, row-ascending per column
+ *       BCSC_idx int64 = (bcsr_pos << 32) | (block_col << 16) | block_row
+ *     Compressed values: [batch, nnz * BH * BW], block i at i*BH*BW, row-major
+ *     inside the block (block_compressed.cu.j2:188-193).
+ */
+#ifndef SPARTA_HIP_H_
+#define SPARTA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPX_VERSION 100
+
+enum spx_dtype { SPX_F32 = 0, SPX_F16 = 1, SPX_BF16 = 2 };
+enum spx_mode { SPX_SDD = 0, SPX_DSD = 1, SPX_DDS = 2 };
+/* how a kernel reads a block index array */
+enum spx_idx_kind {
+    SPX_IDX_BCSR_I32 = 0, /* (row<<16)|col ; value slot = position          */
+    SPX_IDX_BCSC_I32 = 1, /* (col<<16)|row ; value slot = position          */
+    SPX_IDX_BCSC_I64 = 2  /* (slot<<32)|(col<<16)|row ; slot = BCSR position */
+};
+enum spx_error {
+    SPX_OK = 0,
+    SPX_E_NULL = -1,      /* required pointer is NULL                   */
+    SPX_E_SHAPE = -2,     /* shape / divisibility / range violation     */
+    SPX_E_DTYPE = -3,     /* unsupported dtype                          */
+    SPX_E_ALIGN = -4,     /* pointer or stride not sufficiently aligned */
+    SPX_E_WORKSPACE = -5, /* workspace too small                        */
+    SPX_E_CONFIG = -6,    /* unknown mode / tile config / block size    */
+    SPX_E_NO_DEVICE = -7  /* library built without a usable device path */
+};
+
+typedef void* spx_stream_t; /* hipStream_t */
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char* spx_last_error(void);
+int spx_version(void);
+
+/* ------------------------------------------------------------------------ *
+ * BCSR / BCSC index build.
+ * Replaces BCSFunctionContext.build_indexes / _build_BCSR_indexes /
+ * _build_BCSC_indexes (sparta/tesa/block_compressed.py:242-309) and the
+ * bcs_index_1 / bcs_index_2 kernels (block_compressed.cu.j2:67-170), without
+ * the host round trip of block_compressed.py:255: nnz is left in device memory.
+ *
+ * mask      uint8 [H, W]; a block is live iff any byte of its tile is non-zero.
+ * row_ptr   int32 [H/BH + 1] or NULL; bcsr_idx int32 [cap] or NULL (both or none)
+ * col_ptr   int32 [W/BW + 1] or NULL; bcsc_idx int32/int64 [cap] or NULL
+ * bcsc_i64  non-zero: bcsc_idx is int64 and carries the BCSR position.
+ * nnz_dev   int32 [1]: receives the number of live blocks (may exceed cap;
+ *           entries beyond cap are not written).
+ * workspace spx_bcs_index_workspace_bytes(...) bytes, 256-byte aligned.
+ * ------------------------------------------------------------------------ */
+size_t spx_bcs_index_workspace_bytes(int H, int W, int BH, int BW);
+int spx_bcs_index(const uint8_t* mask, int H, int W, int BH, int BW,
+                  int32_t* row_ptr, int32_t* bcsr_idx,
+                  int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                  int32_t* nnz_dev, int cap,
+                  void* workspace, size_t workspace_bytes, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
+ * dense <-> compressed values.  Replace BCSFunctionContext.convert / inverse
+ * (block_compressed.py:311-358) and dense_to_bcs_val / bcs_val_to_dense
+ * (block_compressed.cu.j2:172-220); any element size in {1,2,4,8} bytes.
+ *
+ * nnz_bound  number of blocks to launch over (host nnz, or the idx capacity);
+ * nnz_dev    optional int32[1]: blocks at positions >= *nnz_dev are skipped.
+ * sparse_batch_stride  elements between consecutive batches of `sparse`.
+ * spx_bcs_scatter writes live tiles only: the caller zero-fills `dense` first.
+ * ------------------------------------------------------------------------ */
+int spx_bcs_gather(const void* dense, void* sparse, const void* idx, int idx_kind,
+                   int nnz_bound, const int32_t* nnz_dev, int batch, int H, int W,
+                   int BH, int BW, int elem_bytes, int64_t sparse_batch_stride,
+                   spx_stream_t stream);
+int spx_bcs_scatter(const void* sparse, void* dense, const void* idx, int idx_kind,
+                    int nnz_bound, const int32_t* nnz_dev, int batch, int H, int W,
+                    int BH, int BW, int elem_bytes, int64_t sparse_batch_stride,
+                    spx_stream_t stream);
+
+/* Row / column sums of compressed values (fp32 accumulate), used for the bias
+ * gradient of a compressed sparse-output matmul.  Replace
+ * BCSFunctionContext.row_sum / col_sum (block_compressed.py:360-403) and
+ * bcsr_val_sum_row / bcsr_val_sum_col (block_compressed.cu.j2:222-288).
+ * axis 0: result [batch, H] = sum over W;  axis 1: result [batch, W] = sum
+ * over H.  `result` must be zero-filled by the caller. idx as in spx_bcs_gather. */
+int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
+                int nnz, int batch, int H, int W, int BH, int BW, int dtype, int axis,
+                int64_t sparse_batch_stride, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
+ * Block-sparse matmul C = op(A) op(B) (+ bias), fp32 accumulate on MFMA.
+ * Replaces the launch closures of SparseMatMulKernel.update_func
+ * (sparta/specializer/kernels/matmul.py:151-188) and the six
+ * {sparta,openai}_sparse_matmul_{sdd,dsd,dds}.cuh.j2 templates.
+ *
+ * mode letters name A, B, C in that order (matmul.py:60-84):
+ *   SPX_SDD  A sparse: tile (BM,BK) BCSR if !transA, (BK,BM) BCSC if transA
+ *   SPX_DSD  B sparse: tile (BN,BK) BCSR if  transB, (BK,BN) BCSC if !transB
+ *   SPX_DDS  C sparse: tile (BM,BN) BCSR, one entry per live output block
+ * A is [batch,K,M] if transA else [batch,M,K]; B is [batch,N,K] if transB else
+ * [batch,K,N]; bias (optional) is [batch,N]; C is [batch,M,N].
+ * compressed != 0: the sparse tensor is [batch, nnz*tileH*tileW] compressed
+ * values with sparse_batch_stride elements between batches; otherwise it is
+ * stored dense and the index only selects tiles (a dense DDS output must be
+ * zero-filled by the caller; dead tiles are not written).
+ * ptr  row_ptr (BCSR) or col_ptr (BCSC); unused for DDS (may be NULL).
+ * idx / idx_kind  see spx_idx_kind.  nnz_bound / nnz_dev as in spx_bcs_gather
+ *                 (only DDS launches over blocks).
+ * tile_cfg  index into the tile-config table of the op (0 = default).
+ * ------------------------------------------------------------------------ */
+int spx_matmul(int mode, int dtype, int transA, int transB, int compressed,
+               const void* A, const void* B, const void* bias, void* C,
+               const int32_t* ptr, const void* idx, int idx_kind,
+               int nnz_bound, const int32_t* nnz_dev, int64_t sparse_batch_stride,
+               int batch, int M, int K, int N, int BM, int BK, int BN,
+               int tile_cfg, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
+ * Masked block-sparse softmax over the last axis.
+ * Replaces SparseSoftmaxForwardKernel.update_func / BackwardKernel.update_func
+ * (sparta/specializer/kernels/softmax.py:65-88,120-145) and
+ * sparta_sparse_softmax_{forward,backward}.cuh.j2.
+ *   y = exp((x - max_live) * inv_temperature) / sum_live, 0 on masked entries
+ *   and on fully masked rows.
+ *   grad_x = inv_temperature * (y*grad_y - y * sum_live(y*grad_y))
+ * x / y are [batch,H,W] (compressed == 0; only entries of live blocks are
+ * written, the caller zero-fills y) or [batch, nnz*BH*BW] (compressed != 0;
+ * every entry is written).  mask is uint8 in the same layout as one batch of x.
+ * batch_stride: elements between batches of x / y.
+ * ------------------------------------------------------------------------ */
+int spx_softmax_forward(int dtype, int compressed, const void* x, void* y,
+                        const int32_t* row_ptr, const int32_t* bcsr_idx,
+                        const uint8_t* mask, float inv_temperature,
+                        int batch, int H, int W, int BH, int BW,
+                        int64_t batch_stride, int tile_cfg, spx_stream_t stream);
+int spx_softmax_backward(int dtype, int compressed, const void* grad_y, const void* y,
+                         void* grad_x, const int32_t* row_ptr, const int32_t* bcsr_idx,
+                         const uint8_t* mask, float inv_temperature,
+                         int batch, int H, int W, int BH, int BW,
+                         int64_t batch_stride, int tile_cfg, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
+ * Fused block-sparse attention forward:
+ *   out = softmax_masked(q k^T * inv_temperature) v   per batch*head.
+ * One kernel for the three launches of SparseAttention.forward
+ * (sparta/specializer/operators/sparse_attention.py:76-80); the score matrix
+ * never reaches HBM.  q,out [batch,Nt,E]; k,v [batch,Ns,E]; BCSR index over
+ * (BH,BW) tiles of the [Nt,Ns] mask; mask optional uint8 [Nt,Ns] element mask
+ * (NULL = every element of a live block is live).
+ * ------------------------------------------------------------------------ */
+int spx_attention_forward(int dtype, const void* q, const void* k, const void* v, void* out,
+                          const int32_t* row_ptr, const int32_t* bcsr_idx,
+                          const uint8_t* mask, float inv_temperature,
+                          int batch, int Nt, int Ns, int E, int BH, int BW,
+                          int tile_cfg, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
+ * MoE sparse forward: out[t,:] = tokens[t,:] . W[exp_ids[t]].
+ * Replace sparse_moe_cpp.convert_index / forward
+ * (csrc/moe_sparse_forward.cpp:7-25, csrc/moe_sparse_forward_kernel.cu.j2:58-116,
+ * :120-325, :363-483) with a stable counting sort (no per-expert capacity) and a
+ * gathered GEMM over a flattened (expert, row-tile) list.
+ *   exp_ids int32 [n_tok]; expert_count int32 [n_exp];
+ *   expert_offset int32 [n_exp+1] exclusive prefix; token_perm int32 [n_tok]:
+ *   token_perm[expert_offset[e] + j] = j-th token (ascending) routed to e.
+ *   tokens [n_tok,in_dim]; weight [n_exp,in_dim,out_dim]; out [n_tok,out_dim].
+ * ------------------------------------------------------------------------ */
+int spx_moe_index(const int32_t* exp_ids, int n_tok, int n_exp,
+                  int32_t* expert_count, int32_t* expert_offset, int32_t* token_perm,
+                  spx_stream_t stream);
+int spx_moe_forward(int dtype, const void* tokens, const void* weight, void* out,
+                    const int32_t* expert_offset, const int32_t* token_perm,
+                    int n_tok, int in_dim, int out_dim, int n_exp,
+                    int tile_cfg, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
+ * Tile-configuration table searched by tune(); replaces the Jinja template
+ * parameters and look_up_tables/sparta_matmul_lut.csv.
+ * op: 0 sdd/dsd matmul, 1 dds matmul, 2 softmax, 3 attention, 4 moe.
+ * ------------------------------------------------------------------------ */
+typedef struct spx_tile_cfg {
+    int id;
+    int tile_m;        /* output rows per workgroup (dense dimension)       */
+    int tile_n;        /* output cols per workgroup (0 = the sparse block)  */
+    int waves;         /* wavefronts per workgroup                          */
+    int lds_stages;    /* LDS staging depth                                 */
+    int min_block;     /* smallest sparse block edge the config accepts     */
+    int dtype_mask;    /* bit i set: spx_dtype i supported                  */
+    char name[32];
+} spx_tile_cfg;
+int spx_num_tile_cfgs(int op);
+int spx_tile_cfg_info(int op, int id, spx_tile_cfg* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARTA_HIP_H_ */

@@ -1,0 +1,102 @@
+// Shared host/device helpers for libsparta_hip (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/sparta_hip.h"
+
+namespace spx {
+
+// ---- error reporting -------------------------------------------------------
+char* last_error_buf();  // thread-local, 512 bytes
+inline int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(last_error_buf(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+inline int hip_fail(hipError_t e, const char* what) {
+    snprintf(last_error_buf(), 512, "%s: %s", what, hipGetErrorString(e));
+    return (int)e > 0 ? (int)e : 1;
+}
+
+#define SPX_REQUIRE(cond, code, ...) \
+    do { if (!(cond)) return ::spx::fail((code), __VA_ARGS__); } while (0)
+#define SPX_LAUNCH_CHECK(name) \
+    do { hipError_t e__ = hipGetLastError(); \
+         if (e__ != hipSuccess) return ::spx::hip_fail(e__, name); } while (0)
+
+inline bool is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+inline int ilog2(int x) { int l = 0; while ((1 << l) < x) ++l; return l; }
+inline bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+inline bool valid_block_edge(int b) { return b >= 4 && b <= 256 && is_pow2(b); }
+inline int dtype_bytes(int dtype) { return dtype == SPX_F32 ? 4 : 2; }
+
+// ---- device helpers ---------------------------------------------------------
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct alignas(16) vec16 { uint32_t x, y, z, w; };
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+__device__ __forceinline__ float bf16_to_float(uint16_t v) {
+    return __uint_as_float(((uint32_t)v) << 16);
+}
+__device__ __forceinline__ uint16_t float_to_bf16(float f) {  // round to nearest even
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// Storage types: f32 -> float, f16 -> _Float16, bf16 -> uint16_t wrapper.
+struct bf16_t { uint16_t v; };
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int dtype = SPX_F32;
+    __device__ static float to_float(float v) { return v; }
+    __device__ static float from_float(float v) { return v; }
+};
+template <> struct Elem<_Float16> {
+    static constexpr int dtype = SPX_F16;
+    __device__ static float to_float(_Float16 v) { return (float)v; }
+    __device__ static _Float16 from_float(float v) { return (_Float16)v; }
+};
+template <> struct Elem<bf16_t> {
+    static constexpr int dtype = SPX_BF16;
+    __device__ static float to_float(bf16_t v) { return bf16_to_float(v.v); }
+    __device__ static bf16_t from_float(float v) { bf16_t r; r.v = float_to_bf16(v); return r; }
+};
+
+// Inclusive prefix sum across the 64 lanes of a wavefront.
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int t = __shfl_up(v, d, 64);
+        if (lane >= d) v += t;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_reduce_max(float v) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v = fmaxf(v, __shfl_xor(v, d, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_reduce_sum(float v) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d, 64);
+    return v;
+}
+
+}  // namespace spx

@@ -1,0 +1,9 @@
+// bf16 instantiations of the sparse-output matmul kernel.
+#include "matmul_dds.hpp"
+namespace spx {
+template <>
+int launch_dds<bf16_t>(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, int tile_cfg, hipStream_t st) {
+    (void)tile_cfg;
+    return launch_dds_impl<bf16_t>(p, BM, BN, nnz_bound, batch, st);
+}
+}  // namespace spx

@@ -1,0 +1,8 @@
+// bf16 instantiations of the sparse-operand matmul kernel.
+#include "matmul_spmm.hpp"
+namespace spx {
+template <>
+int launch_spmm<bf16_t>(const SpmmParams& p, int BN, int batch, int tile_cfg, hipStream_t st) {
+    return launch_spmm_impl<bf16_t>(p, BN, batch, tile_cfg, st);
+}
+}  // namespace spx

@@ -1,0 +1,3 @@
+from sparta_amd.specializer.operators import (
+    OperatorBase, SparseLinear, SparseBatchMatMul, SparseSoftmax, SparseAttention, DynamicSparseMoE,
+)

@@ -1,0 +1,177 @@
+"""Sparse attention operator softmax_masked(Q K^T / sqrt(E)) V
+(interface of sparta/specializer/operators/sparse_attention.py:14-238).
+
+It is assembled from three sparse operators that share one BCSR index and one
+compressed layout: a sparse-output matmul for Q K^T, the masked softmax, and a
+sparse-input matmul for P V.  When no gradient is required the forward pass runs
+the fused kernel instead (spx_attention_forward), which keeps the scores in
+registers / LDS and never writes them to HBM.
+"""
+import warnings
+from typing import Any, Dict, List, Optional
+
+import numpy as np
+import torch
+
+from sparta_amd import _lib
+from sparta_amd.specializer.operators.operator_base import OperatorBase
+from sparta_amd.specializer.operators.sparse_matmul import SparseBatchMatMul
+from sparta_amd.specializer.operators.sparse_softmax import SparseSoftmax
+from sparta_amd.specializer.kernels import KernelBase, PortConfig
+
+# operator-level name -> (attribute, sparse port of that operator)
+_PARTS = (('qk', '_matmul_qk', 'C'), ('sm', '_softmax', 'y'), ('out', '_matmul_out', 'A'))
+
+
+class SparseAttention(OperatorBase):
+    r"""Args:
+        mask: (N_target, N_source) mask of the score entries that take part.
+        fused: run the single fused forward kernel when autograd is not recording
+            (default True).  The three-operator pipeline is always built as well and
+            is used whenever gradients are needed.
+
+    Shape: query (B*H, N_target, E), key / value (B*H, N_source, E) -> (B*H, N_target, E).
+    """
+
+    def __init__(self, mask: torch.Tensor, fused: bool = True):
+        super().__init__()
+        self.mask = mask
+        self._Nt, self._Ns = mask.shape
+        self._matmul_qk = SparseBatchMatMul(C_mask=mask, transpose_A=False, transpose_B=True, compressed=True)
+        self._softmax = SparseSoftmax(mask=mask, compressed=True)
+        self._matmul_out = SparseBatchMatMul(A_mask=mask, transpose_A=False, transpose_B=False, compressed=True)
+        self._sparse_port: Optional[PortConfig] = None
+        self._fused = fused
+        self._inv_temperature = 1.0
+        self.ready = False
+
+    def _parts(self):
+        return [(name, getattr(self, attr), port) for name, attr, port in _PARTS]
+
+    # ---- forward ---------------------------------------------------------------------
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
+        if self.ready and self._fused and not (
+                torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)):
+            return self._fused_forward(query, key, value)
+        scores = self._matmul_qk.forward(query, key)
+        probs = self._softmax.forward(scores)
+        return self._matmul_out.forward(probs, value)
+
+    def _fused_forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
+        indexes = self._sparse_port.indexes
+        lead = query.shape[:-2]
+        E = query.shape[-1]
+        batch = int(np.prod(lead)) if len(lead) else 1
+        q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
+        out = torch.empty_like(q)
+        rc = _lib.load().spx_attention_forward(
+            _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
+            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(indexes.raw_mask),
+            float(self._inv_temperature), batch, self._Nt, self._Ns, E,
+            indexes.block_H, indexes.block_W, 0, _lib.current_stream(q.device))
+        _lib.check(rc, 'spx_attention_forward')
+        return out
+
+    # ---- masks -----------------------------------------------------------------------
+    def update_mask(self, mask: torch.Tensor):
+        self.mask = mask
+        if self.ready:
+            self._sparse_port.set_mask(mask)
+            for _, op, _ in self._parts():
+                op._sparse_ctx.update_func()
+        else:
+            for _, op, _ in self._parts():
+                for ports in op._sparse_ctx.sparse_ports.values():
+                    for port in ports:
+                        port.set_mask(mask)
+
+    # ---- build -----------------------------------------------------------------------
+    def _check_qkv(self, query, key, value):
+        qB, kB, vB = (int(np.prod(t.shape[:-2])) for t in (query, key, value))
+        (qN, qE), (kN, kE), (vN, vE) = (t.shape[-2:] for t in (query, key, value))
+        assert qB == kB == vB, 'query, key and value should have the same batch size'
+        assert qN == self._Nt, f'expect query shape (?, {self._Nt}, ?), got {tuple(query.shape)}'
+        assert kN == self._Ns, f'expect key shape (?, {self._Ns}, ?), got {tuple(key.shape)}'
+        assert vN == self._Ns, f'expect value shape (?, {self._Ns}, ?), got {tuple(value.shape)}'
+        assert qE == kE == vE, 'query, key and value should have the same embed dim'
+        return qE
+
+    def _set_temperature(self, E: int):
+        self._softmax.set_temperature(np.sqrt(E))
+        self._inv_temperature = 1.0 / float(np.sqrt(E))
+
+    def build(self, config: Dict[str, Any], sample_inputs: List[torch.Tensor]):
+        query, key, value = sample_inputs
+        self._set_temperature(self._check_qkv(query, key, value))
+        with warnings.catch_warnings():
+            warnings.simplefilter('ignore')
+            scores = self._matmul_qk.forward(query, key)
+            probs = self._softmax.forward(scores)
+        part_inputs = {'qk': [query, key], 'sm': [scores], 'out': [probs, value]}
+
+        # One port (hence one index and one compressed layout) for every selected kernel.
+        shared: Optional[PortConfig] = None
+        for name, op, op_port in self._parts():
+            for kernel_name, placeholder in op._sparse_ctx.get_kernel_placeholders().items():
+                kernel: KernelBase = placeholder.possible_kernels[config[f'{name}/{kernel_name}']['_impl']]
+                kernel_port = placeholder.port_map[op_port]
+                if shared is None:
+                    shared = kernel.ports[kernel_port]
+                else:
+                    shared.connect(kernel, kernel_port)
+        self._sparse_port = shared
+
+        for name, op, _ in self._parts():
+            prefix = f'{name}/'
+            op.build(config={k[len(prefix):]: v for k, v in config.items() if k.startswith(prefix)},
+                     sample_inputs=part_inputs[name])
+        self.ready = True
+
+    def set_sample_inputs(self, sample_inputs: List[torch.Tensor],
+                          sample_grads: Optional[List[torch.Tensor]] = None):
+        query, key, value = sample_inputs
+        self._set_temperature(query.shape[-1])
+        need_grad = sample_grads is not None
+        if need_grad:
+            query, key, value = (t.detach().requires_grad_(True) for t in (query, key, value))
+        with warnings.catch_warnings():
+            warnings.simplefilter('ignore')
+            scores = self._matmul_qk.forward(query, key)
+            probs = self._softmax.forward(scores)
+            grad_scores = grad_probs = None
+            if need_grad:
+                scores.retain_grad()
+                probs.retain_grad()
+                self._matmul_out.forward(probs, value).backward(sample_grads[0])
+                grad_scores, grad_probs = [scores.grad], [probs.grad]
+                query, key, value = query.detach(), key.detach(), value.detach()
+        self._matmul_qk.set_sample_inputs([query, key], grad_scores)
+        self._softmax.set_sample_inputs([scores], grad_probs)
+        self._matmul_out.set_sample_inputs([probs, value], sample_grads)
+
+    # ---- tuning support ----------------------------------------------------------------
+    @staticmethod
+    def _prefixed(parts: Dict[str, Dict[str, Any]], backward: bool):
+        return {
+            f'{name}/{kernel}': value
+            for name in ('qk', 'sm', 'out')
+            for kernel, value in parts[name].items()
+            if backward or kernel.startswith('forward')
+        }
+
+    def get_search_space(self, backward: bool = False):
+        return self._prefixed({name: op.get_search_space(backward=True) for name, op, _ in self._parts()},
+                              backward)
+
+    def get_connections(self, backward: bool = False):
+        """The block shape of the score matrix is shared by all three operators,
+        whether or not backward kernels are tuned."""
+        per_op = [op.get_connections(backward=True) for _, op, _ in self._parts()]
+        return [
+            self._prefixed(dict(zip(('qk', 'sm', 'out'), axis)), backward)
+            for axis in zip(*per_op)
+        ]
+
+    def get_kernel_placeholders(self, backward: bool = False):
+        return self._prefixed({name: op.get_kernel_placeholders(backward=True) for name, op, _ in self._parts()},
+                              backward)

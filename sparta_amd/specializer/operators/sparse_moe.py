@@ -1,0 +1,61 @@
+"""Dynamic sparse mixture-of-experts forward: every token is multiplied by the
+weight of the expert it is routed to (interface of
+sparta/specializer/operators/sparse_moe.py:11-35).
+
+The token -> expert index is rebuilt on the GPU at every call by a stable
+counting sort (no per-expert capacity limit, no host synchronisation) and the
+per-expert products run as one gathered GEMM over a flattened list of
+(expert, row tile) work items, so skewed routing does not leave workgroups idle.
+"""
+from typing import List
+
+import torch
+
+from sparta_amd import _lib
+
+
+class DynamicSparseMoE(torch.nn.Module):
+    """Args:
+        exp_modules: one bias-free torch.nn.Linear per expert, all of one shape.
+
+    forward(tokens [n_tok, in], exp_ids int32 [n_tok]) -> [n_tok, out].
+    """
+
+    def __init__(self, exp_modules: List[torch.nn.Linear]):
+        super().__init__()
+        _lib.load()
+        self.num_exps = len(exp_modules)
+        self.out_hidden, self.in_hidden = exp_modules[0].weight.shape
+        self.device = exp_modules[0].weight.device
+        with torch.no_grad():
+            # [n_exp, in, out]: each expert's weight transposed once, up front
+            stacked = torch.stack([m.weight.t() for m in exp_modules]).contiguous()
+        self.weight = torch.nn.Parameter(stacked)
+        i32 = dict(dtype=torch.int32, device=self.device)
+        self.expert_count = torch.zeros(self.num_exps, **i32)
+        self.expert_offset = torch.zeros(self.num_exps + 1, **i32)
+        self.sparse_index = torch.zeros(0, **i32)  # token permutation, sized at first call
+
+    def forward(self, tokens: torch.Tensor, exp_ids: torch.Tensor):
+        n_tok = tokens.shape[0]
+        assert tokens.shape[1] == self.in_hidden, \
+            f'expected tokens of width {self.in_hidden}, got {tuple(tokens.shape)}'
+        assert exp_ids.shape[0] == n_tok, 'one expert id per token is required'
+        if exp_ids.dtype != torch.int32:
+            exp_ids = exp_ids.to(torch.int32)
+        if self.sparse_index.numel() < n_tok:
+            self.sparse_index = torch.empty(n_tok, dtype=torch.int32, device=tokens.device)
+        lib = _lib.load()
+        stream = _lib.current_stream(tokens.device)
+        rc = lib.spx_moe_index(_lib.dev_ptr(exp_ids.contiguous()), n_tok, self.num_exps,
+                               _lib.dev_ptr(self.expert_count), _lib.dev_ptr(self.expert_offset),
+                               _lib.dev_ptr(self.sparse_index), stream)
+        _lib.check(rc, 'spx_moe_index')
+        tokens = tokens.contiguous()
+        out = torch.empty((n_tok, self.out_hidden), dtype=tokens.dtype, device=tokens.device)
+        rc = lib.spx_moe_forward(_lib.dtype_code(tokens.dtype), _lib.dev_ptr(tokens),
+                                 _lib.dev_ptr(self.weight.detach()), _lib.dev_ptr(out),
+                                 _lib.dev_ptr(self.expert_offset), _lib.dev_ptr(self.sparse_index),
+                                 n_tok, self.in_hidden, self.out_hidden, self.num_exps, 0, stream)
+        _lib.check(rc, 'spx_moe_forward')
+        return out

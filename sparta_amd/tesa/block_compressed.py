@@ -1,0 +1,278 @@
+"""Block-compressed (BCSR / BCSC / both) indexes on the GPU.
+
+Host side of the index builder and of the dense<->compressed converters; the
+device side is libsparta_hip (spx_bcs_index / spx_bcs_gather / spx_bcs_scatter /
+spx_bcs_sum).  Mirrors the classes and attributes of
+sparta/tesa/block_compressed.py:23-413 with two deliberate differences:
+
+* entries are in canonical order (columns ascending inside a block-row for
+  BCSR, rows ascending inside a block-column for BCSC) - one of the orders the
+  reference's atomics may produce, but the same on every run;
+* the number of live blocks stays on the device after a build.  `block_nnz`,
+  `nnz`, `BCSR_idx` and `BCSC_idx` fetch it on first use (one synchronisation,
+  cached), kernels that only walk `row_ptr` / `col_ptr` never need it.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import numpy as np
+import torch
+
+from sparta_amd import _lib
+from sparta_amd.tesa.tesa_base import TeSAIndexes, TeSAFunctionContext
+
+_VALID_EDGES = (4, 8, 16, 32, 64, 128, 256)
+
+
+class BCSIndexes(TeSAIndexes):
+    """Common part of the three index flavours."""
+
+    #: which array orders the compressed values ('bcsr' or 'bcsc')
+    _value_order = 'bcsr'
+
+    def __init__(self, function_context: 'BCSFunctionContext', raw_mask: torch.Tensor,
+                 block_H: int, block_W: int, nnz_dev: torch.Tensor, capacity: int):
+        super().__init__(function_context, raw_mask)
+        self.block_H = block_H
+        self.block_W = block_W
+        self.H, self.W = raw_mask.shape
+        self.row_num = self.H // block_H
+        self.col_num = self.W // block_W
+        self.capacity = capacity
+        self.nnz_dev = nnz_dev
+        self._block_nnz: Optional[int] = None
+
+    # ---- live block count ----------------------------------------------------
+    @property
+    def block_nnz(self) -> int:
+        if self._block_nnz is None:
+            self._block_nnz = int(self.nnz_dev.item())
+        return self._block_nnz
+
+    @property
+    def nnz(self) -> np.int32:
+        return np.int32(self.block_nnz)
+
+    # ---- decoding --------------------------------------------------------------
+    def _value_index(self) -> Tuple[torch.Tensor, int]:
+        """(index buffer at capacity, idx_kind) that orders compressed values."""
+        raise NotImplementedError
+
+    def block_coordinates(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(block_row, block_col) int64 tensors in value order."""
+        raise NotImplementedError
+
+    def get_block_mask(self) -> torch.Tensor:
+        """Rebuild the uint8 [row_num, col_num] block mask from the index."""
+        rows, cols = self.block_coordinates()
+        grid = torch.zeros((self.row_num, self.col_num), dtype=torch.uint8, device=rows.device)
+        grid[rows, cols] = 1
+        return grid
+
+    def get_mask(self) -> torch.Tensor:
+        grid = self.get_block_mask()
+        full = grid.repeat_interleave(self.block_H, dim=0).repeat_interleave(self.block_W, dim=1)
+        return full.contiguous()
+
+    # ---- values ------------------------------------------------------------------
+    def convert(self, dense: torch.Tensor) -> torch.Tensor:
+        """Dense [..., H, W] -> compressed [..., nnz*block_H*block_W]."""
+        idx, kind = self._value_index()
+        return self.function_context.convert(dense, idx, self.block_nnz, self.H, self.W, idx_kind=kind)
+
+    def inverse(self, sparse_val: torch.Tensor) -> torch.Tensor:
+        """Compressed [..., nnz*block_H*block_W] -> zero-filled dense [..., H, W]."""
+        idx, kind = self._value_index()
+        return self.function_context.inverse(sparse_val, idx, self.block_nnz, self.H, self.W, idx_kind=kind)
+
+    def sum(self, sparse_val: torch.Tensor, axis: int = -1) -> torch.Tensor:
+        """Sum compressed values along a dense axis (-1: over W, -2: over H)."""
+        from_end = -axis if axis < 0 else sparse_val.dim() + 1 - axis
+        if from_end not in (1, 2):
+            raise ValueError(f'axis #{axis} is not sparsed, please use torch.sum() instead.')
+        idx, kind = self._value_index()
+        return self.function_context.block_sum(
+            sparse_val, idx, kind, self.block_nnz, self.H, self.W, axis=0 if from_end == 1 else 1)
+
+
+class BCSRIndexes(BCSIndexes):
+    """row_ptr + BCSR_idx, BCSR_idx = (block_row << 16) | block_col."""
+
+    def __init__(self, function_context, raw_mask, row_ptr, bcsr_buf, nnz_dev, block_H, block_W):
+        super().__init__(function_context, raw_mask, block_H, block_W, nnz_dev, bcsr_buf.numel())
+        self.row_ptr = row_ptr
+        self._bcsr_buf = bcsr_buf
+
+    @property
+    def BCSR_idx(self) -> torch.Tensor:
+        return self._bcsr_buf[:self.block_nnz]
+
+    def _value_index(self):
+        return self._bcsr_buf, _lib.IDX_BCSR_I32
+
+    def block_coordinates(self):
+        code = self.BCSR_idx.to(torch.int64)
+        return code >> 16, code & 0xffff
+
+
+class BCSCIndexes(BCSIndexes):
+    """col_ptr + BCSC_idx, BCSC_idx = (block_col << 16) | block_row (int32)."""
+
+    _value_order = 'bcsc'
+
+    def __init__(self, function_context, raw_mask, col_ptr, bcsc_buf, nnz_dev, block_H, block_W):
+        super().__init__(function_context, raw_mask, block_H, block_W, nnz_dev, bcsc_buf.numel())
+        self.col_ptr = col_ptr
+        self._bcsc_buf = bcsc_buf
+
+    @property
+    def BCSC_idx(self) -> torch.Tensor:
+        return self._bcsc_buf[:self.block_nnz]
+
+    def _value_index(self):
+        return self._bcsc_buf, _lib.IDX_BCSC_I32
+
+    def block_coordinates(self):
+        code = self.BCSC_idx.to(torch.int64)
+        return code & 0xffff, (code >> 16) & 0xffff
+
+
+class BCSRCIndexes(BCSRIndexes):
+    """Both orders; values follow the BCSR order and the int64 BCSC_idx carries
+    the BCSR position of each block in its upper half."""
+
+    def __init__(self, function_context, raw_mask, row_ptr, col_ptr, bcsr_buf, bcsc_buf, nnz_dev,
+                 block_H, block_W):
+        super().__init__(function_context, raw_mask, row_ptr, bcsr_buf, nnz_dev, block_H, block_W)
+        self.col_ptr = col_ptr
+        self._bcsc_buf = bcsc_buf
+
+    @property
+    def BCSC_idx(self) -> torch.Tensor:
+        return self._bcsc_buf[:self.block_nnz]
+
+
+class BCSFunctionContext(TeSAFunctionContext):
+    """Index builder / converter for one (block_H, block_W, BCSR, BCSC) choice."""
+
+    def __init__(self, block_H: int, block_W: int, BCSR: bool, BCSC: bool):
+        assert block_H in _VALID_EDGES, f'invalid block height {block_H}'
+        assert block_W in _VALID_EDGES, f'invalid block width {block_W}'
+        assert BCSR or BCSC, 'at least one of BCSR / BCSC is required'
+        _lib.load()
+        self._block_H = block_H
+        self._block_W = block_W
+        self._block_size = block_H * block_W
+        self._BCSR = BCSR
+        self._BCSC = BCSC
+        self._workspaces: Dict[Tuple[int, int, str], torch.Tensor] = {}
+
+    # ---- index build ------------------------------------------------------------
+    def _workspace(self, H: int, W: int, device) -> torch.Tensor:
+        key = (H, W, str(device))
+        ws = self._workspaces.get(key)
+        if ws is None:
+            nbytes = _lib.load().spx_bcs_index_workspace_bytes(H, W, self._block_H, self._block_W)
+            assert nbytes > 0, f'mask shape ({H}, {W}) does not fit block ({self._block_H}, {self._block_W})'
+            ws = torch.empty((nbytes,), dtype=torch.uint8, device=device)
+            self._workspaces[key] = ws
+        return ws
+
+    def build_indexes(self, mask: torch.Tensor, capacity: Optional[int] = None) -> BCSIndexes:
+        """mask: uint8 (or any 1-byte dtype) [H, W] on the GPU.  `capacity` bounds the
+        number of index entries kept (default: every block)."""
+        assert mask.dim() == 2, 'only 2D mask is supported'
+        if mask.dtype != torch.uint8:
+            mask = (mask != 0).to(torch.uint8)
+        mask = mask.contiguous()
+        H, W = mask.shape
+        BH, BW = self._block_H, self._block_W
+        assert H % BH == 0 and W % BW == 0, f'mask shape ({H}, {W}) does not fit block ({BH}, {BW})'
+        R, Cn = H // BH, W // BW
+        cap = R * Cn if capacity is None else int(capacity)
+        dev = mask.device
+        i32 = dict(dtype=torch.int32, device=dev)
+        nnz_dev = torch.empty((1,), **i32)
+        row_ptr = bcsr = col_ptr = bcsc = None
+        if self._BCSR:
+            row_ptr = torch.empty((R + 1,), **i32)
+            bcsr = torch.empty((cap,), **i32)
+        both = self._BCSR and self._BCSC
+        if self._BCSC:
+            col_ptr = torch.empty((Cn + 1,), **i32)
+            bcsc = torch.empty((cap,), dtype=torch.int64 if both else torch.int32, device=dev)
+        ws = self._workspace(H, W, dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().spx_bcs_index(
+                _lib.dev_ptr(mask), H, W, BH, BW,
+                _lib.dev_ptr(row_ptr), _lib.dev_ptr(bcsr), _lib.dev_ptr(col_ptr), _lib.dev_ptr(bcsc),
+                1 if both else 0, _lib.dev_ptr(nnz_dev), cap, _lib.dev_ptr(ws), ws.numel(),
+                _lib.current_stream(dev))
+        _lib.check(rc, 'spx_bcs_index')
+        if both:
+            return BCSRCIndexes(self, mask, row_ptr, col_ptr, bcsr, bcsc, nnz_dev, BH, BW)
+        if self._BCSR:
+            return BCSRIndexes(self, mask, row_ptr, bcsr, nnz_dev, BH, BW)
+        return BCSCIndexes(self, mask, col_ptr, bcsc, nnz_dev, BH, BW)
+
+    # ---- values ------------------------------------------------------------------
+    def convert(self, dense: torch.Tensor, index: torch.Tensor, block_nnz: int, H: int, W: int,
+                idx_kind: int = _lib.IDX_BCSR_I32) -> torch.Tensor:
+        assert dense.shape[-2] == H and dense.shape[-1] == W, \
+            f'expected a (..., {H}, {W}) tensor, got {tuple(dense.shape)}'
+        lead = tuple(dense.shape[:-2])
+        batch = int(np.prod(lead)) if lead else 1
+        dense = dense.contiguous()
+        out = torch.empty((batch, block_nnz * self._block_size), dtype=dense.dtype, device=dense.device)
+        with torch.cuda.device(dense.device):
+            rc = _lib.load().spx_bcs_gather(
+                _lib.dev_ptr(dense), _lib.dev_ptr(out), _lib.dev_ptr(index), idx_kind, block_nnz, None,
+                batch, H, W, self._block_H, self._block_W, dense.element_size(),
+                block_nnz * self._block_size, _lib.current_stream(dense.device))
+        _lib.check(rc, 'spx_bcs_gather')
+        return out.reshape(lead + (-1,))
+
+    def inverse(self, sparse_val: torch.Tensor, index: torch.Tensor, block_nnz: int, H: int, W: int,
+                idx_kind: int = _lib.IDX_BCSR_I32) -> torch.Tensor:
+        assert sparse_val.shape[-1] == block_nnz * self._block_size, \
+            f'expected (..., {block_nnz * self._block_size}) values, got {tuple(sparse_val.shape)}'
+        lead = tuple(sparse_val.shape[:-1])
+        batch = int(np.prod(lead)) if lead else 1
+        sparse_val = sparse_val.contiguous()
+        dense = torch.zeros((batch, H, W), dtype=sparse_val.dtype, device=sparse_val.device)
+        with torch.cuda.device(sparse_val.device):
+            rc = _lib.load().spx_bcs_scatter(
+                _lib.dev_ptr(sparse_val), _lib.dev_ptr(dense), _lib.dev_ptr(index), idx_kind, block_nnz, None,
+                batch, H, W, self._block_H, self._block_W, sparse_val.element_size(),
+                block_nnz * self._block_size, _lib.current_stream(sparse_val.device))
+        _lib.check(rc, 'spx_bcs_scatter')
+        return dense.reshape(lead + (H, W))
+
+    def block_sum(self, sparse_val: torch.Tensor, index: torch.Tensor, idx_kind: int, block_nnz: int,
+                  H: int, W: int, axis: int) -> torch.Tensor:
+        """axis 0: [..., H] sums over W; axis 1: [..., W] sums over H (fp32 accumulate)."""
+        lead = tuple(sparse_val.shape[:-1])
+        batch = int(np.prod(lead)) if lead else 1
+        vals = sparse_val.contiguous().to(torch.float32)
+        n_out = H if axis == 0 else W
+        result = torch.zeros((batch, n_out), dtype=torch.float32, device=vals.device)
+        with torch.cuda.device(vals.device):
+            rc = _lib.load().spx_bcs_sum(
+                _lib.dev_ptr(vals), _lib.dev_ptr(result), _lib.dev_ptr(index), idx_kind, block_nnz,
+                batch, H, W, self._block_H, self._block_W, _lib.F32, axis,
+                block_nnz * self._block_size, _lib.current_stream(vals.device))
+        _lib.check(rc, 'spx_bcs_sum')
+        return result.to(sparse_val.dtype).reshape(lead + (n_out,))
+
+
+_bcs_function_cache: Dict[Tuple[int, int, bool, bool], BCSFunctionContext] = {}
+
+
+def get_bcs_function(block_H: int, block_W: int, BCSR: bool, BCSC: bool) -> BCSFunctionContext:
+    """Cached BCSFunctionContext per (block_H, block_W, BCSR, BCSC)."""
+    key = (block_H, block_W, bool(BCSR), bool(BCSC))
+    ctx = _bcs_function_cache.get(key)
+    if ctx is None:
+        ctx = _bcs_function_cache[key] = BCSFunctionContext(*key)
+    return ctx

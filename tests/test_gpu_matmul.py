@@ -1,0 +1,162 @@
+"""GPU parity of the block-sparse matmul kernels against the numpy oracle.
+Cases follow the reference's test/unit/test_sparse_matmul.py:98-174 (batch 4,
+M=128, K=256, N=192, 8x8-granular mask at 90%) over every mode, transpose,
+bias and storage variant, both implementation slots and three dtypes."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import bcs, ops
+from sparta_amd.specializer.kernels import SparTASparseMatMulKernel, OpenAISparseMatMulKernel
+from helpers import randn, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def run_case(gpu, mode, tA, tB, biased, compressed, dtype, blocks, impl='sparta',
+             batch=4, M=128, K=256, N=192, gran=(8, 8), sparsity=0.9, seed=2022):
+    BM, BK, BN = blocks
+    A_shape = (K, M) if tA else (M, K)
+    B_shape = (N, K) if tB else (K, N)
+    a_np, a_t = randn((batch,) + A_shape, seed, dtype)
+    b_np, b_t = randn((batch,) + B_shape, seed + 1, dtype)
+    bias_np, bias_t = randn((batch, N), seed + 2, dtype)
+    mask_shape = {'sdd': A_shape, 'dsd': B_shape, 'dds': (M, N)}[mode]
+    mask_np = ops.block_mask(mask_shape, gran, sparsity, seed=seed + 3)
+    mask = torch.from_numpy(mask_np).to(gpu)
+
+    cls = SparTASparseMatMulKernel if impl == 'sparta' else OpenAISparseMatMulKernel
+    kernel = cls(mode=mode, biased=biased, transpose_A=tA, transpose_B=tB, compressed=compressed)
+    port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
+    kernel.ports[port].set_mask(mask)
+    kernel.set_shape(batch, M, K, N)
+    kernel.compile({'BLOCK_SIZE_M_VALUE': BM, 'BLOCK_SIZE_K_VALUE': BK, 'BLOCK_SIZE_N_VALUE': BN})
+    indexes = kernel.ports[port].indexes
+    tile = {'sdd': (BK, BM) if tA else (BM, BK), 'dsd': (BN, BK) if tB else (BK, BN), 'dds': (BM, BN)}[mode]
+    assert (indexes.block_H, indexes.block_W) == tile
+
+    want = ops.matmul_reference(a_np, b_np, bias_np if biased else None, mode=mode, transpose_A=tA,
+                                transpose_B=tB, mask=mask_np, block=tile, dtype=np.float64)
+    A = a_t.to(gpu)
+    B = b_t.to(gpu)
+    # masked operands go in masked (the kernel reads every element of a live block)
+    if mode == 'sdd':
+        A = A * mask.to(dtype)
+        if compressed:
+            A = indexes.convert(A)
+    elif mode == 'dsd':
+        B = B * mask.to(dtype)
+        if compressed:
+            B = indexes.convert(B)
+    args = [A, B] + ([bias_t.to(gpu)] if biased else [])
+    C = kernel(*args)
+    if mode == 'dds' and compressed:
+        fmt_idx = indexes.BCSR_idx.cpu().numpy()
+        want = bcs.convert(want, fmt_idx, 'bcsr', BM, BN)
+    assert C.dtype == dtype and tuple(C.shape) == want.shape
+    assert_close(C, want, dtype, f'{mode} tA={tA} tB={tB} bias={biased} comp={compressed} {dtype}')
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('tA', [False, True])
+@pytest.mark.parametrize('tB', [False, True])
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('biased', [False, True])
+def test_matmul_fp32_all_variants(mode, tA, tB, compressed, biased, gpu):
+    run_case(gpu, mode, tA, tB, biased, compressed, torch.float32, (32, 32, 32))
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('tA', [False, True])
+@pytest.mark.parametrize('tB', [False, True])
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_matmul_half_all_variants(mode, tA, tB, compressed, dtype, gpu):
+    run_case(gpu, mode, tA, tB, True, compressed, dtype, (32, 32, 32))
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('tA,tB', [(False, True), (True, False)])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+def test_matmul_openai_slot(mode, tA, tB, dtype, gpu):
+    run_case(gpu, mode, tA, tB, True, True, dtype, (32, 64, 32), impl='openai')
+
+
+BLOCKS = [b for b in itertools.product([16, 32, 64], repeat=3)]
+
+
+@pytest.mark.parametrize('blocks', BLOCKS)
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+def test_matmul_block_shapes(blocks, mode, gpu):
+    # alternate dtype / transposes over the 27 block shapes to keep the suite short
+    k = BLOCKS.index(blocks)
+    dtype = [torch.float32, torch.float16, torch.bfloat16][k % 3]
+    run_case(gpu, mode, bool(k & 1), bool(k & 2), bool(k & 4), bool(k & 8) or True, dtype, blocks,
+             batch=2, M=192, K=128, N=256, gran=(16, 16), sparsity=0.8, seed=k)
+
+
+def test_matmul_all_ones_mask_is_plain_gemm(gpu):
+    a_np, a = randn((1, 256, 128), 1, torch.float32)
+    b_np, b = randn((1, 64, 128), 2, torch.float32)
+    mask = torch.ones((64, 128), dtype=torch.uint8, device=gpu)
+    kernel = SparTASparseMatMulKernel(mode='dsd', biased=False, transpose_A=False, transpose_B=True, compressed=False)
+    kernel.ports['B'].set_mask(mask)
+    kernel.set_shape(1, 256, 128, 64)
+    kernel.compile({'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32})
+    C = kernel(a.to(gpu), b.to(gpu))
+    assert_close(C, a_np @ b_np.transpose(0, 2, 1), torch.float32)
+
+
+def test_matmul_empty_mask_gives_zero_or_bias(gpu):
+    _, a = randn((1, 128, 64), 1, torch.float16)
+    _, b = randn((1, 64, 64), 2, torch.float16)
+    bias_np, bias = randn((1, 64), 3, torch.float16)
+    mask = torch.zeros((64, 64), dtype=torch.uint8, device=gpu)
+    kernel = SparTASparseMatMulKernel(mode='dsd', biased=True, transpose_A=False, transpose_B=True, compressed=True)
+    kernel.ports['B'].set_mask(mask)
+    kernel.set_shape(1, 128, 64, 64)
+    kernel.compile({'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32})
+    w = kernel.ports['B'].indexes.convert(b.to(gpu))
+    assert w.shape == (1, 0)
+    C = kernel(a.to(gpu), w, bias.to(gpu))
+    assert_close(C, np.broadcast_to(bias_np[:, None, :], (1, 128, 64)), torch.float16)
+
+
+def test_matmul_ragged_m(gpu):
+    """M that is not a multiple of the workgroup tile (dense dimension of 'dsd')."""
+    for M in (16, 48, 200):
+        run_case(gpu, 'dsd', False, True, True, True, torch.float16, (32, 32, 32), batch=1, M=M, K=128, N=64)
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+def test_matmul_headline_shape_fp16(mode, gpu):
+    """4096^3 fp16, 32x32 blocks at 95%: compared with a dense fp32 product of the
+    masked operands computed on the GPU by torch (the CPU oracle takes minutes at
+    this size; the small-shape tests above tie the kernels to the oracle)."""
+    M = K = N = 4096
+    g = torch.Generator().manual_seed(2022)
+    A = torch.randn((1, M, K), generator=g).half().to(gpu)
+    B = torch.randn((1, N, K), generator=g).half().to(gpu)
+    mask_np = ops.block_mask((4096, 4096), (32, 32), 0.95, seed=2022)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    kernel = SparTASparseMatMulKernel(mode=mode, biased=False, transpose_A=False, transpose_B=True, compressed=True)
+    port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
+    kernel.ports[port].set_mask(mask)
+    kernel.set_shape(1, M, K, N)
+    kernel.compile({'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32})
+    idx = kernel.ports[port].indexes
+    Af, Bf = A.float(), B.float()
+    if mode == 'sdd':
+        Af = Af * mask
+        C = kernel(idx.convert(A * mask.half()), B)
+    elif mode == 'dsd':
+        Bf = Bf * mask
+        C = kernel(A, idx.convert(B * mask.half()))
+    else:
+        C = idx.inverse(kernel(A, B))
+    want = torch.matmul(Af, Bf.transpose(1, 2))
+    if mode == 'dds':
+        want = want * mask
+    torch.testing.assert_close(C.float(), want, rtol=1e-2, atol=1e-2)

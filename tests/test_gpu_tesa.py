@@ -1,0 +1,118 @@
+"""GPU parity of the index builder and the converters against the numpy oracle
+(bit-exact).  Shapes follow the reference's test/unit/test_tesa.py (1024x768
+element-granular mask at 99.9% sparsity, every block shape in {4..128}^2) plus
+the benchmark configurations."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bcs, ops
+from sparta_amd.tesa import get_bcs_function
+
+pytestmark = pytest.mark.gpu
+
+EDGES = [4, 8, 16, 32, 64, 128]
+
+
+def _check_indexes(mask_np, BH, BW, gpu):
+    mask = torch.from_numpy(mask_np).to(gpu)
+    H, W = mask_np.shape
+    row_ptr, bcsr, col_ptr, bcsc64, nnz = bcs.build_bcsrc(mask_np, BH, BW)
+    _, bcsc32, _ = bcs.build_bcsc(mask_np, BH, BW)
+
+    r = get_bcs_function(BH, BW, True, False).build_indexes(mask)
+    assert r.block_nnz == nnz
+    assert np.array_equal(r.row_ptr.cpu().numpy(), row_ptr)
+    assert np.array_equal(r.BCSR_idx.cpu().numpy(), bcsr)
+    assert r.row_ptr.dtype == torch.int32 and r.BCSR_idx.dtype == torch.int32
+
+    c = get_bcs_function(BH, BW, False, True).build_indexes(mask)
+    assert c.block_nnz == nnz
+    assert np.array_equal(c.col_ptr.cpu().numpy(), col_ptr)
+    assert np.array_equal(c.BCSC_idx.cpu().numpy(), bcsc32)
+    assert c.BCSC_idx.dtype == torch.int32
+
+    rc = get_bcs_function(BH, BW, True, True).build_indexes(mask)
+    assert rc.block_nnz == nnz
+    assert np.array_equal(rc.row_ptr.cpu().numpy(), row_ptr)
+    assert np.array_equal(rc.col_ptr.cpu().numpy(), col_ptr)
+    assert np.array_equal(rc.BCSR_idx.cpu().numpy(), bcsr)
+    assert np.array_equal(rc.BCSC_idx.cpu().numpy(), bcsc64)
+    assert rc.BCSC_idx.dtype == torch.int64
+    live = bcs.reduce_block_mask(mask_np, BH, BW)
+    for idx in (r, c, rc):
+        assert np.array_equal(idx.get_block_mask().cpu().numpy().astype(bool), live)
+    return r, c, rc
+
+
+@pytest.mark.parametrize('BH', EDGES)
+@pytest.mark.parametrize('BW', EDGES)
+def test_index_reference_shapes(BH, BW, gpu):
+    mask_np = ops.block_mask((1024, 768), (1, 1), 0.999, seed=2023)
+    r, c, rc = _check_indexes(mask_np, BH, BW, gpu)
+    # convert / inverse / sum against the oracle, fp32, batch 2
+    dense_np = (np.random.default_rng(1).random((2, 1024, 768), dtype=np.float32) * mask_np)
+    dense = torch.from_numpy(dense_np).to(gpu)
+    for idx, fmt, arr in ((r, 'bcsr', r.BCSR_idx), (c, 'bcsc', c.BCSC_idx), (rc, 'bcsr', rc.BCSR_idx)):
+        want = bcs.convert(dense_np, arr.cpu().numpy(), fmt, BH, BW)
+        got = idx.convert(dense)
+        assert np.array_equal(got.cpu().numpy(), want)
+        assert np.array_equal(idx.inverse(got).cpu().numpy(), dense_np)
+        np.testing.assert_allclose(idx.sum(got, axis=-1).cpu().numpy(), dense_np.sum(-1), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(idx.sum(got, axis=-2).cpu().numpy(), dense_np.sum(-2), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize('shape,block,gran,sparsity', [
+    ((4096, 4096), (32, 32), (32, 32), 0.95),    # 4096^3 headline mask
+    ((1024, 1024), (32, 32), (8, 8), 0.90),      # README case, 8x8 granular
+    ((1024, 1024), (16, 16), (8, 8), 0.90),
+    ((4096, 4096), (64, 64), (64, 64), 0.90),    # attention layout grid
+    ((3072, 768), (32, 64), (32, 64), 0.90),     # FFN weights
+    ((768, 3072), (32, 64), (32, 64), 0.90),
+    ((64, 96), (4, 4), (1, 1), 0.5),
+    ((256, 8), (4, 8), (1, 1), 0.9),             # single block column
+    ((8, 20), (4, 4), (1, 1), 0.3),              # row pitch not a multiple of 16
+])
+def test_index_bench_shapes(shape, block, gran, sparsity, gpu):
+    _check_indexes(ops.block_mask(shape, gran, sparsity, seed=2022), block[0], block[1], gpu)
+
+
+@pytest.mark.parametrize('fill', [0, 1])
+def test_index_all_or_nothing(fill, gpu):
+    mask_np = np.full((256, 512), fill, dtype=np.uint8)
+    r, c, rc = _check_indexes(mask_np, 16, 32, gpu)
+    assert r.block_nnz == (16 * 16 if fill else 0)
+    x = torch.rand((1, 256, 512), device=gpu)
+    assert r.convert(x).shape == (1, r.block_nnz * 16 * 32)
+
+
+def test_index_single_element_makes_block_live(gpu):
+    mask_np = np.zeros((128, 128), dtype=np.uint8)
+    mask_np[77, 3] = 1
+    mask_np[127, 127] = 255
+    r, _, _ = _check_indexes(mask_np, 32, 32, gpu)
+    assert r.BCSR_idx.cpu().tolist() == [(2 << 16) | 0, (3 << 16) | 3]
+
+
+def test_index_is_deterministic(gpu):
+    mask = torch.from_numpy(ops.block_mask((2048, 2048), (1, 1), 0.99, seed=5)).to(gpu)
+    fn = get_bcs_function(32, 32, True, True)
+    first = fn.build_indexes(mask)
+    a, b = first.BCSR_idx.clone(), first.BCSC_idx.clone()
+    for _ in range(5):
+        again = fn.build_indexes(mask)
+        assert torch.equal(again.BCSR_idx, a) and torch.equal(again.BCSC_idx, b)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.uint8, torch.float64])
+def test_convert_other_element_sizes(dtype, gpu):
+    mask_np = ops.block_mask((512, 256), (16, 32), 0.7, seed=3)
+    idx = get_bcs_function(16, 32, True, False).build_indexes(torch.from_numpy(mask_np).to(gpu))
+    src = (torch.rand((3, 512, 256)) * 100).to(dtype) * torch.from_numpy(mask_np).to(dtype)
+    got = idx.convert(src.to(gpu))
+    want = bcs.convert(src.view(torch.uint8 if dtype == torch.uint8 else torch.int16 if src.element_size() == 2
+                                else torch.int64).numpy(), idx.BCSR_idx.cpu().numpy(), 'bcsr', 16, 32)
+    raw = got.cpu().view(torch.uint8 if dtype == torch.uint8 else torch.int16 if src.element_size() == 2
+                         else torch.int64).numpy()
+    assert np.array_equal(raw, want)
+    assert torch.equal(idx.inverse(got).cpu(), src)
