@@ -60,8 +60,8 @@ static int launch_convert(const void* src, void* dst, const void* idx, int idx_k
                           int nnz_bound, const int32_t* nnz_dev, int batch, int H, int W,
                           int BH, int BW, int elem_bytes, int64_t sparse_batch_stride,
                           hipStream_t st) {
-    SPX_REQUIRE(src && dst, SPX_E_NULL, "dense / sparse buffer is NULL");
-    SPX_REQUIRE(idx || nnz_bound == 0, SPX_E_NULL, "index array is NULL");
+    SPX_REQUIRE((src && dst && idx) || nnz_bound == 0 || batch == 0, SPX_E_NULL,
+                "dense, sparse and index buffers are required");
     SPX_REQUIRE(idx_kind >= 0 && idx_kind <= 2, SPX_E_CONFIG, "unknown idx_kind %d", idx_kind);
     SPX_REQUIRE(valid_block_edge(BH) && valid_block_edge(BW), SPX_E_CONFIG,
                 "block size (%d,%d) must be a power of two in [4,256]", BH, BW);

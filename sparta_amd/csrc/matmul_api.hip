@@ -78,7 +78,13 @@ extern "C" int spx_matmul(int mode, int dtype, int transA, int transB, int compr
     using namespace spx;
     SPX_REQUIRE(mode == SPX_SDD || mode == SPX_DSD || mode == SPX_DDS, SPX_E_CONFIG, "unknown mode %d", mode);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
-    SPX_REQUIRE(A && B && C, SPX_E_NULL, "A, B and C are required");
+    {
+        // an empty compressed operand / result (no live block) may be NULL
+        const bool empty_ok = compressed && nnz_bound == 0;
+        SPX_REQUIRE(A || (mode == SPX_SDD && empty_ok), SPX_E_NULL, "A is required");
+        SPX_REQUIRE(B || (mode == SPX_DSD && empty_ok), SPX_E_NULL, "B is required");
+        SPX_REQUIRE(C || (mode == SPX_DDS && empty_ok), SPX_E_NULL, "C is required");
+    }
     SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
     SPX_REQUIRE(M > 0 && K > 0 && N > 0, SPX_E_SHAPE, "M, K, N must be positive");
     SPX_REQUIRE((BM == 16 || BM == 32 || BM == 64) && (BK == 16 || BK == 32 || BK == 64) &&
