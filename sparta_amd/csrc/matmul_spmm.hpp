@@ -203,10 +203,35 @@ static int launch_spmm_inst(const SpmmParams& p, int batch, hipStream_t st) {
     return 0;
 }
 
-// tile_cfg: 0 = pick by size, 1 = 64-row tiles, 2 = 128-row tiles.
+template <typename T>
+int launch_spmm_direct(const SpmmParams& p, int BN, int batch, int wm, hipStream_t st);
+template <typename T>
+int launch_spmm_panel(const SpmmParams& p, int BN, int batch, int nst, hipStream_t st);
+
+// tile_cfg: 0 = pick by layout and size;
+//   1 / 2  LDS-staged kernel, 64 / 128-row workgroup tiles (any layout);
+//   3 / 4  register-direct kernel, 64 / 256-row workgroup tiles (k-contiguous operands);
+//   5 / 6  panel kernel, 256-row workgroup tiles, 2 / 3 load stages (k-contiguous
+//          operands, block depth a multiple of 64 bytes).
 template <typename T>
 int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipStream_t st) {
-    int wm = tile_cfg == 1 ? 1 : tile_cfg == 2 ? 2 : (p.Mc >= 1024 ? 2 : 1);
+    const bool kcontig = p.d_kcontig && p.s_kcontig;
+    const bool panel_ok = kcontig && (p.BK * (int)sizeof(T)) % 64 == 0;
+    if (tile_cfg < 0 || tile_cfg > 6) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    if (tile_cfg == 0) {
+        if (panel_ok && p.Mc >= 512) tile_cfg = 5;
+        else if (kcontig) tile_cfg = p.Mc >= 1024 ? 4 : 3;
+        else tile_cfg = p.Mc >= 1024 ? 2 : 1;
+    }
+    if (tile_cfg >= 5) {
+        if (!panel_ok) return fail(SPX_E_CONFIG, "tile config %d needs k-contiguous operands and 64-byte block rows", tile_cfg);
+        return launch_spmm_panel<T>(p, BN, batch, tile_cfg == 6 ? 3 : 2, st);
+    }
+    if (tile_cfg >= 3) {
+        if (!kcontig) return fail(SPX_E_CONFIG, "tile config %d needs k-contiguous operands", tile_cfg);
+        return launch_spmm_direct<T>(p, BN, batch, tile_cfg == 4 ? 4 : 1, st);
+    }
+    const int wm = tile_cfg == 2 ? 2 : 1;
     if (wm == 2) {
         switch (BN) {
             case 16: return launch_spmm_inst<T, 16, 2>(p, batch, st);

@@ -1,0 +1,8 @@
+// bf16 instantiations of the register-direct sparse-operand matmul kernel.
+#include "matmul_spmm_direct.hpp"
+namespace spx {
+template <>
+int launch_spmm_direct<bf16_t>(const SpmmParams& p, int BN, int batch, int wm, hipStream_t st) {
+    return launch_spmm_direct_impl<bf16_t>(p, BN, batch, wm, st);
+}
+}  // namespace spx

@@ -1,0 +1,306 @@
+// Sparse-operand matmul, panel variant for k-contiguous operands: the main kernel
+// of SparseLinear(weight_mask) ('dsd', weight stored [N,K]) and of its 'sdd'
+// mirror.  Canonical problem as in matmul_spmm.hpp: out[m,n] = sum_k D[m,k] S[k,n].
+//
+// Each wavefront owns a 64 x BN output tile and is fully independent (no
+// workgroup barrier anywhere).  One pipeline step covers 64 bytes of k (32 x
+// 16-bit or 16 x fp32) of one live block:
+//   * global -> registers with a coalesced mapping: 4 consecutive lanes read the
+//     64 contiguous bytes of one row, so a wave load touches 16 cache lines
+//     instead of the 64 an MFMA-layout load would touch;
+//   * registers -> private LDS (6 KB per wave) with an XOR swizzle, read back as
+//     conflict-free 16-byte MFMA fragments (lane = row % 16, k group = lane / 16);
+//   * NST register stages keep NST steps of loads in flight per wave.
+// Workgroups are numbered so that all tiles of one 256-row panel of D run on
+// one XCD and share its L2 (workgroup L is dispatched to XCD L % 8).
+#pragma once
+#include <type_traits>
+#include "matmul_spmm.hpp"
+
+namespace spx {
+
+constexpr int kPanelXcd = 8;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct PanelMma {
+    // one step = 64 bytes of k per row
+    static constexpr bool WIDE = sizeof(T) == 2;
+    typedef typename std::conditional<WIDE, Mma32<typename std::conditional<WIDE, T, _Float16>::type>,
+                                      Mma16<typename std::conditional<WIDE, float, T>::type>>::type M;
+    static constexpr int KC = 64 / (int)sizeof(T);  // k per step
+};
+
+template <typename T, int BN, int BK, int NST, bool SWAP>
+__global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mtiles) {
+    typedef typename PanelMma<T>::M MMA;
+    typedef typename MMA::frag Frag;
+    constexpr int KC = PanelMma<T>::KC;
+    constexpr int CH = BK / KC;          // steps per block
+    constexpr int NT = BN / 16;
+    constexpr int WL = BN / 16;          // 16-byte loads per lane for the S rows
+    constexpr int ROWS = 64 + BN;        // LDS rows (64 bytes each) per wave
+    constexpr int E16 = 16 / (int)sizeof(T);
+    static_assert(BK % KC == 0, "block depth must be a multiple of the step");
+
+    __shared__ __align__(16) char lds_all[4 * ROWS * 64];
+
+    const int nb = p.Nc / BN;
+    const int L = blockIdx.x;
+    const int xcd = L % kPanelXcd;
+    const int seq = L / kPanelXcd;
+    const int mt = (seq / nb) * kPanelXcd + xcd;
+    const int j = seq % nb;
+    if (mt >= n_mtiles) return;
+    const int64_t b = blockIdx.y;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15;
+    const int g4 = lane >> 4;
+    const int m0 = mt * 256 + wave * 64;
+    if (m0 >= p.Mc) return;  // waves are independent: leaving early is safe
+    char* lds = lds_all + wave * (ROWS * 64);
+
+    const T* D = reinterpret_cast<const T*>(p.D) + b * p.d_batch;
+    const T* S = reinterpret_cast<const T*>(p.S) + b * p.s_batch;
+
+    // coalesced load mapping: lane -> (row within a 16-row group, 16-byte chunk)
+    const int lrow = lane >> 2;
+    const int lchk = lane & 3;
+    const T* dptr[4];
+    int wofs[4];  // LDS byte offsets of this lane's chunk for the 4 row groups of D
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int row = q * 16 + lrow;
+        int m = m0 + row;
+        if (m >= p.Mc) m = p.Mc - 1;  // rows past the end re-read the last row; never stored
+        dptr[q] = D + (int64_t)m * p.d_ld + lchk * E16;
+        wofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
+    }
+    int sofs[WL];
+#pragma unroll
+    for (int q = 0; q < WL; ++q) {
+        const int row = 64 + q * 16 + lrow;
+        sofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
+    }
+    // fragment read offsets (row = tile*16 + r16, chunk g4)
+    int aofs[4], bofs[NT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = i * 16 + r16;
+        aofs[i] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int row = 64 + t * 16 + r16;
+        bofs[t] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
+    }
+
+    f32x4 acc[4][NT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int e_begin = p.ptr[j];
+    const int n_blk = p.ptr[j + 1] - e_begin;
+    const int n_it = n_blk * CH;
+    const int64_t sld = p.compressed ? BK : p.s_ld;
+
+    // The first 64 index entries of the block-column live in one VGPR pair (lane l
+    // holds entry l) and are broadcast with readlane, which keeps the index fetch
+    // off the critical path of every step; longer columns fall back to scalar loads.
+    int kb_vec = 0, slot_vec = 0;
+    if (lane < n_blk) {
+        if (p.idx_kind == SPX_IDX_BCSC_I64) {
+            const long long v = reinterpret_cast<const long long*>(p.idx)[e_begin + lane];
+            kb_vec = (int)(v & 0xffff);
+            slot_vec = (int)(v >> 32);
+        } else {
+            kb_vec = reinterpret_cast<const int32_t*>(p.idx)[e_begin + lane] & 0xffff;
+            slot_vec = e_begin + lane;
+        }
+    }
+
+    // Stage registers are separate named arrays (not an array of stages) so that
+    // they stay in VGPRs.
+    u32x4 d0[4], s0[WL], d1[4], s1[WL], d2[4], s2[WL];
+
+#define SPX_PANEL_ISSUE(IT, DREG, SREG)                                                            \
+    do {                                                                                           \
+        const int er_ = (IT) / CH;                                                                 \
+        const int ch_ = (IT) % CH;                                                                 \
+        int kb_;                                                                                   \
+        int64_t slot_;                                                                             \
+        if (er_ < 64) {                                                                            \
+            kb_ = __builtin_amdgcn_readlane(kb_vec, er_);                                          \
+            slot_ = __builtin_amdgcn_readlane(slot_vec, er_);                                      \
+        } else if (p.idx_kind == SPX_IDX_BCSC_I64) {                                               \
+            const long long v_ = reinterpret_cast<const long long*>(p.idx)[e_begin + er_];         \
+            kb_ = (int)(v_ & 0xffff);                                                              \
+            slot_ = v_ >> 32;                                                                      \
+        } else {                                                                                   \
+            kb_ = reinterpret_cast<const int32_t*>(p.idx)[e_begin + er_] & 0xffff;                 \
+            slot_ = e_begin + er_;                                                                 \
+        }                                                                                          \
+        const int koff_ = kb_ * BK + ch_ * KC;                                                     \
+        const T* sblk_ = p.compressed ? S + slot_ * (int64_t)(BK * BN) + ch_ * KC                  \
+                                      : S + (int64_t)j * BN * p.s_ld + koff_;                      \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
+            DREG[q] = *reinterpret_cast<const u32x4*>(dptr[q] + koff_);                            \
+        _Pragma("unroll") for (int q = 0; q < WL; ++q)                                             \
+            SREG[q] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)(q * 16 + lrow) * sld + lchk * E16); \
+    } while (0)
+
+// All global loads and LDS writes of the pipeline are issued unconditionally (steps
+// past the end re-load the last step and are not accumulated): with no branch
+// around a memory instruction the number of loads in flight is the same on every
+// path, so each wait only covers the oldest stage and NST-1 stages stay in flight.
+#define SPX_PANEL_STEP(IT, DREG, SREG)                                                             \
+    do {                                                                                           \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
+            *reinterpret_cast<u32x4*>(lds + wofs[q]) = DREG[q];                                    \
+        _Pragma("unroll") for (int q = 0; q < WL; ++q)                                             \
+            *reinterpret_cast<u32x4*>(lds + sofs[q]) = SREG[q];                                    \
+        {                                                                                          \
+            const int nx_ = (IT) + NST < n_it ? (IT) + NST : n_it - 1;                             \
+            SPX_PANEL_ISSUE(nx_, DREG, SREG);                                                      \
+        }                                                                                          \
+        if ((IT) < n_it) {                                                                         \
+            Frag af_[4], bf_[NT];                                                                  \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i)                                          \
+                af_[i] = *reinterpret_cast<const Frag*>(lds + aofs[i]);                            \
+            _Pragma("unroll") for (int t = 0; t < NT; ++t)                                         \
+                bf_[t] = *reinterpret_cast<const Frag*>(lds + bofs[t]);                            \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i)                                          \
+                _Pragma("unroll") for (int t = 0; t < NT; ++t)                                     \
+                    acc[i][t] = SWAP ? MMA::mma(bf_[t], af_[i], acc[i][t])                         \
+                                     : MMA::mma(af_[i], bf_[t], acc[i][t]);                        \
+        }                                                                                          \
+    } while (0)
+
+    if (n_it > 0) {
+        SPX_PANEL_ISSUE(0, d0, s0);
+        SPX_PANEL_ISSUE((1 < n_it ? 1 : n_it - 1), d1, s1);
+        if (NST > 2) SPX_PANEL_ISSUE((2 < n_it ? 2 : n_it - 1), d2, s2);
+        for (int it = 0; it < n_it; it += NST) {
+            SPX_PANEL_STEP(it, d0, s0);
+            SPX_PANEL_STEP(it + 1, d1, s1);
+            if (NST > 2) SPX_PANEL_STEP(it + 2, d2, s2);
+        }
+    }
+#undef SPX_PANEL_ISSUE
+#undef SPX_PANEL_STEP
+
+    // ---- epilogue: registers -> private LDS -> 16-byte row-contiguous stores -----------
+    // (LDS instructions of one wave execute in order, so the region can be reused
+    // without a barrier once the last fragment reads have been issued.)
+    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
+    T* out = reinterpret_cast<T*>(p.out) + b * p.o_batch;
+    T* eT = reinterpret_cast<T*>(lds);
+    if constexpr (SWAP) {
+        // out[m][n], n contiguous.  One 16-row slab per pass: LDS [16][BN + pad].
+        constexpr int LDE = BN + E16;
+        constexpr int CPR = BN / E16;  // 16-byte chunks per row
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                T vals[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v = acc[i][t][q];
+                    const int n = j * BN + t * 16 + g4 * 4 + q;
+                    if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m0 + i * 16 + r16 < p.Mc ? m0 + i * 16 + r16 : 0) : n]);
+                    vals[q] = Elem<T>::from_float(v);
+                }
+                T* dst = eT + r16 * LDE + t * 16 + g4 * 4;
+                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+            }
+#pragma unroll
+            for (int c0 = 0; c0 < 16 * CPR; c0 += 64) {
+                const int c = c0 + lane;
+                const int row = c / CPR;
+                const int chunk = c % CPR;
+                const int m = m0 + i * 16 + row;
+                if (c < 16 * CPR && m < p.Mc)
+                    *reinterpret_cast<u32x4*>(out + (int64_t)m * p.o_ld + (int64_t)j * BN + chunk * E16) =
+                        *reinterpret_cast<const u32x4*>(eT + row * LDE + chunk * E16);
+            }
+        }
+    } else {
+        // out[n][m], m contiguous.  One 16-column slab per pass: LDS [16 n][64 m + pad].
+        constexpr int LDE = 64 + E16;
+        constexpr int CPR = 64 / E16;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                T vals[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v = acc[i][t][q];
+                    const int m = m0 + i * 16 + g4 * 4 + q;
+                    if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m < p.Mc ? m : 0) : j * BN + t * 16 + r16]);
+                    vals[q] = Elem<T>::from_float(v);
+                }
+                T* dst = eT + r16 * LDE + i * 16 + g4 * 4;
+                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+            }
+#pragma unroll
+            for (int c0 = 0; c0 < 16 * CPR; c0 += 64) {
+                const int c = c0 + lane;
+                const int nrow = c / CPR;
+                const int chunk = c % CPR;
+                const int m = m0 + chunk * E16;
+                if (m < p.Mc)
+                    *reinterpret_cast<u32x4*>(out + ((int64_t)j * BN + t * 16 + nrow) * p.o_ld + m) =
+                        *reinterpret_cast<const u32x4*>(eT + nrow * LDE + chunk * E16);
+            }
+        }
+    }
+}
+
+template <typename T, int BN, int BK, int NST, bool SWAP>
+static int launch_spmm_panel_inst(const SpmmParams& p, int batch, hipStream_t st) {
+    const int n_mtiles = (p.Mc + 255) / 256;
+    const int nb = p.Nc / BN;
+    const int64_t groups = (n_mtiles + kPanelXcd - 1) / kPanelXcd;
+    const int64_t nblocks = groups * kPanelXcd * nb;
+    if (nblocks > 0x7fffffffLL) return fail(SPX_E_SHAPE, "problem too large for one launch");
+    hipLaunchKernelGGL((spmm_panel_kernel<T, BN, BK, NST, SWAP>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st,
+                       p, n_mtiles);
+    SPX_LAUNCH_CHECK("spmm_panel_kernel");
+    return 0;
+}
+
+// Supported: 16-bit types with BK in {32,64}, fp32 with BK in {16,32,64}; BN in {16,32,64}.
+template <typename T>
+bool spmm_panel_supported(int BN, int BK) {
+    const int kc = 64 / (int)sizeof(T);
+    return BK % kc == 0 && (BN == 16 || BN == 32 || BN == 64);
+}
+
+template <typename T, int NST>
+int launch_spmm_panel_impl(const SpmmParams& p, int BN, int batch, hipStream_t st) {
+    const bool swap = p.out_ncontig != 0;
+#define SPX_PANEL_CASE(bn, bk)                                                                  \
+    if (BN == bn && p.BK == bk) {                                                               \
+        if constexpr (bk % (64 / (int)sizeof(T)) == 0) {                                        \
+            return swap ? launch_spmm_panel_inst<T, bn, bk, NST, true>(p, batch, st)            \
+                        : launch_spmm_panel_inst<T, bn, bk, NST, false>(p, batch, st);          \
+        }                                                                                       \
+    }
+    SPX_PANEL_CASE(16, 16) SPX_PANEL_CASE(16, 32) SPX_PANEL_CASE(16, 64)
+    SPX_PANEL_CASE(32, 16) SPX_PANEL_CASE(32, 32) SPX_PANEL_CASE(32, 64)
+    SPX_PANEL_CASE(64, 16) SPX_PANEL_CASE(64, 32) SPX_PANEL_CASE(64, 64)
+#undef SPX_PANEL_CASE
+    return fail(SPX_E_CONFIG, "block (%d,%d) not supported by the panel kernel", p.BK, BN);
+}
+
+template <typename T>
+int launch_spmm_panel(const SpmmParams& p, int BN, int batch, int nst, hipStream_t st);
+
+}  // namespace spx

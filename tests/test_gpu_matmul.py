@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 
 def run_case(gpu, mode, tA, tB, biased, compressed, dtype, blocks, impl='sparta',
-             batch=4, M=128, K=256, N=192, gran=(8, 8), sparsity=0.9, seed=2022):
+             batch=4, M=128, K=256, N=192, gran=(8, 8), sparsity=0.9, seed=2022, tile_cfg=0):
     BM, BK, BN = blocks
     A_shape = (K, M) if tA else (M, K)
     B_shape = (N, K) if tB else (K, N)
@@ -32,7 +32,8 @@ def run_case(gpu, mode, tA, tB, biased, compressed, dtype, blocks, impl='sparta'
     port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
     kernel.ports[port].set_mask(mask)
     kernel.set_shape(batch, M, K, N)
-    kernel.compile({'BLOCK_SIZE_M_VALUE': BM, 'BLOCK_SIZE_K_VALUE': BK, 'BLOCK_SIZE_N_VALUE': BN})
+    kernel.compile({'BLOCK_SIZE_M_VALUE': BM, 'BLOCK_SIZE_K_VALUE': BK, 'BLOCK_SIZE_N_VALUE': BN,
+                    'TILE_CFG': tile_cfg})
     indexes = kernel.ports[port].indexes
     tile = {'sdd': (BK, BM) if tA else (BM, BK), 'dsd': (BN, BK) if tB else (BK, BN), 'dds': (BM, BN)}[mode]
     assert (indexes.block_H, indexes.block_W) == tile
@@ -95,6 +96,20 @@ def test_matmul_block_shapes(blocks, mode, gpu):
     dtype = [torch.float32, torch.float16, torch.bfloat16][k % 3]
     run_case(gpu, mode, bool(k & 1), bool(k & 2), bool(k & 4), bool(k & 8) or True, dtype, blocks,
              batch=2, M=192, K=128, N=256, gran=(16, 16), sparsity=0.8, seed=k)
+
+
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize('mode', ['sdd', 'dsd'])
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 64, 32)),
+                                          (torch.float32, (16, 16, 64)), (torch.float16, (32, 64, 16)),
+                                          (torch.float32, (32, 32, 32))])
+def test_matmul_tile_configs(tile_cfg, mode, compressed, dtype, blocks, gpu):
+    """Every kernel family behind TILE_CFG gives the same masked-dense result
+    (k-contiguous layout, which all of them accept); M is ragged on purpose."""
+    run_case(gpu, mode, False, True, True, compressed, dtype, blocks, batch=2,
+             M=320 if mode == 'dsd' else 192, K=256, N=192 if mode == 'dsd' else 328, gran=(16, 16),
+             sparsity=0.7, seed=11, tile_cfg=tile_cfg)
 
 
 def test_matmul_all_ones_mask_is_plain_gemm(gpu):
