@@ -31,9 +31,9 @@ def matmul_reference(A, B, bias=None, *, mode, transpose_A, transpose_B, mask, b
         A = A * mask
     elif mode == 'dsd':
         B = B * mask
-    a = 'bkm' if transpose_A else 'bmk'
-    b = 'bnk' if transpose_B else 'bkn'
-    C = np.einsum(f'{a},{b}->bmn', A, B, optimize=True)
+    lhs = np.swapaxes(A, -1, -2) if transpose_A else A   # [Bt, M, K]
+    rhs = np.swapaxes(B, -1, -2) if transpose_B else B   # [Bt, K, N]
+    C = np.matmul(lhs, rhs)
     if bias is not None:
         C = C + bias.astype(dtype)[:, None, :]
     if mode == 'dds':

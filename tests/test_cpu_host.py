@@ -1,0 +1,249 @@
+"""CPU tier: the shared library loads and exports the whole C ABI, host-side
+argument validation answers before any launch, the Python operator / tuner layer
+behaves like the reference's (search-space keys, connections, trial counts), and
+the oracle reproduces the committed golden vectors.  Nothing here launches a
+kernel."""
+import ctypes
+import os
+import random
+import re
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import sparta_amd as sparta
+from sparta_amd import _lib
+from sparta_amd.nn import tune, SparseLinear, SparseBatchMatMul, SparseSoftmax, SparseAttention
+from oracle import bcs, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLD = np.load(os.path.join(ROOT, 'tests', 'golden', 'vectors.npz'))
+
+
+# ---------------------------------------------------------------- C ABI -----------
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, 'include', 'sparta_hip.h')).read()
+    header = re.sub(r'/\*.*?\*/', '', header, flags=re.S)
+    declared = set(re.findall(r'\b(spx_[a-z_0-9]+)\s*\(', header))
+    assert len(declared) >= 15
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f'{name} is declared in sparta_hip.h but not exported'
+    assert declared == set(_lib.EXPORTED_SYMBOLS)
+    assert lib.spx_version() == 100
+
+
+def test_host_validation_without_gpu():
+    lib = _lib.load()
+    assert lib.spx_bcs_index_workspace_bytes(4096, 4096, 32, 32) > 4096 * 4096 // 1024
+    assert lib.spx_bcs_index_workspace_bytes(100, 100, 32, 32) == 0
+    rc = lib.spx_bcs_index(None, 64, 64, 3, 32, None, None, None, None, 0, None, 0, None, 0, None)
+    assert rc == _lib.E_CONFIG and 'power of two' in _lib.last_error()
+    rc = lib.spx_bcs_index(None, 64, 60, 32, 32, None, None, None, None, 0, None, 0, None, 0, None)
+    assert rc == _lib.E_SHAPE
+    rc = lib.spx_bcs_index(None, 64, 64, 32, 32, None, None, None, None, 0, None, 0, None, 0, None)
+    assert rc == _lib.E_NULL
+    one = ctypes.c_void_p(256)  # never dereferenced: validation fails first
+    rc = lib.spx_matmul(7, 0, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
+    assert rc == _lib.E_CONFIG
+    rc = lib.spx_matmul(1, 9, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
+    assert rc == _lib.E_DTYPE
+    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 64, 64, 32, 48, 32, 0, None)
+    assert rc == _lib.E_CONFIG
+    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 80, 64, 32, 32, 32, 0, None)
+    assert rc == _lib.E_SHAPE and 'K=80' in _lib.last_error()
+    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 1, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
+    assert rc == _lib.E_CONFIG  # BCSC index handed to a BCSR-mode kernel
+    rc = lib.spx_softmax_forward(1, 0, one, one, one, one, one, 1.0, 1, 64, 64, 5, 32, 0, 0, None)
+    assert rc == _lib.E_CONFIG
+    with pytest.raises(AssertionError):
+        _lib.check(_lib.E_SHAPE, 'x')
+    with pytest.raises(ValueError):
+        _lib.check(_lib.E_NULL, 'x')
+    with pytest.raises(RuntimeError):
+        _lib.check(700, 'x')
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    with pytest.raises(RuntimeError, match='GPU only'):
+        _lib.dev_ptr(torch.zeros(4))
+
+
+# ------------------------------------------------------- golden vectors / oracle ----
+def test_oracle_reproduces_golden_index_vectors():
+    for i in range(4):
+        H, W, BH, BW, nnz = GOLD[f'idx{i}_meta'].tolist()
+        mask = GOLD[f'idx{i}_mask']
+        row_ptr, bcsr, col_ptr, bcsc64, n = bcs.build_bcsrc(mask, BH, BW)
+        assert n == nnz
+        assert np.array_equal(row_ptr, GOLD[f'idx{i}_row_ptr']) and np.array_equal(bcsr, GOLD[f'idx{i}_bcsr'])
+        assert np.array_equal(col_ptr, GOLD[f'idx{i}_col_ptr']) and np.array_equal(bcsc64, GOLD[f'idx{i}_bcsc64'])
+        assert np.array_equal(bcs.build_bcsc(mask, BH, BW)[1], GOLD[f'idx{i}_bcsc32'])
+
+
+def test_torch_reference_functions_match_the_oracle():
+    """sparta_amd.testing.* (used by the tuner's correctness check) against the
+    golden vectors written by the numpy oracle."""
+    x, g, mask = (torch.from_numpy(GOLD[k]) for k in ('sm_x', 'sm_g', 'sm_mask'))
+    y = sparta.testing.sparse_softmax_forward_reference(x.double(), mask, 8.0)
+    np.testing.assert_allclose(y.numpy(), GOLD['sm_y'], rtol=1e-7, atol=1e-9)
+    gx = sparta.testing.sparse_softmax_backward_reference(g.double(), y, mask, 8.0)
+    np.testing.assert_allclose(gx.numpy(), GOLD['sm_gx'], rtol=1e-7, atol=1e-9)
+    q, k, v, amask = (torch.from_numpy(GOLD[n]) for n in ('att_q', 'att_k', 'att_v', 'att_mask'))
+    out = sparta.testing.sparse_multi_head_attention_reference(q.double(), k.double(), v.double(), amask)
+    np.testing.assert_allclose(out.numpy(), GOLD['att_out'], rtol=1e-7, atol=1e-9)
+
+
+def test_block_mask_generator():
+    torch.manual_seed(0)
+    m = sparta.testing.block_mask((64, 128), block=(8, 16), sparsity=0.5, device='cpu')
+    assert m.shape == (64, 128) and m.dtype == torch.uint8
+    tiles = m.reshape(8, 8, 8, 16).swapaxes(1, 2)
+    assert bool((tiles.amin(dim=(2, 3)) == tiles.amax(dim=(2, 3))).all())
+    with pytest.raises(AssertionError):
+        sparta.testing.block_mask((10, 10), block=(4, 4), device='cpu')
+    with pytest.raises(ValueError):
+        sparta.testing.block_mask((8, 8), algo='magic', device='cpu')
+
+
+# ------------------------------------------------------------- operator layer --------
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('trans_A', [False, True])
+@pytest.mark.parametrize('trans_B', [False, True])
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('backward', [False, True])
+def test_sparse_matmul_search_space(mode, compressed, trans_A, trans_B, backward):
+    """Key structure of test/unit/test_search_space.py:31-56."""
+    mask = torch.zeros((64, 64))
+    port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
+    op = SparseBatchMatMul(**{f'{port}_mask': mask}, transpose_A=trans_A, transpose_B=trans_B,
+                           compressed=compressed)
+    space = op.get_search_space(backward=backward)
+    names = ['forward:C'] + (['backward:A', 'backward:B'] if backward else [])
+    assert set(space) == set(names)
+    params = {f'BLOCK_SIZE_{d}_VALUE' for d in 'MKN'}
+    for kernel_space in space.values():
+        assert set(kernel_space) == {'sparta', 'openai'}
+        assert set(kernel_space['sparta']) == params and set(kernel_space['openai']) == params
+        assert kernel_space['sparta']['BLOCK_SIZE_M_VALUE']._value == [16, 32, 64]
+        assert [kernel_space['openai'][f'BLOCK_SIZE_{d}_VALUE']._value for d in 'MKN'] == [[32], [64], [32]]
+    connections = op.get_connections(backward=backward)
+    assert len(connections) == (2 if compressed and backward else 0)
+
+
+def test_derived_backward_kernels_of_sparse_linear():
+    """SparseLinear(weight_mask) = dsd(tA=F,tB=T); its gradients are
+    dsd(tA=F,tB=F) reading a BCSC index and dds(tA=T,tB=F)
+    (sparta/specializer/funtional/batch_matmul.py:47-71)."""
+    lin = torch.nn.Linear(64, 96)
+    op = SparseLinear(lin, weight_mask=torch.ones((96, 64), dtype=torch.uint8))
+    ks = op._sparse_ctx._kernels
+    k = {n: p.possible_kernels['sparta'] for n, p in ks.items()}
+    assert (k['forward:C']._mode, k['forward:C']._transpose_A, k['forward:C']._transpose_B) == ('dsd', False, True)
+    assert (k['backward:A']._mode, k['backward:A']._transpose_A, k['backward:A']._transpose_B) == ('dsd', False, False)
+    assert (k['backward:B']._mode, k['backward:B']._transpose_A, k['backward:B']._transpose_B) == ('dds', True, False)
+    assert k['forward:C']._bcs_mode == 'BCSR' and k['backward:A']._bcs_mode == 'BCSC'
+    assert ks['forward:C'].port_map == {'B': 'B'} and ks['backward:A'].port_map == {'B': 'B'}
+    assert ks['backward:B'].port_map == {'B': 'C'}
+    conn = op.get_connections(backward=True)
+    assert conn[0] == {'forward:C': 'BLOCK_SIZE_N_VALUE', 'backward:A': 'BLOCK_SIZE_K_VALUE',
+                       'backward:B': 'BLOCK_SIZE_M_VALUE'}
+    assert conn[1] == {'forward:C': 'BLOCK_SIZE_K_VALUE', 'backward:A': 'BLOCK_SIZE_N_VALUE',
+                       'backward:B': 'BLOCK_SIZE_N_VALUE'}
+
+
+def _count_trials(module, sample_inputs, sample_grads=None):
+    calls = {'n': 0}
+
+    def debug_func(idx, params):
+        calls['n'] += 1
+        return random.random()
+
+    try:
+        tune(module, sample_inputs=sample_inputs, sample_grads=sample_grads, algo='grid',
+             max_trials=sys.maxsize, backward_weight=0 if sample_grads is None else 0.5,
+             verbose=False, debug_func=debug_func)
+    except AssertionError:
+        pass
+    return calls['n']
+
+
+@pytest.mark.parametrize('backward', [False, True])
+def test_tuner_trial_counts(backward):
+    """Trial counts of test/unit/test_tuners.py with a fake measurement."""
+    grads = lambda *shape: [torch.zeros(shape)] if backward else None
+    lin = SparseLinear(torch.nn.Linear(128, 128), weight_mask=torch.ones((128, 128), dtype=torch.uint8))
+    assert _count_trials(lin, [torch.zeros((128, 128))], grads(128, 128)) == (27 + 1) * (3 if backward else 1)
+    mm = SparseBatchMatMul(C_mask=torch.ones((128, 128), dtype=torch.uint8), transpose_A=False,
+                           transpose_B=True, compressed=True)
+    assert _count_trials(mm, [torch.zeros((4, 128, 128)), torch.zeros((4, 128, 128))],
+                         grads(4, 128, 128)) == (27 + 1) * (3 if backward else 1)
+    sm = SparseSoftmax(mask=torch.ones((128, 128), dtype=torch.uint8), temperature=128, compressed=True)
+    assert _count_trials(sm, [torch.zeros((128, 128))], grads(128, 128)) == 100 * (2 if backward else 1)
+    att = SparseAttention(mask=torch.ones((128, 128), dtype=torch.uint8))
+    qkv = [torch.rand((1, 128, 128)) for _ in range(3)]
+    expected = (27 + 1) * (6 if backward else 2) + 45 * (2 if backward else 1)
+    assert _count_trials(att, qkv, [torch.rand((1, 128, 128))] if backward else None) == expected
+
+
+def test_grid_and_random_tuners():
+    from sparta_amd.nn.module_tuner import GridSearchTuner, RandomSearchTuner
+    from sparta_amd.common.tuning import TunableItemCfg
+    space = {'a': TunableItemCfg('choice', [1, 2]), 'b': TunableItemCfg('choice', [10, 20, 30])}
+    seen = []
+    t = GridSearchTuner(space, lambda i, c: seen.append((i, c['a'], c['b'])) or c['a'] * c['b'])
+    t.tune()
+    assert [(a, b) for _, a, b in seen] == [(1, 10), (1, 20), (1, 30), (2, 10), (2, 20), (2, 30)]  # last fastest
+    assert t.best_config == {'a': 1, 'b': 10} and t.best_result == 10
+    seen.clear()
+    random.seed(0)
+    r = RandomSearchTuner(space, lambda i, c: seen.append(c) or 0.0, max_trials=4)
+    r.tune()
+    assert len(seen) == 4 and all(c['a'] in (1, 2) and c['b'] in (10, 20, 30) for c in seen)
+    empty = GridSearchTuner({}, lambda i, c: 1.0)
+    empty.tune()
+    assert empty.best_config == {}
+
+
+def test_operator_argument_errors():
+    lin = torch.nn.Linear(32, 64)
+    with pytest.raises(ValueError):
+        SparseLinear(lin)
+    with pytest.raises(ValueError):
+        SparseLinear(torch.nn.Conv1d(1, 1, 1), weight_mask=torch.ones((64, 32)))
+    with pytest.raises(AssertionError):
+        SparseLinear(lin, weight_mask=torch.ones((32, 64)))
+    op = SparseLinear(lin, weight_mask=torch.ones((64, 32)))
+    with pytest.raises(ValueError):
+        op.update_mask(input_mask=torch.ones((4, 32)), weight_mask=torch.ones((64, 32)))
+    with pytest.raises(ValueError):
+        SparseBatchMatMul()
+    with pytest.raises(AssertionError):
+        SparseSoftmax(mask=torch.ones((8, 8))).update_mask(torch.ones((4, 8)))
+    with pytest.warns(UserWarning, match='not compiled'):
+        y = op(torch.zeros((2, 32)))
+    assert y.shape == (2, 64)
+    from sparta_amd.specializer.kernels import SparTASparseMatMulKernel, OpenAISparseMatMulKernel
+    with pytest.raises(ValueError):
+        SparTASparseMatMulKernel(mode='ddd')
+    with pytest.raises(ValueError, match='not compiled'):
+        SparTASparseMatMulKernel(mode='dsd')(None, None)
+    with pytest.raises(AssertionError):
+        OpenAISparseMatMulKernel(mode='dsd')._check_parameters({'BLOCK_SIZE_K_VALUE': 32})
+    with pytest.raises(AssertionError):
+        SparTASparseMatMulKernel(mode='dsd')._check_parameters(
+            {'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 8, 'BLOCK_SIZE_N_VALUE': 32})
+
+
+def test_search_space_filtering_by_fixed_params():
+    from sparta_amd.specializer.kernels import SparTASparseMatMulKernel, OpenAISparseMatMulKernel
+    k = SparTASparseMatMulKernel(mode='dsd')
+    space = k.get_search_space({'BLOCK_SIZE_K_VALUE': 64})
+    assert space['BLOCK_SIZE_K_VALUE']._value == [64] and space['BLOCK_SIZE_M_VALUE']._value == [16, 32, 64]
+    assert k.get_search_space({'BLOCK_SIZE_K_VALUE': 128}) is None
+    assert k.get_search_space({'NOT_A_PARAM': 1}) is None
+    assert OpenAISparseMatMulKernel(mode='dsd').get_search_space({'BLOCK_SIZE_K_VALUE': 32}) is None
+    assert OpenAISparseMatMulKernel(mode='dsd').get_search_space({'BLOCK_SIZE_K_VALUE': 64}) is not None
+    k.set_parameters({'_impl': 'sparta', '_name': 'x', 'THREAD_SIZE_M_VALUE': 4})  # tolerated keys
