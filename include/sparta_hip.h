@@ -182,15 +182,20 @@ int spx_attention_forward(int dtype, const void* q, const void* k, const void* v
  * (csrc/moe_sparse_forward.cpp:7-25, csrc/moe_sparse_forward_kernel.cu.j2:58-116,
  * :120-325, :363-483) with a stable counting sort (no per-expert capacity) and a
  * gathered GEMM over a flattened (expert, row-tile) list.
- *   exp_ids int32 [n_tok]; expert_count int32 [n_exp];
+ *   exp_ids int32 [n_tok], every value in [0, n_exp); expert_count int32 [n_exp];
  *   expert_offset int32 [n_exp+1] exclusive prefix; token_perm int32 [n_tok]:
  *   token_perm[expert_offset[e] + j] = j-th token (ascending) routed to e.
- *   tokens [n_tok,in_dim]; weight [n_exp,in_dim,out_dim]; out [n_tok,out_dim].
+ *   workspace: spx_moe_index_workspace_bytes(n_tok, n_exp) bytes, 256-byte aligned.
+ *   tokens [n_tok,in_dim]; out [n_tok,out_dim];
+ *   weight [n_exp,in_dim,out_dim] (weight_layout 0, the reference's stacked
+ *   weight.T, sparse_moe.py:19-22) or [n_exp,out_dim,in_dim] (weight_layout 1, the
+ *   layout of nn.Linear.weight; in_dim contiguous, the faster one here).
  * ------------------------------------------------------------------------ */
+size_t spx_moe_index_workspace_bytes(int n_tok, int n_exp);
 int spx_moe_index(const int32_t* exp_ids, int n_tok, int n_exp,
                   int32_t* expert_count, int32_t* expert_offset, int32_t* token_perm,
-                  spx_stream_t stream);
-int spx_moe_forward(int dtype, const void* tokens, const void* weight, void* out,
+                  void* workspace, size_t workspace_bytes, spx_stream_t stream);
+int spx_moe_forward(int dtype, const void* tokens, const void* weight, int weight_layout, void* out,
                     const int32_t* expert_offset, const int32_t* token_perm,
                     int n_tok, int in_dim, int out_dim, int n_exp,
                     int tile_cfg, spx_stream_t stream);

@@ -1,0 +1,400 @@
+// MoE sparse forward: out[t,:] = tokens[t,:] . W[exp_ids[t]].
+//
+//  spx_moe_index   stable counting sort of the tokens by expert, three launches,
+//                  no atomics on global memory, no per-expert capacity, no host
+//                  round trip: (1) per-chunk histograms, (2) one workgroup scans
+//                  them in (expert, chunk) order, (3) every chunk places its
+//                  tokens in ascending order behind its scanned base.
+//  spx_moe_forward one gathered GEMM over a flattened (expert, 128-row tile) list:
+//                  a workgroup looks its tile up in the prefix of per-expert tile
+//                  counts, gathers its token rows through token_perm, and walks
+//                  K in 64-wide stages through LDS ([row][k], XOR-swizzled 16-byte
+//                  chunks) into 16x16 MFMAs; rows are scattered back on store.
+// Replaces convert_sparse_index / BATCH_BLOCK_SPARSE_MATMUL[_FP16] of the
+// reference (csrc/moe_sparse_forward_kernel.cu.j2:58-71,120-325,363-483), whose
+// grid is sized by the largest expert and whose fp16 path accumulates in fp16.
+#include "common.hpp"
+#include "mma.hpp"
+
+namespace spx {
+
+constexpr int MOE_CHUNK = 1024;   // tokens per workgroup in the index kernels
+constexpr int MOE_MAX_EXP = 2048; // LDS table capacity of the placement kernel
+
+// ---- index -------------------------------------------------------------------
+__global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, int n_tok, int n_exp,
+                                                       int32_t* partial /* [n_chunk][n_exp] */) {
+    extern __shared__ int hist[];
+    for (int e = threadIdx.x; e < n_exp; e += 256) hist[e] = 0;
+    __syncthreads();
+    const int base = blockIdx.x * MOE_CHUNK;
+    for (int i = threadIdx.x; i < MOE_CHUNK; i += 256) {
+        const int t = base + i;
+        if (t < n_tok) {
+            const int e = exp_ids[t];
+            if (e >= 0 && e < n_exp) atomicAdd(&hist[e], 1);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < n_exp; e += 256) partial[(int64_t)blockIdx.x * n_exp + e] = hist[e];
+}
+
+// One workgroup: exclusive scan of partial[] in (expert, chunk) order, in place;
+// also writes expert_count and expert_offset.
+__global__ __launch_bounds__(1024) void moe_scan_kernel(int32_t* partial, int n_chunk, int n_exp,
+                                                        int32_t* expert_count, int32_t* expert_offset) {
+    __shared__ int lds[32];
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int n = n_chunk * n_exp;
+    int carry = 0;
+    if (n == 0)
+        for (int e = threadIdx.x; e < n_exp; e += 1024) expert_offset[e] = 0;
+    for (int base = 0; base < n; base += 1024) {
+        const int i = base + threadIdx.x;  // position in (expert, chunk) order
+        int v = 0, e = 0, c = 0;
+        if (i < n) {
+            e = i / n_chunk;
+            c = i - e * n_chunk;
+            v = partial[(int64_t)c * n_exp + e];
+        }
+        const int inc = wave_inclusive_scan(v);
+        if (lane == 63) lds[wave] = inc;
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int w = 0; w < 16; ++w) {
+            const int t = lds[w];
+            if (w < wave) before += t;
+            total += t;
+        }
+        if (i < n) {
+            const int excl = carry + before + inc - v;
+            partial[(int64_t)c * n_exp + e] = excl;
+            if (c == 0) expert_offset[e] = excl;
+        }
+        carry += total;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) expert_offset[n_exp] = carry;
+    __syncthreads();
+    // counts from consecutive offsets (offsets were written by this workgroup)
+    for (int e = threadIdx.x; e < n_exp; e += 1024) expert_count[e] = expert_offset[e + 1] - expert_offset[e];
+}
+
+// Stable placement of one chunk.  Waves take 64 tokens at a time; inside a wave the
+// rank among equal experts comes from ballots, between waves from a small table.
+__global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, int n_tok, int n_exp,
+                                                        const int32_t* base_of /* scanned partial */,
+                                                        int32_t* token_perm) {
+    extern __shared__ int sm[];
+    int* running = sm;               // [n_exp] tokens of expert e already placed by this chunk
+    int* wavecnt = sm + n_exp;       // [4][n_exp] tokens of expert e in the current pass, per wave
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 5 * n_exp; i += 256) sm[i] = 0;
+    __syncthreads();
+    const int chunk0 = blockIdx.x * MOE_CHUNK;
+    const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (int pass = 0; pass < MOE_CHUNK; pass += 256) {
+        const int t = chunk0 + pass + threadIdx.x;
+        int e = -1;
+        if (t < n_tok) {
+            e = exp_ids[t];
+            if (e < 0 || e >= n_exp) e = -1;
+        }
+        // intra-wave rank and per-wave count of my expert
+        int rank = 0, cnt = 0;
+        bool leader = false;
+        unsigned long long todo = __ballot(e >= 0);
+        while (todo) {
+            const int src = __ffsll((long long)todo) - 1;
+            const int e0 = __shfl(e, src, 64);
+            const unsigned long long same = __ballot(e == e0);
+            if (e == e0) {
+                rank = __popcll(same & lt_mask);
+                cnt = __popcll(same);
+                leader = lane == src;
+            }
+            todo &= ~same;
+        }
+        if (leader) wavecnt[wave * n_exp + e] = cnt;
+        __syncthreads();
+        if (e >= 0) {
+            int before = running[e];
+            for (int w = 0; w < wave; ++w) before += wavecnt[w * n_exp + e];
+            token_perm[base_of[(int64_t)blockIdx.x * n_exp + e] + before + rank] = t;
+        }
+        __syncthreads();
+        if (leader) {
+            atomicAdd(&running[e], cnt);
+            wavecnt[wave * n_exp + e] = 0;
+        }
+        __syncthreads();
+    }
+}
+
+// ---- gathered GEMM -------------------------------------------------------------
+struct MoeParams {
+    const void* tokens;
+    const void* weight;
+    void* out;
+    const int32_t* expert_offset;
+    const int32_t* token_perm;
+    int n_tok, K, N, n_exp;
+    int w_kcontig;  // weight [E, N, K] if set, else [E, K, N]
+};
+
+constexpr int MOE_TM = 128, MOE_TN = 128;
+// k per LDS stage: 128 bytes per row for every element type
+template <typename T> struct MoeKt { static constexpr int value = 128 / (int)sizeof(T); };
+
+// LDS tile: rows of 128 bytes = 8 chunks of 16 bytes; chunk c of row r is stored at
+// chunk position c ^ (r & 7).
+template <typename T>
+__device__ __forceinline__ int moe_lds_off(int row, int chunk) {
+    return (row * 8 + (chunk ^ (row & 7))) * 16;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int MOE_KT = MoeKt<T>::value;
+    constexpr int CPR = MOE_KT / VE;                 // 16-byte chunks per LDS row (8)
+    constexpr int TILE_BYTES = MOE_TM * MOE_KT * (int)sizeof(T);
+    extern __shared__ __align__(16) char smem[];
+    char* As = smem;
+    char* Bs = smem + TILE_BYTES;
+    __shared__ int s_expert, s_row0, s_rows;
+
+    // ---- which (expert, row tile) is mine ------------------------------------------
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const int y = blockIdx.y;
+        int tiles_before = 0;
+        int found_e = -1, found_row0 = 0, found_rows = 0;
+        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
+            const int e = e0 + lane;
+            int cnt = 0, off = 0;
+            if (e < p.n_exp) {
+                off = p.expert_offset[e];
+                cnt = p.expert_offset[e + 1] - off;
+            }
+            const int tiles = (cnt + MOE_TM - 1) / MOE_TM;
+            const int inc = wave_inclusive_scan(tiles);
+            const int excl = tiles_before + inc - tiles;
+            const bool mine = y >= excl && y < excl + tiles;
+            const unsigned long long hit = __ballot(mine);
+            if (hit) {
+                const int src = __ffsll((long long)hit) - 1;
+                const int lt = y - __shfl(excl, src, 64);
+                found_e = e0 + src;
+                found_row0 = __shfl(off, src, 64) + lt * MOE_TM;
+                found_rows = min(MOE_TM, __shfl(cnt, src, 64) - lt * MOE_TM);
+            }
+            tiles_before += __shfl(inc, 63, 64);
+        }
+        if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
+    }
+    __syncthreads();
+    const int expert = s_expert;
+    if (expert < 0) return;  // uniform: this tile index is past the last tile
+    const int row0 = s_row0, rows = s_rows;
+    const int n0 = blockIdx.x * MOE_TN;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;  // 2 x 2 waves, each 64 x 64
+
+    const T* X = reinterpret_cast<const T*>(p.tokens);
+    const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
+
+    // staging map: thread -> (row, 16-byte chunk) pairs; 128 rows x CPR chunks per tile
+    constexpr int LOADS = MOE_TM * CPR / 256;
+    int a_tok[LOADS];
+#pragma unroll
+    for (int q = 0; q < LOADS; ++q) {
+        const int v = q * 256 + threadIdx.x;
+        const int r = v / CPR;
+        a_tok[q] = p.token_perm[row0 + (r < rows ? r : rows - 1)];
+    }
+
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    for (int k0 = 0; k0 < p.K; k0 += MOE_KT) {
+        // ---- stage A (gathered token rows) and B (weight rows n0..n0+127) ---------------
+#pragma unroll
+        for (int q = 0; q < LOADS; ++q) {
+            const int v = q * 256 + threadIdx.x;
+            const int r = v / CPR, c = v % CPR;
+            const u32x4 val = *reinterpret_cast<const u32x4*>(X + (int64_t)a_tok[q] * p.K + k0 + c * VE);
+            *reinterpret_cast<u32x4*>(As + moe_lds_off<T>(r, c)) = val;
+        }
+        if (p.w_kcontig) {
+#pragma unroll
+            for (int q = 0; q < LOADS; ++q) {
+                const int v = q * 256 + threadIdx.x;
+                const int r = v / CPR, c = v % CPR;
+                const int n = n0 + r < p.N ? n0 + r : p.N - 1;
+                const u32x4 val = *reinterpret_cast<const u32x4*>(W + (int64_t)n * p.K + k0 + c * VE);
+                *reinterpret_cast<u32x4*>(Bs + moe_lds_off<T>(r, c)) = val;
+            }
+        } else {
+            // weight stored [K, N]: 16-byte loads along n, transposed into [n][k]
+            constexpr int NV = MOE_TN / VE;  // vectors per k row
+            for (int v = threadIdx.x; v < MOE_KT * NV; v += 256) {
+                const int k = v / NV, nv = v % NV;
+                union { u32x4 v4; T e[VE]; } u;
+                const int n = n0 + nv * VE;
+                if (n + VE <= p.N) {
+                    u.v4 = *reinterpret_cast<const u32x4*>(W + (int64_t)(k0 + k) * p.N + n);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < VE; ++i) u.e[i] = W[(int64_t)(k0 + k) * p.N + (n + i < p.N ? n + i : p.N - 1)];
+                }
+#pragma unroll
+                for (int i = 0; i < VE; ++i) {
+                    const int r = nv * VE + i;
+                    reinterpret_cast<T*>(Bs + moe_lds_off<T>(r, k / VE))[k % VE] = u.e[i];
+                }
+            }
+        }
+        __syncthreads();
+        // ---- MFMA over the stage -----------------------------------------------------------
+        if constexpr (HasMma32<T>::value) {
+#pragma unroll
+            for (int kc = 0; kc < MOE_KT; kc += 32) {
+                typename Mma32<T>::frag af[4], bf[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma32<T>::frag*>(As + moe_lds_off<T>(wm * 64 + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma32<T>::frag*>(Bs + moe_lds_off<T>(wn * 64 + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[i][t] = Mma32<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < MOE_KT; kc += 16) {
+                typename Mma16<T>::frag af[4], bf[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wm * 64 + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wn * 64 + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- scatter the rows back: lane holds out[m = i*16 + r16][n = t*16 + g4*4 .. +3] -----
+    T* out = reinterpret_cast<T*>(p.out);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = wm * 64 + i * 16 + r16;
+        if (r >= rows) continue;
+        const int tok = p.token_perm[row0 + r];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int n = n0 + wn * 64 + t * 16 + g4 * 4;
+            T vals[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
+            T* dst = out + (int64_t)tok * p.N + n;
+            if (n + 4 <= p.N) {
+                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+            } else {
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < p.N) dst[q] = vals[q];
+            }
+        }
+    }
+}
+
+static size_t moe_index_ws(int n_tok, int n_exp) {
+    const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
+    return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * n_exp * sizeof(int32_t), 256);
+}
+
+}  // namespace spx
+
+extern "C" size_t spx_moe_index_workspace_bytes(int n_tok, int n_exp) {
+    if (n_tok < 0 || n_exp <= 0 || n_exp > spx::MOE_MAX_EXP) return 0;
+    return spx::moe_index_ws(n_tok, n_exp);
+}
+
+extern "C" int spx_moe_index(const int32_t* exp_ids, int n_tok, int n_exp,
+                             int32_t* expert_count, int32_t* expert_offset, int32_t* token_perm,
+                             void* workspace, size_t workspace_bytes, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(n_tok >= 0, SPX_E_SHAPE, "negative token count");
+    SPX_REQUIRE(n_exp > 0 && n_exp <= MOE_MAX_EXP, SPX_E_SHAPE, "n_exp=%d must be in [1,%d]", n_exp, MOE_MAX_EXP);
+    SPX_REQUIRE(expert_count && expert_offset && workspace, SPX_E_NULL, "expert_count, expert_offset and workspace are required");
+    SPX_REQUIRE((exp_ids && token_perm) || n_tok == 0, SPX_E_NULL, "exp_ids and token_perm are required");
+    SPX_REQUIRE(workspace_bytes >= moe_index_ws(n_tok, n_exp), SPX_E_WORKSPACE,
+                "workspace of %zu bytes is smaller than the %zu required", workspace_bytes, moe_index_ws(n_tok, n_exp));
+    SPX_REQUIRE(aligned(workspace, 256), SPX_E_ALIGN, "workspace must be 256-byte aligned");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    int32_t* partial = reinterpret_cast<int32_t*>(workspace);
+    const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
+    if (n_chunk > 0) {
+        hipLaunchKernelGGL(moe_hist_kernel, dim3(n_chunk), dim3(256), n_exp * sizeof(int), st, exp_ids, n_tok, n_exp, partial);
+        SPX_LAUNCH_CHECK("moe_hist_kernel");
+    }
+    hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, st, partial, n_chunk, n_exp, expert_count, expert_offset);
+    SPX_LAUNCH_CHECK("moe_scan_kernel");
+    if (n_chunk > 0) {
+        hipLaunchKernelGGL(moe_place_kernel, dim3(n_chunk), dim3(256), 5 * n_exp * sizeof(int), st, exp_ids, n_tok, n_exp,
+                           partial, token_perm);
+        SPX_LAUNCH_CHECK("moe_place_kernel");
+    }
+    return 0;
+}
+
+extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight, int weight_layout, void* out,
+                               const int32_t* expert_offset, const int32_t* token_perm,
+                               int n_tok, int in_dim, int out_dim, int n_exp,
+                               int tile_cfg, spx_stream_t stream) {
+    using namespace spx;
+    (void)tile_cfg;
+    SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
+    SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
+    SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
+    const int es = dtype_bytes(dtype);
+    SPX_REQUIRE(in_dim % (128 / es) == 0, SPX_E_SHAPE, "in_dim=%d must be a multiple of %d", in_dim, 128 / es);
+    SPX_REQUIRE(out_dim % (16 / es) == 0, SPX_E_SHAPE, "out_dim=%d must be a multiple of %d", out_dim, 16 / es);
+    if (n_tok == 0) return 0;
+    SPX_REQUIRE(tokens && weight && out && expert_offset && token_perm, SPX_E_NULL, "a required buffer is NULL");
+    SPX_REQUIRE(aligned(tokens, 16) && aligned(weight, 16) && aligned(out, 16), SPX_E_ALIGN, "buffers must be 16-byte aligned");
+    MoeParams p;
+    p.tokens = tokens; p.weight = weight; p.out = out;
+    p.expert_offset = expert_offset; p.token_perm = token_perm;
+    p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
+    p.w_kcontig = weight_layout == 1;
+    const int max_tiles = (n_tok + MOE_TM - 1) / MOE_TM + n_exp;
+    SPX_REQUIRE(max_tiles <= 65535, SPX_E_SHAPE, "too many row tiles for one launch");
+    dim3 grid((out_dim + MOE_TN - 1) / MOE_TN, max_tiles, 1);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const size_t smem = 2 * (size_t)MOE_TM * 128;
+    switch (dtype) {
+        case SPX_F32: hipLaunchKernelGGL(moe_gemm_kernel<float>, grid, dim3(256), smem, st, p); break;
+        case SPX_F16: hipLaunchKernelGGL(moe_gemm_kernel<_Float16>, grid, dim3(256), smem, st, p); break;
+        default: hipLaunchKernelGGL(moe_gemm_kernel<bf16_t>, grid, dim3(256), smem, st, p); break;
+    }
+    SPX_LAUNCH_CHECK("moe_gemm_kernel");
+    return 0;
+}

@@ -31,6 +31,11 @@ class DynamicSparseMoE(torch.nn.Module):
             # [n_exp, in, out]: each expert's weight transposed once, up front
             stacked = torch.stack([m.weight.t() for m in exp_modules]).contiguous()
         self.weight = torch.nn.Parameter(stacked)
+        # [n_exp, out, in] copy (in contiguous): the layout the GEMM kernel reads fastest.
+        # It is refreshed whenever `weight` has been modified in place.
+        self._weight_nk = None
+        self._weight_nk_version = -1
+        self._workspace = torch.zeros(0, dtype=torch.uint8, device=self.device)
         i32 = dict(dtype=torch.int32, device=self.device)
         self.expert_count = torch.zeros(self.num_exps, **i32)
         self.expert_offset = torch.zeros(self.num_exps + 1, **i32)
@@ -46,15 +51,24 @@ class DynamicSparseMoE(torch.nn.Module):
         if self.sparse_index.numel() < n_tok:
             self.sparse_index = torch.empty(n_tok, dtype=torch.int32, device=tokens.device)
         lib = _lib.load()
+        ws_bytes = lib.spx_moe_index_workspace_bytes(n_tok, self.num_exps)
+        if self._workspace.numel() < ws_bytes:
+            self._workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=tokens.device)
+        if self._weight_nk is None or self._weight_nk_version != self.weight._version:
+            with torch.no_grad():
+                self._weight_nk = self.weight.detach().transpose(1, 2).contiguous()
+            self._weight_nk_version = self.weight._version
         stream = _lib.current_stream(tokens.device)
         rc = lib.spx_moe_index(_lib.dev_ptr(exp_ids.contiguous()), n_tok, self.num_exps,
                                _lib.dev_ptr(self.expert_count), _lib.dev_ptr(self.expert_offset),
-                               _lib.dev_ptr(self.sparse_index), stream)
+                               _lib.dev_ptr(self.sparse_index), _lib.dev_ptr(self._workspace),
+                               self._workspace.numel(), stream)
         _lib.check(rc, 'spx_moe_index')
         tokens = tokens.contiguous()
         out = torch.empty((n_tok, self.out_hidden), dtype=tokens.dtype, device=tokens.device)
+        weight = self._weight_nk.to(tokens.dtype) if self._weight_nk.dtype != tokens.dtype else self._weight_nk
         rc = lib.spx_moe_forward(_lib.dtype_code(tokens.dtype), _lib.dev_ptr(tokens),
-                                 _lib.dev_ptr(self.weight.detach()), _lib.dev_ptr(out),
+                                 _lib.dev_ptr(weight), 1, _lib.dev_ptr(out),
                                  _lib.dev_ptr(self.expert_offset), _lib.dev_ptr(self.sparse_index),
                                  n_tok, self.in_hidden, self.out_hidden, self.num_exps, 0, stream)
         _lib.check(rc, 'spx_moe_forward')
