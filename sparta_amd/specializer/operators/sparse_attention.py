@@ -42,6 +42,8 @@ class SparseAttention(OperatorBase):
         self._matmul_out = SparseBatchMatMul(A_mask=mask, transpose_A=False, transpose_B=False, compressed=True)
         self._sparse_port: Optional[PortConfig] = None
         self._fused = fused
+        self._fused_mask_key = None   # index object the cached element mask belongs to
+        self._fused_mask = None
         self._inv_temperature = 1.0
         self.ready = False
 
@@ -50,15 +52,28 @@ class SparseAttention(OperatorBase):
 
     # ---- forward ---------------------------------------------------------------------
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
-        if self.ready and self._fused and not (
+        if self.ready and self._fused and self._fused_supported(query) and not (
                 torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)):
             return self._fused_forward(query, key, value)
         scores = self._matmul_qk.forward(query, key)
         probs = self._softmax.forward(scores)
         return self._matmul_out.forward(probs, value)
 
+    def _fused_supported(self, query: torch.Tensor) -> bool:
+        """The fused kernel covers 16-bit inputs, head dims 32 / 64 / 128 and score
+        blocks of 16..128; everything else takes the three-operator pipeline."""
+        indexes = self._sparse_port.indexes
+        return (query.dtype in (torch.float16, torch.bfloat16) and query.shape[-1] in (32, 64, 128)
+                and indexes.block_H in (16, 32, 64, 128) and indexes.block_W in (16, 32, 64, 128))
+
     def _fused_forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
         indexes = self._sparse_port.indexes
+        if self._fused_mask_key is not indexes:
+            # A mask that is uniform inside its blocks needs no per-element test in the
+            # kernel; decided once per index build (one synchronising comparison).
+            block_level = torch.equal(indexes.get_mask(), indexes.raw_mask != 0)
+            self._fused_mask = None if block_level else indexes.raw_mask
+            self._fused_mask_key = indexes
         lead = query.shape[:-2]
         E = query.shape[-1]
         batch = int(np.prod(lead)) if len(lead) else 1
@@ -66,7 +81,7 @@ class SparseAttention(OperatorBase):
         out = torch.empty_like(q)
         rc = _lib.load().spx_attention_forward(
             _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
-            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(indexes.raw_mask),
+            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(self._fused_mask),
             float(self._inv_temperature), batch, self._Nt, self._Ns, E,
             indexes.block_H, indexes.block_W, 0, _lib.current_stream(q.device))
         _lib.check(rc, 'spx_attention_forward')
