@@ -195,6 +195,156 @@ __global__ __launch_bounds__(1024) void emit_kernel(EmitParams p) {
     }
 }
 
+// Fast path of the emit step for block grids of at most 2048 row words and 2048
+// column words: every thread owns two consecutive words, the prefix sums run in
+// registers + LDS, and only the final arrays touch global memory.
+constexpr int EMIT_FAST_WORDS = 2048;
+
+__device__ __forceinline__ int block_exclusive_scan_1024(int v, int* lds, int* total) {
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int inc = wave_inclusive_scan(v);
+    __syncthreads();  // lds may still be read from a previous call
+    if (lane == 63) lds[wave] = inc;
+    __syncthreads();
+    int before = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const int t = lds[w];
+        if (w < wave) before += t;
+        tot += t;
+    }
+    *total = tot;
+    return before + inc - v;
+}
+
+__global__ __launch_bounds__(1024) void emit_fast_kernel(EmitParams p) {
+    __shared__ unsigned long long s_bits[EMIT_FAST_WORDS];
+    __shared__ int s_base[EMIT_FAST_WORDS];
+    __shared__ int s_scan[16];
+    const int tid = threadIdx.x;
+
+    // ---- row words: word g = r * WPR + wi covers columns wi*64 .. wi*64+63 of row r ----
+    const int NW = p.R * p.WPR;
+    unsigned long long w[2];
+    int cnt[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int g = tid * 2 + i;
+        unsigned long long word = 0;
+        if (g < NW) {
+            const int r = g / p.WPR;
+            const int c0 = (g - r * p.WPR) * 64;
+            const uint8_t* src = p.live + (int64_t)r * p.Cn + c0;
+            const int n = p.Cn - c0 < 64 ? p.Cn - c0 : 64;
+            if ((p.Cn & 7) == 0) {
+                // liveness bytes are 0 or 1: one multiply gathers the low bit of 8 bytes
+                const unsigned long long* src8 = reinterpret_cast<const unsigned long long*>(src);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (k * 8 < n) {
+                        const unsigned long long x = src8[k];
+                        word |= ((x * 0x0102040810204080ULL) >> 56) << (k * 8);
+                    }
+                }
+            } else {
+#pragma unroll 8
+                for (int k = 0; k < n; ++k) word |= (unsigned long long)(src[k] != 0) << k;
+            }
+        }
+        w[i] = word;
+        cnt[i] = __popcll(word);
+    }
+    int nnz;
+    const int tbase = block_exclusive_scan_1024(cnt[0] + cnt[1], s_scan, &nnz);
+    int base[2] = {tbase, tbase + cnt[0]};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int g = tid * 2 + i;
+        if (g < EMIT_FAST_WORDS) { s_bits[g] = w[i]; s_base[g] = base[i]; }
+        if (g < NW) {
+            const int r = g / p.WPR;
+            const int wi = g - r * p.WPR;
+            if (p.row_ptr && wi == 0) p.row_ptr[r] = base[i];
+            if (p.bcsr_idx) {
+                unsigned long long bits = w[i];
+                int pos = base[i];
+                while (bits) {
+                    const int c = __ffsll((long long)bits) - 1;
+                    bits &= bits - 1;
+                    if (pos < p.cap) p.bcsr_idx[pos] = (r << 16) | (wi * 64 + c);
+                    ++pos;
+                }
+            }
+        }
+    }
+    if (tid == 0) {
+        p.nnz_dev[0] = nnz;
+        if (p.row_ptr) p.row_ptr[p.R] = nnz;
+    }
+    if (!p.col_ptr) return;
+    __syncthreads();  // s_bits / s_base complete
+
+    // ---- column words: word g = c * WPC + ri covers rows ri*64 .. ri*64+63 of column c ----
+    const int NWC = p.Cn * p.WPC;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int g = tid * 2 + i;
+        unsigned long long word = 0;
+        if (g < NWC) {
+            const int c = g / p.WPC;
+            const int r0 = (g - c * p.WPC) * 64;
+            const int n = p.R - r0 < 64 ? p.R - r0 : 64;
+            // bit (r, c) comes from the row words already in LDS
+            const int wi = c >> 6, cb = c & 63;
+            const unsigned long long* col = s_bits + r0 * p.WPR + wi;
+            if (n == 64) {
+#pragma unroll 16
+                for (int k = 0; k < 64; ++k) word |= ((col[k * p.WPR] >> cb) & 1ull) << k;
+            } else {
+                for (int k = 0; k < n; ++k) word |= ((col[k * p.WPR] >> cb) & 1ull) << k;
+            }
+        }
+        w[i] = word;
+        cnt[i] = __popcll(word);
+    }
+    int nnz2;
+    const int cbase = block_exclusive_scan_1024(cnt[0] + cnt[1], s_scan, &nnz2);
+    base[0] = cbase;
+    base[1] = cbase + cnt[0];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int g = tid * 2 + i;
+        if (g < NWC) {
+            const int c = g / p.WPC;
+            const int ri = g - c * p.WPC;
+            if (ri == 0) p.col_ptr[c] = base[i];
+            if (p.bcsc_idx) {
+                unsigned long long bits = w[i];
+                int pos = base[i];
+                const int wi = c >> 6, cb = c & 63;
+                while (bits) {
+                    const int k = __ffsll((long long)bits) - 1;
+                    bits &= bits - 1;
+                    const int r = ri * 64 + k;
+                    if (pos < p.cap) {
+                        if (p.bcsc_i64) {
+                            const int gw = r * p.WPR + wi;
+                            const unsigned long long below = cb == 0 ? 0ull : (s_bits[gw] & (~0ull >> (64 - cb)));
+                            const long long bpos = s_base[gw] + __popcll(below);
+                            reinterpret_cast<long long*>(p.bcsc_idx)[pos] = (bpos << 32) | ((long long)c << 16) | (long long)r;
+                        } else {
+                            reinterpret_cast<int32_t*>(p.bcsc_idx)[pos] = (c << 16) | r;
+                        }
+                    }
+                    ++pos;
+                }
+            }
+        }
+    }
+    if (tid == 0) p.col_ptr[p.Cn] = nnz2;
+}
+
 struct IndexWorkspace {
     size_t live_off, wbits_off, wbase_off, cbase_off, total;
     int R, Cn, WPR, WPC;
@@ -295,7 +445,10 @@ extern "C" int spx_bcs_index(const uint8_t* mask, int H, int W, int BH, int BW,
     ep.col_ptr = col_ptr; ep.bcsc_idx = bcsc_idx; ep.bcsc_i64 = bcsc_i64;
     ep.nnz_dev = nnz_dev; ep.cap = cap;
     ep.R = ws.R; ep.Cn = ws.Cn; ep.WPR = ws.WPR; ep.WPC = ws.WPC;
-    hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
+    if (ws.R * ws.WPR <= EMIT_FAST_WORDS && ws.Cn * ws.WPC <= EMIT_FAST_WORDS)
+        hipLaunchKernelGGL(emit_fast_kernel, dim3(1), dim3(1024), 0, st, ep);
+    else
+        hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
     SPX_LAUNCH_CHECK("emit_kernel");
     return 0;
 }

@@ -202,7 +202,8 @@ def _capture_samples(module: torch.nn.Module, sample_inputs, sample_grads, with_
 def tune_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Tensor],
                          sample_grads: Optional[List[torch.Tensor]] = None, algo: str = 'grid',
                          max_trials: int = sys.maxsize, backward_weight: float = 0,
-                         verbose: bool = False, debug_func: Optional[Callable] = None):
+                         verbose: bool = False, debug_func: Optional[Callable] = None,
+                         tile_configs: bool = False):
     """Find, tune and build every sparse operator inside `module`.
 
     Args:
@@ -214,11 +215,22 @@ def tune_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Tens
         backward_weight: weight of backward latencies; 0 tunes forward kernels only.
         verbose: log every trial.
         debug_func: replaces build + measurement of a trial (for tests).
+        tile_configs: also search the gfx950 tile configurations of the matmul
+            kernels (parameter TILE_CFG); off by default, which leaves exactly the
+            reference's search space.
 
     Returns:
         {operator name: best config}; names are 'root' or 'root/child/...'.
     """
     inputs, grads = _capture_samples(module, sample_inputs, sample_grads, backward_weight > 0)
+
+    def set_tile_search(op: OperatorBase, name: str):
+        for placeholder in op.get_kernel_placeholders(backward=True).values():
+            for kernel in placeholder.possible_kernels.values():
+                if hasattr(kernel, 'enable_tile_search'):
+                    kernel.enable_tile_search(tile_configs)
+
+    iter_sparse_modules(module, 'root', set_tile_search)
     _logger.setLevel(logging.DEBUG if verbose else logging.WARNING)
     best_configs = {}
 
