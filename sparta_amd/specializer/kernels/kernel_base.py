@@ -46,6 +46,10 @@ class PortConfig:
     def __post_init__(self):
         self.mask: Optional[torch.Tensor] = None
         self.indexes: Optional[BCSIndexes] = None
+        # Dynamic masks: keep compressed values at index capacity and let kernels read
+        # the live block count from device memory, so a mask update never waits for
+        # the host.
+        self.at_capacity = False
         self._block_H = 0
         self._block_W = 0
 
@@ -78,6 +82,7 @@ class PortConfig:
         assert self.is_sparse == other.is_sparse, 'cannot connect a sparse port with a dense one'
         self.BCSR = self.BCSR or other.BCSR
         self.BCSC = self.BCSC or other.BCSC
+        self.at_capacity = self.at_capacity or other.at_capacity
         kernel.ports[port_name] = self
 
 

@@ -144,8 +144,15 @@ class SparseMatMulKernel(KernelBase):
             ptr, idx = indexes.col_ptr, indexes._bcsc_buf
             idx_kind = _lib.IDX_BCSC_I64 if idx.dtype == torch.int64 else _lib.IDX_BCSC_I32
         dds = self._mode == 'dds'
-        # Only a compressed operand / a sparse output need the live block count on the host.
-        nnz = indexes.block_nnz if (compressed or dds) else 0
+        # Only a compressed operand / a sparse output need the live block count on the
+        # host; a port in at-capacity mode leaves it on the device.
+        at_capacity = self.ports[self._sparse_port].at_capacity
+        nnz_dev_p = None
+        if at_capacity:
+            nnz = indexes.capacity
+            nnz_dev_p = _lib.dev_ptr(indexes.nnz_dev)
+        else:
+            nnz = indexes.block_nnz if (compressed or dds) else 0
         sparse_stride = nnz * tile_elems
         if dds and compressed:
             C_shape = (batch_size, nnz * BM * BN)
@@ -165,7 +172,7 @@ class SparseMatMulKernel(KernelBase):
             rc = lib.spx_matmul(
                 mode_code, _lib.dtype_code(A.dtype), tA, tB, compressed,
                 _lib.dev_ptr(A.contiguous()), _lib.dev_ptr(B.contiguous()), _lib.dev_ptr(bias), _lib.dev_ptr(C),
-                ptr_p, idx_p, idx_kind, nnz, None, sparse_stride,
+                ptr_p, idx_p, idx_kind, nnz, nnz_dev_p, sparse_stride,
                 batch_size, M, K, N, BM, BK, BN, tile_cfg, _lib.current_stream(A.device))
             _lib.check(rc, 'spx_matmul')
             return C
@@ -188,7 +195,8 @@ class SparseMatMulKernel(KernelBase):
             if self._sparse_port == 'C':
                 outputs[0] = indexes.convert(outputs[0])
             else:
-                inputs[masked] = indexes.convert(inputs[masked])
+                inputs[masked] = indexes.convert(inputs[masked],
+                                                 at_capacity=self.ports[self._sparse_port].at_capacity)
 
     def reference(self, *args):
         """Masked-dense result; the sparse-output mode multiplies by the block

@@ -16,6 +16,10 @@ class SparseLinear(OperatorBase):
             after `build` the `weight` parameter holds the BCSR-compressed values.
         output_mask: mask of the output [batch, out_features] -> 'dds' kernel, dense storage.
         Exactly one of the three masks must be given.
+        dynamic: the mask changes every few steps.  Compressed weights are then kept
+            at full capacity and `update_mask` enqueues the index rebuild and the
+            re-compression without ever waiting for the host (the reference
+            synchronises once per rebuild).
 
     Shape: input (B, in_features) -> output (B, out_features).
 
@@ -33,7 +37,8 @@ class SparseLinear(OperatorBase):
     _PORT_OF = {'input': 'A', 'weight': 'B', 'output': 'C'}
 
     def __init__(self, raw_module: torch.nn.Linear, input_mask: Optional[torch.Tensor] = None,
-                 weight_mask: Optional[torch.Tensor] = None, output_mask: Optional[torch.Tensor] = None):
+                 weight_mask: Optional[torch.Tensor] = None, output_mask: Optional[torch.Tensor] = None,
+                 dynamic: bool = False):
         super().__init__(raw_module)
         N, K = raw_module.weight.shape
         biased = raw_module.bias is not None
@@ -52,6 +57,8 @@ class SparseLinear(OperatorBase):
         else:
             raise ValueError('expected a sparse mask on input / weight / output')
         self._shape = {'batch_size': 1, 'M': M, 'K': K, 'N': N}
+        self._dynamic = dynamic
+        self._set_dynamic(dynamic)
         self.update_mask(input_mask, weight_mask, output_mask)
 
     def update_mask(self, input_mask: Optional[torch.Tensor] = None,
@@ -87,7 +94,7 @@ class SparseLinear(OperatorBase):
         weight = self._raw_weight
         indexes = self.get_sparse_indexes('B')
         if indexes is not None:
-            weight = indexes.convert(weight.detach())
+            weight = indexes.convert(weight.detach(), at_capacity=self._dynamic)
         self.weight = torch.nn.Parameter(weight, requires_grad=True)
 
     def _compile(self, config: Optional[Dict[str, Dict[str, Any]]] = None):

@@ -76,9 +76,16 @@ class BCSIndexes(TeSAIndexes):
         return full.contiguous()
 
     # ---- values ------------------------------------------------------------------
-    def convert(self, dense: torch.Tensor) -> torch.Tensor:
-        """Dense [..., H, W] -> compressed [..., nnz*block_H*block_W]."""
+    def convert(self, dense: torch.Tensor, at_capacity: bool = False) -> torch.Tensor:
+        """Dense [..., H, W] -> compressed [..., nnz*block_H*block_W].
+
+        With `at_capacity` the result has room for `capacity` blocks, of which the
+        first nnz are written; the launch reads nnz from device memory, so nothing
+        synchronises with the host (for masks that change every step)."""
         idx, kind = self._value_index()
+        if at_capacity:
+            return self.function_context.convert(dense, idx, self.capacity, self.H, self.W, idx_kind=kind,
+                                                 nnz_dev=self.nnz_dev)
         return self.function_context.convert(dense, idx, self.block_nnz, self.H, self.W, idx_kind=kind)
 
     def inverse(self, sparse_val: torch.Tensor) -> torch.Tensor:
@@ -218,7 +225,7 @@ class BCSFunctionContext(TeSAFunctionContext):
 
     # ---- values ------------------------------------------------------------------
     def convert(self, dense: torch.Tensor, index: torch.Tensor, block_nnz: int, H: int, W: int,
-                idx_kind: int = _lib.IDX_BCSR_I32) -> torch.Tensor:
+                idx_kind: int = _lib.IDX_BCSR_I32, nnz_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
         assert dense.shape[-2] == H and dense.shape[-1] == W, \
             f'expected a (..., {H}, {W}) tensor, got {tuple(dense.shape)}'
         lead = tuple(dense.shape[:-2])
@@ -227,8 +234,8 @@ class BCSFunctionContext(TeSAFunctionContext):
         out = torch.empty((batch, block_nnz * self._block_size), dtype=dense.dtype, device=dense.device)
         with torch.cuda.device(dense.device):
             rc = _lib.load().spx_bcs_gather(
-                _lib.dev_ptr(dense), _lib.dev_ptr(out), _lib.dev_ptr(index), idx_kind, block_nnz, None,
-                batch, H, W, self._block_H, self._block_W, dense.element_size(),
+                _lib.dev_ptr(dense), _lib.dev_ptr(out), _lib.dev_ptr(index), idx_kind, block_nnz,
+                _lib.dev_ptr(nnz_dev), batch, H, W, self._block_H, self._block_W, dense.element_size(),
                 block_nnz * self._block_size, _lib.current_stream(dense.device))
         _lib.check(rc, 'spx_bcs_gather')
         return out.reshape(lead + (-1,))

@@ -1,0 +1,246 @@
+"""GPU tests of the operator layer (the drop-in API): SparseLinear with each mask
+kind, tune() / build(), mask updates, autograd through the sparse kernels, the
+README flow of the reference, and the host-sync-free dynamic mode.  Targets are
+the numpy oracle or dense torch autograd on the masked operands, as in the
+reference's test/unit/test_sparse_matmul.py:177-339 and test_sparse_softmax.py."""
+import numpy as np
+import pytest
+import torch
+
+import sparta_amd as sparta
+from oracle import ops
+from helpers import randn, rand, assert_close
+
+pytestmark = pytest.mark.gpu
+
+CFG32 = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32}
+
+
+def dense_linear(K, N, w, b, gpu, dtype=torch.float32):
+    lin = torch.nn.Linear(K, N, bias=b is not None, device=gpu, dtype=dtype)
+    with torch.no_grad():
+        lin.weight.copy_(w.to(gpu))
+        if b is not None:
+            lin.bias.copy_(b.to(gpu))
+    return lin
+
+
+def test_readme_flow_fp32(gpu):
+    """README case: 1024^3 fp32, 8x8-granular 90% weight mask, tune(rand), compare
+    with the masked dense linear (tolerance 1e-4)."""
+    M = K = N = 1024
+    x_np, x = rand((M, K), 1)
+    w_np, w = rand((N, K), 2)
+    b_np, b = rand((N,), 3)
+    mask_np = ops.block_mask((N, K), (8, 8), 0.9, seed=2022)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    lin = dense_linear(K, N, w * torch.from_numpy(mask_np), b, gpu)
+    op = sparta.nn.SparseLinear(lin, weight_mask=mask)
+    best = sparta.nn.tune(op, sample_inputs=[x.to(gpu)], max_trials=10, algo='rand')
+    assert set(best) == {'root'} and best['root']['forward:C']['_impl'] in ('sparta', 'openai')
+    assert op.ready and op.weight.dim() == 1
+    y = op(x.to(gpu))
+    want = ops.matmul_reference(x_np[None], w_np[None], b_np[None], mode='dsd', transpose_A=False,
+                                transpose_B=True, mask=mask_np, dtype=np.float64)[0]
+    g, wnt = y.detach().double().cpu().numpy(), want
+    assert np.all(np.abs(g - wnt) <= 1e-4 + 1e-4 * np.abs(wnt)), np.abs(g - wnt).max()
+
+
+@pytest.mark.parametrize('kind', ['input', 'weight', 'output'])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+def test_sparse_linear_forward_backward_and_mask_updates(kind, dtype, gpu, M=128, K=256, N=192):
+    x_np, x = randn((M, K), 4, dtype)
+    w_np, w = randn((N, K), 5, dtype, scale=0.5)
+    b_np, b = randn((N,), 6, dtype)
+    gy_np, gy = randn((M, N), 7, dtype)
+    shape = {'input': (M, K), 'weight': (N, K), 'output': (M, N)}[kind]
+    op = None
+    for seed in range(3):
+        mask_np = ops.block_mask(shape, (8, 8), 0.9, seed=seed)
+        mask = torch.from_numpy(mask_np).to(gpu)
+        # As in the reference, the weight is handed over already masked: values inside
+        # live blocks are used as they are.
+        w_in = w * torch.from_numpy(mask_np).to(dtype) if kind == 'weight' else w
+        if op is None:
+            op = sparta.nn.SparseLinear(dense_linear(K, N, w_in, b, gpu, dtype), **{f'{kind}_mask': mask})
+            cfg = {k: dict(CFG32) for k in ('forward:C', 'backward:A', 'backward:B')}
+            op.build(cfg, sample_inputs=[x.to(gpu)])
+        else:
+            op._raw_weight = w_in.to(gpu)
+            op.update_mask(**{f'{kind}_mask': mask})
+        # dense torch reference on the masked operands (autograd gives the gradients)
+        xr = (x.to(gpu).float() * (mask if kind == 'input' else 1)).requires_grad_(True)
+        wr = (w.to(gpu).float() * (mask if kind == 'weight' else 1)).requires_grad_(True)
+        br = b.to(gpu).float().requires_grad_(True)
+        block_mask = op.get_sparse_indexes({'input': 'A', 'weight': 'B', 'output': 'C'}[kind]).get_mask()
+        yr = torch.nn.functional.linear(xr, wr, br)
+        if kind == 'output':
+            yr = yr * block_mask
+        yr.backward(gy.to(gpu).float())
+
+        xs = (x.to(gpu) * (mask.to(dtype) if kind == 'input' else 1)).requires_grad_(True)
+        y = op(xs)
+        assert_close(y, yr.detach().double().cpu().numpy(), dtype, f'{kind} forward')
+        grad_in = gy.to(gpu) * (block_mask.to(dtype) if kind == 'output' else 1)
+        y.backward(grad_in)
+        gx_want = xr.grad * (block_mask if kind == 'input' else 1)  # masked inputs get no gradient
+        assert_close(xs.grad, gx_want.double().cpu().numpy(), dtype, f'{kind} grad_x')
+        gw = op.weight.grad
+        if kind == 'weight':
+            gw = op.get_sparse_indexes('B').inverse(gw)
+            gw_want = wr.grad * block_mask
+        else:
+            gw_want = wr.grad
+        assert_close(gw, gw_want.double().cpu().numpy(), dtype, f'{kind} grad_w')
+        assert_close(op.bias.grad, br.grad.double().cpu().numpy(), dtype, f'{kind} grad_b')
+        op.weight.grad = None
+        op.bias.grad = None
+
+
+@pytest.mark.parametrize('mode,tA,tB,compressed', [
+    ('sdd', False, False, True), ('dsd', True, True, True), ('dds', False, True, True),
+    ('dds', True, False, False), ('sdd', True, True, False),
+])
+def test_sparse_batch_matmul_operator(mode, tA, tB, compressed, gpu, Bt=3, M=128, K=192, N=64):
+    a_np, a = randn((Bt, K, M) if tA else (Bt, M, K), 8)
+    b_np, b = randn((Bt, N, K) if tB else (Bt, K, N), 9)
+    g_np, g = randn((Bt, M, N), 10)
+    port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
+    shape = {'A': a.shape[1:], 'B': b.shape[1:], 'C': (M, N)}[port]
+    mask_np = ops.block_mask(shape, (8, 8), 0.9, seed=11)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    op = sparta.nn.SparseBatchMatMul(**{f'{port}_mask': mask}, transpose_A=tA, transpose_B=tB,
+                                     compressed=compressed)
+    cfg = {k: dict(CFG32) for k in ('forward:C', 'backward:A', 'backward:B')}
+    op.build(cfg, sample_inputs=[a.to(gpu), b.to(gpu)])
+    idx = op.get_sparse_indexes(port)
+    block_mask = idx.get_mask()
+
+    ar = (a.to(gpu) * (mask if port == 'A' else 1)).requires_grad_(True)
+    br_ = (b.to(gpu) * (mask if port == 'B' else 1)).requires_grad_(True)
+    cr = torch.matmul(ar.transpose(1, 2) if tA else ar, br_.transpose(1, 2) if tB else br_)
+    if port == 'C':
+        cr = cr * block_mask
+    cr.backward(g.to(gpu))
+
+    a_in = (a.to(gpu) * (mask if port == 'A' else 1))
+    b_in = (b.to(gpu) * (mask if port == 'B' else 1))
+    if compressed and port == 'A':
+        a_in = idx.convert(a_in)
+    if compressed and port == 'B':
+        b_in = idx.convert(b_in)
+    a_in.requires_grad_(True)
+    b_in.requires_grad_(True)
+    c = op(a_in, b_in)
+    c_dense = idx.inverse(c) if (compressed and port == 'C') else c
+    assert_close(c_dense, cr.detach().double().cpu().numpy(), torch.float32, 'forward')
+    grad = g.to(gpu) * (block_mask if port == 'C' else 1)
+    c.backward(idx.convert(grad) if (compressed and port == 'C') else grad)
+    ga = idx.inverse(a_in.grad) if (compressed and port == 'A') else a_in.grad
+    gb = idx.inverse(b_in.grad) if (compressed and port == 'B') else b_in.grad
+    ga_want = ar.grad * (block_mask if port == 'A' else 1)
+    gb_want = br_.grad * (block_mask if port == 'B' else 1)
+    assert_close(ga, ga_want.double().cpu().numpy(), torch.float32, 'grad A')
+    assert_close(gb, gb_want.double().cpu().numpy(), torch.float32, 'grad B')
+
+
+@pytest.mark.parametrize('batch', [None, 4])
+@pytest.mark.parametrize('compressed', [False, True])
+def test_sparse_softmax_operator(batch, compressed, gpu, H=128, W=256):
+    shape = (H, W) if batch is None else (batch, H, W)
+    x_np, x = randn(shape, 12, scale=3.0)
+    g_np, g = randn(shape, 13)
+    mask_np = ops.block_mask((H, W), (8, 8), 0.9, seed=14)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    T = float(np.sqrt(W))
+    op = sparta.nn.SparseSoftmax(mask, temperature=T, compressed=compressed)
+    cfg = {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': 32, 'BLOCK_SIZE_W_VALUE': 32, 'ROW_TILE_VALUE': 4}
+    sample = x.to(gpu)
+    op.build({'forward:y': dict(cfg), 'backward:x': dict(cfg)}, sample_inputs=[sample])
+    idx = op.get_sparse_indexes('y')
+    xin = (x.to(gpu) * mask)
+    if compressed:
+        xin = idx.convert(xin)
+    xin.requires_grad_(True)
+    y = op(xin)
+    y_dense = idx.inverse(y) if compressed else y
+    want_y = ops.softmax_forward_reference(x_np, mask_np, T)
+    assert_close(y_dense.reshape(shape), want_y, torch.float32, 'softmax op forward')
+    gin = g.to(gpu) * mask
+    y.backward((idx.convert(gin) if compressed else gin).reshape(y.shape))
+    gx = idx.inverse(xin.grad) if compressed else xin.grad
+    want_gx = ops.softmax_backward_reference(g_np, y_dense.detach().double().cpu().numpy().reshape(shape), mask_np, T)
+    assert_close(gx.reshape(shape), want_gx, torch.float32, 'softmax op backward')
+
+
+def test_tune_grid_builds_best_config(gpu):
+    M, K, N = 256, 128, 128
+    x_np, x = randn((M, K), 15)
+    w_np, w = randn((N, K), 16)
+    mask_np = ops.block_mask((N, K), (16, 16), 0.8, seed=17)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    lin = dense_linear(K, N, w * torch.from_numpy(mask_np), None, gpu)
+    op = sparta.nn.SparseLinear(lin, weight_mask=mask)
+    best = sparta.nn.tune(op, sample_inputs=[x.to(gpu)], algo='grid', max_trials=12, tile_configs=False)
+    cfg = best['root']['forward:C']
+    assert {'_impl', 'BLOCK_SIZE_M_VALUE', 'BLOCK_SIZE_K_VALUE', 'BLOCK_SIZE_N_VALUE'} <= set(cfg)
+    want = ops.matmul_reference(x_np[None], w_np[None], None, mode='dsd', transpose_A=False, transpose_B=True,
+                                mask=mask_np, dtype=np.float64)[0]
+    assert_close(op(x.to(gpu)), want, torch.float32, 'tuned op')
+    # the same config builds a fresh operator through sparta.nn.build
+    op2 = sparta.nn.SparseLinear(dense_linear(K, N, w * torch.from_numpy(mask_np), None, gpu), weight_mask=mask)
+    sparta.nn.build(op2, [x.to(gpu)], best)
+    assert_close(op2(x.to(gpu)), want, torch.float32, 'built op')
+
+
+def test_tune_inside_a_combined_module(gpu):
+    class Net(torch.nn.Module):
+        def __init__(self, a, b):
+            super().__init__()
+            self.fc1, self.act, self.fc2 = a, torch.nn.ReLU(), b
+
+        def forward(self, x):
+            return self.fc2(self.act(self.fc1(x)))
+
+    torch.manual_seed(0)
+    l1 = torch.nn.Linear(128, 256, device=gpu)
+    l2 = torch.nn.Linear(256, 64, device=gpu)
+    m1 = sparta.testing.block_mask((256, 128), block=(32, 32), sparsity=0.5, device=gpu)
+    m2 = sparta.testing.block_mask((64, 256), block=(32, 32), sparsity=0.5, device=gpu)
+    with torch.no_grad():
+        l1.weight.mul_(m1)
+        l2.weight.mul_(m2)
+    x = torch.rand((64, 128), device=gpu)
+    want = l2(torch.relu(l1(x))).detach()
+    net = Net(sparta.nn.SparseLinear(l1, weight_mask=m1), sparta.nn.SparseLinear(l2, weight_mask=m2))
+    best = sparta.nn.tune(net, sample_inputs=[x], algo='rand', max_trials=4)
+    assert set(best) == {'root/fc1', 'root/fc2'}
+    torch.testing.assert_close(net(x), want, rtol=1e-4, atol=1e-4)
+
+
+def test_dynamic_mode_never_fetches_nnz(gpu):
+    """dynamic=True: index rebuild, weight re-compression and matmul are enqueued
+    without reading the live block count back to the host."""
+    M, K, N = 256, 256, 512
+    x_np, x = randn((M, K), 18, torch.float16)
+    w_np, w = randn((N, K), 19, torch.float16, scale=0.1)
+    op = None
+    for seed in range(4):
+        mask_np = ops.block_mask((N, K), (32, 64), 0.9, seed=seed)
+        mask = torch.from_numpy(mask_np).to(gpu)
+        if op is None:
+            op = sparta.nn.SparseLinear(dense_linear(K, N, w, None, gpu, torch.float16), weight_mask=mask,
+                                        dynamic=True)  # 32x64-granular mask: no masked value inside live blocks
+            op.build({'forward:C': {'_impl': 'openai', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 64,
+                                    'BLOCK_SIZE_N_VALUE': 32}}, sample_inputs=[x.to(gpu)])
+        else:
+            op.update_mask(weight_mask=mask)
+        with torch.no_grad():
+            y = op(x.to(gpu))
+        idx = op.get_sparse_indexes('B')
+        assert idx._block_nnz is None, 'the live block count was synchronised to the host'
+        assert op.weight.numel() == N * K  # stored at capacity
+        want = ops.matmul_reference(x_np[None], w_np[None], None, mode='dsd', transpose_A=False,
+                                    transpose_B=True, mask=mask_np, dtype=np.float64)[0]
+        assert_close(y, want, torch.float16, f'dynamic seed {seed}')
+        assert idx.block_nnz == int(mask_np.reshape(N // 32, 32, K // 64, 64).any(axis=(1, 3)).sum())
