@@ -105,16 +105,38 @@ def cpu_baseline(x, w, mask, nnz):
     }
 
 
+def measured_traffic_bytes():
+    """HBM bytes per launch of the matmul kernel from the committed rocprofv3 --pmc
+    summary (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size), or
+    None if that summary is absent."""
+    path = os.path.join(ROOT, 'profiles', 'spmm_panel_c2_traffic.json')
+    try:
+        with open(path) as f:
+            return json.load(f)['traffic_bytes_per_launch']
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run one plain 256 MiB device copy, so that a rocprofv3 --pmc run of this '
+                         'command shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic')
+    ap.add_argument('--config', default='headline',
+                    help="'headline' (default, the one JSON line the harness reads) or one of c1..c5 / all: "
+                         "secondary measurements of the other benchmark configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).', file=sys.stderr)
         sys.exit(2)
+    if args.config != 'headline':
+        import bench_configs
+        bench_configs.run(args.config, args.steps, args.warmup, time_graph, time_eager)
+        return
 
     import torch
     import sparta_amd as sparta
@@ -135,6 +157,13 @@ def main():
                             'BLOCK_SIZE_N_VALUE': 32}}
     op.build(config, sample_inputs=[x])
     nnz = op.get_sparse_indexes('B').block_nnz
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=device)
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)  # one elementwise kernel: 256 MiB read + 256 MiB written
+        torch.cuda.synchronize()
+        del src, dst
 
     with torch.no_grad():
         y = op(x)
@@ -183,7 +212,7 @@ def main():
             'peak': HBM_PEAK_GBS,
             'unit': 'GB/s',
             'frac': bytes_alg / sec / 1e9 / HBM_PEAK_GBS,
-            'traffic': None,
+            'traffic': measured_traffic_bytes(),
             'kernel': 'sparse-operand matmul (dsd)',
             'algorithmic_bytes': int(bytes_alg),
         },

@@ -1,0 +1,184 @@
+"""Secondary measurements for the benchmark configurations other than the headline
+line of bench.py: `python bench.py --config c1|c2|c3|c4|c5|all`.  Prints one JSON
+object per measurement.  Inputs are synthetic, generated on the CPU with fixed
+seeds and copied to the GPU."""
+import json
+import math
+
+import numpy as np
+
+
+def _grid_attention(n_blocks=64, seed=2022):
+    grid = np.zeros((n_blocks, n_blocks), dtype=np.uint8)
+    i, j = np.indices(grid.shape)
+    grid[(i - j >= 0) & (i - j <= 4)] = 1
+    grid |= (np.random.default_rng(seed).random(grid.shape) < 0.02).astype(np.uint8)
+    return grid
+
+
+def _emit(name, sec, flops=None, bytes_alg=None, extra=None):
+    out = {'config': name, 'ms': sec * 1e3}
+    if flops:
+        out['effective_tflops'] = flops / sec / 1e12
+        out['mfma_frac_fp16_peak'] = flops / sec / 1e12 / 2500.0
+    if bytes_alg:
+        out['algorithmic_gbs'] = bytes_alg / sec / 1e9
+        out['hbm_frac'] = bytes_alg / sec / 1e9 / 8000.0
+    out.update(extra or {})
+    print(json.dumps(out), flush=True)
+
+
+def run(which, steps, warmup, time_graph, time_eager):
+    import torch
+    import sparta_amd as sparta
+    from oracle import ops
+    from sparta_amd.specializer.kernels import SparTASparseMatMulKernel
+    from sparta_amd.tesa import get_bcs_function
+
+    dev = torch.device('cuda:0')
+    todo = ['c1', 'c2', 'c3', 'c4', 'c5'] if which == 'all' else [which]
+    steps = min(steps, 100)
+
+    def timed(fn):
+        try:
+            return time_graph(torch, fn, steps, warmup) / steps
+        except Exception:
+            return time_eager(torch, fn, steps, warmup) / steps
+
+    cfg32 = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32}
+    with torch.no_grad():
+        if 'c1' in todo:
+            g = torch.Generator().manual_seed(2022)
+            x = torch.rand((1024, 1024), generator=g).to(dev)
+            w = torch.rand((1024, 1024), generator=g)
+            b = torch.rand((1024,), generator=g)
+            mask_np = ops.block_mask((1024, 1024), (8, 8), 0.9, seed=2022)
+            lin = torch.nn.Linear(1024, 1024, device=dev)
+            lin.weight.copy_((w * torch.from_numpy(mask_np)).to(dev))
+            lin.bias.copy_(b.to(dev))
+            for blk in (16, 32):
+                op = sparta.nn.SparseLinear(lin, weight_mask=torch.from_numpy(mask_np).to(dev))
+                cfg = dict(cfg32, BLOCK_SIZE_K_VALUE=blk, BLOCK_SIZE_N_VALUE=blk)
+                op.build({'forward:C': cfg}, sample_inputs=[x])
+                nnz = op.get_sparse_indexes('B').block_nnz
+                sec = timed(lambda: op(x))
+                _emit(f'c1 SparseLinear fp32 1024^3 8x8@90%, {blk}x{blk} tiles', sec, flops=2.0 * 1024 * nnz * blk * blk,
+                      extra={'nnz_blocks': nnz, 'useful_gflop_8x8': 0.215})
+            sec = timed(lambda: lin(x))
+            _emit('c1 dense torch Linear fp32', sec, flops=2.0 * 1024 ** 3)
+
+        if 'c2' in todo:
+            M = K = N = 4096
+            g = torch.Generator().manual_seed(2022)
+            A = torch.randn((1, M, K), generator=g).half().to(dev)
+            B = torch.randn((1, N, K), generator=g).half().to(dev)
+            mask = torch.from_numpy(ops.block_mask((4096, 4096), (32, 32), 0.95, seed=2022)).to(dev)
+            for mode in ('sdd', 'dsd', 'dds'):
+                k = SparTASparseMatMulKernel(mode=mode, biased=False, transpose_A=False, transpose_B=True, compressed=True)
+                port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
+                k.ports[port].set_mask(mask)
+                k.set_shape(1, M, K, N)
+                k.compile(dict(cfg32))
+                idx = k.ports[port].indexes
+                args = {'sdd': (idx.convert(A), B), 'dsd': (A, idx.convert(B)), 'dds': (A, B)}[mode]
+                nnz = idx.block_nnz
+                sec = timed(lambda: k(*args))
+                _emit(f'c2 {mode} 4096^3 fp16 32x32@95%', sec, flops=nnz * 2.0 * 4096 * 1024,
+                      bytes_alg=2 * 4096 * 4096 * 2 + nnz * 2048, extra={'nnz_blocks': nnz})
+            sec = timed(lambda: torch.matmul(A[0], B[0].t()))
+            _emit('c2 dense torch.matmul fp16 4096^3', sec, flops=2.0 * 4096 ** 3)
+            for both in (False, True):
+                fn = get_bcs_function(32, 32, True, both)
+                sec = timed(lambda: fn.build_indexes(mask))
+                _emit(f"c2 index build 4096x4096 mask ({'BCSR+BCSC' if both else 'BCSR'})", sec, bytes_alg=4096 * 4096)
+
+        if 'c3' in todo:
+            BH, N, E, blk = 96, 4096, 64, 64
+            grid = _grid_attention()
+            mask = torch.from_numpy(np.kron(grid, np.ones((blk, blk), dtype=np.uint8))).to(dev)
+            g = torch.Generator().manual_seed(2022)
+            q, k_, v = (torch.randn((BH, N, E), generator=g).half().to(dev) for _ in range(3))
+            att = sparta.nn.SparseAttention(mask=mask)
+            mm = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 64, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 64}
+            att.build({'qk/forward:C': dict(mm),
+                       'sm/forward:y': {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': 64, 'BLOCK_SIZE_W_VALUE': 64, 'ROW_TILE_VALUE': 4},
+                       'out/forward:C': {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 64, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 32}},
+                      sample_inputs=[q, k_, v])
+            nnz = att._sparse_port.indexes.block_nnz
+            flops = 2 * nnz * 2.0 * blk * blk * E * BH
+            sec = timed(lambda: att(q, k_, v))
+            _emit('c3 fused sparse attention 96x4096x64 fp16, 64x64 blocks', sec, flops=flops,
+                  bytes_alg=4 * BH * N * E * 2, extra={'nnz_blocks': nnz})
+            att._fused = False
+            sec = timed(lambda: att(q, k_, v))
+            _emit('c3 three-operator pipeline (dds, softmax, sdd)', sec, flops=flops)
+            qq, kk, vv = (t.view(8, 12, N, E) for t in (q, k_, v))
+            sec = timed(lambda: torch.nn.functional.scaled_dot_product_attention(qq, kk, vv))
+            _emit('c3 dense torch SDPA (no mask)', sec, flops=4.0 * BH * N * N * E)
+
+        if 'c4' in todo:
+            T, D, F = 8192, 768, 3072
+            g = torch.Generator().manual_seed(2022)
+            x = torch.randn((T, D), generator=g).half().to(dev)
+            l1 = torch.nn.Linear(D, F, bias=False, device=dev, dtype=torch.float16)
+            l2 = torch.nn.Linear(F, D, bias=False, device=dev, dtype=torch.float16)
+            l1.weight.copy_((0.02 * torch.randn((F, D), generator=g)).half().to(dev))
+            l2.weight.copy_((0.02 * torch.randn((D, F), generator=g)).half().to(dev))
+
+            def topk_mask(shape, seed):
+                rows, cols = shape[0] // 32, shape[1] // 64
+                score = torch.randn((rows, cols), generator=torch.Generator().manual_seed(seed)).abs()
+                keep = math.ceil(0.1 * rows * cols)
+                thr = score.flatten().topk(keep).values[-1]
+                grid = (score >= thr).to(torch.uint8)
+                return grid.repeat_interleave(32, 0).repeat_interleave(64, 1).contiguous().to(dev)
+
+            masks1 = [topk_mask((F, D), s) for s in range(4)]
+            masks2 = [topk_mask((D, F), 100 + s) for s in range(4)]
+            cfg = {'forward:C': {'_impl': 'openai', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 32}}
+            for dynamic in (True, False):
+                op1 = sparta.nn.SparseLinear(l1, weight_mask=masks1[0], dynamic=dynamic)
+                op2 = sparta.nn.SparseLinear(l2, weight_mask=masks2[0], dynamic=dynamic)
+                op1.build(cfg, sample_inputs=[x])
+                op2.build(cfg, sample_inputs=[torch.relu(op1(x))])
+                m1 = masks1[1].clone()
+                m2 = masks2[1].clone()
+
+                def step():
+                    op1.update_mask(weight_mask=m1)
+                    op2.update_mask(weight_mask=m2)
+                    return op2(torch.relu(op1(x)))
+
+                if dynamic:
+                    sec = timed(step)  # no host sync inside: capturable
+                    tag = 'hip graph replay'
+                else:
+                    sec = time_eager(torch, step, steps, warmup) / steps
+                    tag = 'eager (one host sync per rebuild, as in the reference)'
+                _emit(f'c4 dynamic-mask FFN 8192x768->3072->768 fp16, rebuild timed, dynamic={dynamic}', sec,
+                      flops=2 * 2.0 * T * 115 * 32 * 64, extra={'timing': tag})
+            fwd_only = timed(lambda: op2(torch.relu(op1(x))))
+            _emit('c4 same FFN, masks fixed (no rebuild)', fwd_only, flops=2 * 2.0 * T * 115 * 32 * 64)
+            sec = timed(lambda: l2(torch.relu(l1(x))))
+            _emit('c4 dense torch FFN fp16', sec, flops=2 * 2.0 * T * D * F)
+
+        if 'c5' in todo:
+            n_tok, n_exp, K, N = 16384, 8, 1024, 4096
+            g = torch.Generator().manual_seed(2022)
+            mods = []
+            for _ in range(n_exp):
+                lin = torch.nn.Linear(K, N, bias=False, dtype=torch.float16, device=dev)
+                lin.weight.copy_((0.02 * torch.randn((N, K), generator=g)).half().to(dev))
+                mods.append(lin)
+            moe = sparta.nn.DynamicSparseMoE(mods)
+            p = np.arange(1, n_exp + 1, dtype=np.float64) ** -1.2
+            ids = torch.from_numpy(np.random.default_rng(2022).choice(n_exp, size=n_tok, p=p / p.sum()).astype(np.int32)).to(dev)
+            x = torch.randn((n_tok, K), generator=g).half().to(dev)
+            moe(x, ids)
+            sec = timed(lambda: moe(x, ids))
+            _emit('c5 MoE forward 16384 tok, 1024->4096, 8 experts Zipf(1.2), index rebuild included', sec,
+                  flops=2.0 * n_tok * K * N, bytes_alg=(n_tok * K + n_exp * K * N + n_tok * N) * 2,
+                  extra={'expert_counts': moe.expert_count.cpu().tolist()})
+            w0 = mods[0].weight
+            sec = timed(lambda: torch.matmul(x, w0.t()))
+            _emit('c5 dense torch.matmul with the same FLOPs (16384x1024x4096)', sec, flops=2.0 * n_tok * K * N)

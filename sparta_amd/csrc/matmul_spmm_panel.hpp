@@ -225,8 +225,8 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
                 const int chunk = c % CPR;
                 const int m = m0 + i * 16 + row;
                 if (c < 16 * CPR && m < p.Mc)
-                    *reinterpret_cast<u32x4*>(out + (int64_t)m * p.o_ld + (int64_t)j * BN + chunk * E16) =
-                        *reinterpret_cast<const u32x4*>(eT + row * LDE + chunk * E16);
+                    __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(eT + row * LDE + chunk * E16),
+                                                reinterpret_cast<u32x4*>(out + (int64_t)m * p.o_ld + (int64_t)j * BN + chunk * E16));
             }
         }
     } else {
@@ -256,8 +256,8 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
                 const int chunk = c % CPR;
                 const int m = m0 + chunk * E16;
                 if (m < p.Mc)
-                    *reinterpret_cast<u32x4*>(out + ((int64_t)j * BN + t * 16 + nrow) * p.o_ld + m) =
-                        *reinterpret_cast<const u32x4*>(eT + nrow * LDE + chunk * E16);
+                    __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(eT + nrow * LDE + chunk * E16),
+                                                reinterpret_cast<u32x4*>(out + ((int64_t)j * BN + t * 16 + nrow) * p.o_ld + m));
             }
         }
     }
