@@ -99,6 +99,13 @@ int spx_bcs_scatter(const void* sparse, void* dense, const void* idx, int idx_ki
                     int BH, int BW, int elem_bytes, int64_t sparse_batch_stride,
                     spx_stream_t stream);
 
+/* Launch order for matmuls that walk one row_ptr / col_ptr segment per workgroup:
+ * order[0..n) = the n segments sorted by descending length (longest first), so
+ * that the long segments start early and the short ones fill the tail.  Purely a
+ * scheduling hint (results do not depend on it); no counterpart in the reference,
+ * whose grids follow the natural order (matmul.py:143-149).  ptr int32 [n+1]. */
+int spx_bcs_schedule(const int32_t* ptr, int n, int32_t* order, spx_stream_t stream);
+
 /* Row / column sums of compressed values (fp32 accumulate), used for the bias
  * gradient of a compressed sparse-output matmul.  Replace
  * BCSFunctionContext.row_sum / col_sum (block_compressed.py:360-403) and
@@ -128,11 +135,12 @@ int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
  * ptr  row_ptr (BCSR) or col_ptr (BCSC); unused for DDS (may be NULL).
  * idx / idx_kind  see spx_idx_kind.  nnz_bound / nnz_dev as in spx_bcs_gather
  *                 (only DDS launches over blocks).
+ * sched     optional output of spx_bcs_schedule for `ptr` (NULL = natural order).
  * tile_cfg  index into the tile-config table of the op (0 = default).
  * ------------------------------------------------------------------------ */
 int spx_matmul(int mode, int dtype, int transA, int transB, int compressed,
                const void* A, const void* B, const void* bias, void* C,
-               const int32_t* ptr, const void* idx, int idx_kind,
+               const int32_t* ptr, const void* idx, int idx_kind, const int32_t* sched,
                int nnz_bound, const int32_t* nnz_dev, int64_t sparse_batch_stride,
                int batch, int M, int K, int N, int BM, int BK, int BN,
                int tile_cfg, spx_stream_t stream);

@@ -42,7 +42,8 @@ _SIGNATURES = {
     'spx_bcs_gather': (_I, [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
     'spx_bcs_scatter': (_I, [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
     'spx_bcs_sum': (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _L, _P]),
-    'spx_matmul': (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P, _L,
+    'spx_bcs_schedule': (_I, [_P, _I, _P, _P]),
+    'spx_matmul': (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _L,
                         _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     'spx_softmax_forward': (_I, [_I, _I, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _L, _I, _P]),
     'spx_softmax_backward': (_I, [_I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _L, _I, _P]),

@@ -345,6 +345,32 @@ __global__ __launch_bounds__(1024) void emit_fast_kernel(EmitParams p) {
     if (tid == 0) p.col_ptr[p.Cn] = nnz2;
 }
 
+// Launch order: segments of ptr sorted by descending length (bucketed at 255).
+__global__ __launch_bounds__(1024) void schedule_kernel(const int32_t* ptr, int n, int32_t* order) {
+    __shared__ int bins[256];
+    if (threadIdx.x < 256) bins[threadIdx.x] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const int c = ptr[i + 1] - ptr[i];
+        atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {  // exclusive scan of the 256 bins by one wavefront
+        int carry = 0;
+        for (int b0 = 0; b0 < 256; b0 += 64) {
+            const int v = bins[b0 + threadIdx.x];
+            const int inc = wave_inclusive_scan(v);
+            bins[b0 + threadIdx.x] = carry + inc - v;
+            carry += __shfl(inc, 63, 64);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const int c = ptr[i + 1] - ptr[i];
+        order[atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1)] = i;
+    }
+}
+
 struct IndexWorkspace {
     size_t live_off, wbits_off, wbase_off, cbase_off, total;
     int R, Cn, WPR, WPC;
@@ -450,5 +476,15 @@ extern "C" int spx_bcs_index(const uint8_t* mask, int H, int W, int BH, int BW,
     else
         hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
     SPX_LAUNCH_CHECK("emit_kernel");
+    return 0;
+}
+
+extern "C" int spx_bcs_schedule(const int32_t* ptr, int n, int32_t* order, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(n >= 0, SPX_E_SHAPE, "negative segment count");
+    if (n == 0) return 0;
+    SPX_REQUIRE(ptr && order, SPX_E_NULL, "ptr and order are required");
+    hipLaunchKernelGGL(schedule_kernel, dim3(1), dim3(1024), 0, reinterpret_cast<hipStream_t>(stream), ptr, n, order);
+    SPX_LAUNCH_CHECK("schedule_kernel");
     return 0;
 }

@@ -8,7 +8,7 @@ namespace spx {
 template <typename T>
 static int run_matmul(int mode, int transA, int transB, int compressed,
                       const void* A, const void* B, const void* bias, void* C,
-                      const int32_t* ptr, const void* idx, int idx_kind,
+                      const int32_t* ptr, const void* idx, int idx_kind, const int32_t* sched,
                       int nnz_bound, const int32_t* nnz_dev, int64_t sparse_batch_stride,
                       int batch, int M, int K, int N, int BM, int BK, int BN,
                       int tile_cfg, hipStream_t st) {
@@ -33,7 +33,7 @@ static int run_matmul(int mode, int transA, int transB, int compressed,
     }
 
     SpmmParams p;
-    p.bias = bias; p.out = C; p.ptr = ptr; p.idx = idx; p.idx_kind = idx_kind;
+    p.bias = bias; p.out = C; p.ptr = ptr; p.idx = idx; p.idx_kind = idx_kind; p.sched = sched;
     p.K = K; p.BK = BK; p.log_bk = ilog2(BK);
     p.compressed = compressed;
     p.o_batch = (int64_t)M * N;
@@ -71,7 +71,7 @@ static int run_matmul(int mode, int transA, int transB, int compressed,
 
 extern "C" int spx_matmul(int mode, int dtype, int transA, int transB, int compressed,
                           const void* A, const void* B, const void* bias, void* C,
-                          const int32_t* ptr, const void* idx, int idx_kind,
+                          const int32_t* ptr, const void* idx, int idx_kind, const int32_t* sched,
                           int nnz_bound, const int32_t* nnz_dev, int64_t sparse_batch_stride,
                           int batch, int M, int K, int N, int BM, int BK, int BN,
                           int tile_cfg, spx_stream_t stream) {
@@ -116,13 +116,13 @@ extern "C" int spx_matmul(int mode, int dtype, int transA, int transB, int compr
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     switch (dtype) {
         case SPX_F32:
-            return run_matmul<float>(mode, transA, transB, compressed, A, B, bias, C, ptr, idx, idx_kind, nnz_bound,
+            return run_matmul<float>(mode, transA, transB, compressed, A, B, bias, C, ptr, idx, idx_kind, sched, nnz_bound,
                                      nnz_dev, sparse_batch_stride, batch, M, K, N, BM, BK, BN, tile_cfg, st);
         case SPX_F16:
-            return run_matmul<_Float16>(mode, transA, transB, compressed, A, B, bias, C, ptr, idx, idx_kind, nnz_bound,
+            return run_matmul<_Float16>(mode, transA, transB, compressed, A, B, bias, C, ptr, idx, idx_kind, sched, nnz_bound,
                                         nnz_dev, sparse_batch_stride, batch, M, K, N, BM, BK, BN, tile_cfg, st);
         default:
-            return run_matmul<bf16_t>(mode, transA, transB, compressed, A, B, bias, C, ptr, idx, idx_kind, nnz_bound,
+            return run_matmul<bf16_t>(mode, transA, transB, compressed, A, B, bias, C, ptr, idx, idx_kind, sched, nnz_bound,
                                       nnz_dev, sparse_batch_stride, batch, M, K, N, BM, BK, BN, tile_cfg, st);
     }
 }

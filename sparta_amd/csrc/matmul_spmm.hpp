@@ -23,6 +23,7 @@ struct SpmmParams {
     void* out;
     const int32_t* ptr;
     const void* idx;
+    const int32_t* sched;  // optional launch order of the block-columns (longest first)
     int idx_kind;
     int Mc, K, Nc;       // canonical sizes (Mc: dense rows, Nc: sparse-side cols)
     int BK, log_bk;

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void spmm_direct_kernel(SpmmParams p, int n_mt
     const int xcd = L % kNumXcd;
     const int seq = L / kNumXcd;
     const int mt = (seq / nb) * kNumXcd + xcd;
-    const int j = seq % nb;
+    const int j = p.sched ? p.sched[seq % nb] : seq % nb;
     if (mt >= n_mtiles) return;
     const int64_t b = blockIdx.y;
 

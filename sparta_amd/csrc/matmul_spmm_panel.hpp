@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
     const int xcd = L % kPanelXcd;
     const int seq = L / kPanelXcd;
     const int mt = (seq / nb) * kPanelXcd + xcd;
-    const int j = seq % nb;
+    const int j = p.sched ? p.sched[seq % nb] : seq % nb;
     if (mt >= n_mtiles) return;
     const int64_t b = blockIdx.y;
 

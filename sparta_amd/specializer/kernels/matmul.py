@@ -144,6 +144,8 @@ class SparseMatMulKernel(KernelBase):
             ptr, idx = indexes.col_ptr, indexes._bcsc_buf
             idx_kind = _lib.IDX_BCSC_I64 if idx.dtype == torch.int64 else _lib.IDX_BCSC_I32
         dds = self._mode == 'dds'
+        sched = None if dds else indexes.launch_order('row' if self._bcs_mode == 'BCSR' else 'col')
+        sched_p = _lib.dev_ptr(sched)
         # Only a compressed operand / a sparse output need the live block count on the
         # host; a port in at-capacity mode leaves it on the device.
         at_capacity = self.ports[self._sparse_port].at_capacity
@@ -164,7 +166,7 @@ class SparseMatMulKernel(KernelBase):
         ptr_p, idx_p = _lib.dev_ptr(ptr), _lib.dev_ptr(idx)
 
         def matmul_func(A: torch.Tensor, B: torch.Tensor, bias: torch.Tensor = None,
-                        _keepalive=(indexes, ptr, idx)):
+                        _keepalive=(indexes, ptr, idx, sched)):
             assert A.dtype == B.dtype, f'operand dtypes differ: {A.dtype} vs {B.dtype}'
             C = alloc(C_shape, dtype=A.dtype, device=A.device)
             if bias is not None:
@@ -172,7 +174,7 @@ class SparseMatMulKernel(KernelBase):
             rc = lib.spx_matmul(
                 mode_code, _lib.dtype_code(A.dtype), tA, tB, compressed,
                 _lib.dev_ptr(A.contiguous()), _lib.dev_ptr(B.contiguous()), _lib.dev_ptr(bias), _lib.dev_ptr(C),
-                ptr_p, idx_p, idx_kind, nnz, nnz_dev_p, sparse_stride,
+                ptr_p, idx_p, idx_kind, sched_p, nnz, nnz_dev_p, sparse_stride,
                 batch_size, M, K, N, BM, BK, BN, tile_cfg, _lib.current_stream(A.device))
             _lib.check(rc, 'spx_matmul')
             return C

@@ -54,6 +54,21 @@ class BCSIndexes(TeSAIndexes):
     def nnz(self) -> np.int32:
         return np.int32(self.block_nnz)
 
+    # ---- scheduling hint -----------------------------------------------------------
+    def launch_order(self, by: str) -> torch.Tensor:
+        """int32 permutation of the block rows (by='row') or block columns (by='col'),
+        longest first; computed on the GPU once per index and cached."""
+        cache = self.__dict__.setdefault('_launch_order', {})
+        if by not in cache:
+            ptr = self.row_ptr if by == 'row' else self.col_ptr
+            n = ptr.numel() - 1
+            order = torch.empty((n,), dtype=torch.int32, device=ptr.device)
+            rc = _lib.load().spx_bcs_schedule(_lib.dev_ptr(ptr), n, _lib.dev_ptr(order),
+                                              _lib.current_stream(ptr.device))
+            _lib.check(rc, 'spx_bcs_schedule')
+            cache[by] = order
+        return cache[by]
+
     # ---- decoding --------------------------------------------------------------
     def _value_index(self) -> Tuple[torch.Tensor, int]:
         """(index buffer at capacity, idx_kind) that orders compressed values."""

@@ -46,15 +46,15 @@ def test_host_validation_without_gpu():
     rc = lib.spx_bcs_index(None, 64, 64, 32, 32, None, None, None, None, 0, None, 0, None, 0, None)
     assert rc == _lib.E_NULL
     one = ctypes.c_void_p(256)  # never dereferenced: validation fails first
-    rc = lib.spx_matmul(7, 0, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
+    rc = lib.spx_matmul(7, 0, 0, 1, 1, one, one, None, one, one, one, 0, None, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
     assert rc == _lib.E_CONFIG
-    rc = lib.spx_matmul(1, 9, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
+    rc = lib.spx_matmul(1, 9, 0, 1, 1, one, one, None, one, one, one, 0, None, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
     assert rc == _lib.E_DTYPE
-    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 64, 64, 32, 48, 32, 0, None)
+    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 0, None, 1, None, 0, 1, 64, 64, 64, 32, 48, 32, 0, None)
     assert rc == _lib.E_CONFIG
-    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 0, 1, None, 0, 1, 64, 80, 64, 32, 32, 32, 0, None)
+    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 0, None, 1, None, 0, 1, 64, 80, 64, 32, 32, 32, 0, None)
     assert rc == _lib.E_SHAPE and 'K=80' in _lib.last_error()
-    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 1, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
+    rc = lib.spx_matmul(1, 1, 0, 1, 1, one, one, None, one, one, one, 1, None, 1, None, 0, 1, 64, 64, 64, 32, 32, 32, 0, None)
     assert rc == _lib.E_CONFIG  # BCSC index handed to a BCSR-mode kernel
     rc = lib.spx_softmax_forward(1, 0, one, one, one, one, one, 1.0, 1, 64, 64, 5, 32, 0, 0, None)
     assert rc == _lib.E_CONFIG
