@@ -30,19 +30,23 @@ template <typename T> struct PanelMma {
     static constexpr int KC = 64 / (int)sizeof(T);  // k per step
 };
 
-template <typename T, int BN, int BK, int NST, bool SWAP>
+// SHW: the S (sparse) block of a step is loaded once per workgroup - each of the four
+// wavefronts fetches a quarter - into a double-buffered shared LDS tile, at the price
+// of one workgroup barrier per step; otherwise every wavefront loads it privately.
+template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW>
 __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mtiles) {
     typedef typename PanelMma<T>::M MMA;
     typedef typename MMA::frag Frag;
     constexpr int KC = PanelMma<T>::KC;
     constexpr int CH = BK / KC;          // steps per block
     constexpr int NT = BN / 16;
-    constexpr int WL = BN / 16;          // 16-byte loads per lane for the S rows
-    constexpr int ROWS = 64 + BN;        // LDS rows (64 bytes each) per wave
+    constexpr int WL = SHW ? 1 : BN / 16;  // 16-byte loads per lane for the S rows
+    constexpr int ROWS = SHW ? 80 : 64 + BN;  // private LDS rows (64 bytes each) per wave
+    constexpr int SH_BYTES = SHW ? 2 * BN * 64 : 0;  // shared, double-buffered S tile
     constexpr int E16 = 16 / (int)sizeof(T);
     static_assert(BK % KC == 0, "block depth must be a multiple of the step");
 
-    __shared__ __align__(16) char lds_all[4 * ROWS * 64];
+    __shared__ __align__(16) char lds_all[4 * ROWS * 64 + SH_BYTES];
 
     const int nb = p.Nc / BN;
     const int L = blockIdx.x;
@@ -58,8 +62,9 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
     const int r16 = lane & 15;
     const int g4 = lane >> 4;
     const int m0 = mt * 256 + wave * 64;
-    if (m0 >= p.Mc) return;  // waves are independent: leaving early is safe
+    if (!SHW && m0 >= p.Mc) return;  // independent waves may leave early; with a shared S tile all four stay
     char* lds = lds_all + wave * (ROWS * 64);
+    char* wsh = lds_all + 4 * ROWS * 64;
 
     const T* D = reinterpret_cast<const T*>(p.D) + b * p.d_batch;
     const T* S = reinterpret_cast<const T*>(p.S) + b * p.s_batch;
@@ -78,10 +83,18 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
         wofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
     }
     int sofs[WL];
+    // shared S tile: this wave stages chunks wave*BN .. wave*BN+BN-1 of the BN*4 chunks
+    const int sh_chunk = wave * BN + lane;
+    const int sh_row = sh_chunk >> 2, sh_chk = sh_chunk & 3;
+    const bool sh_active = lane < BN;
 #pragma unroll
     for (int q = 0; q < WL; ++q) {
-        const int row = 64 + q * 16 + lrow;
-        sofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
+        if constexpr (SHW) {
+            sofs[q] = sh_row * 64 + ((sh_chk ^ ((sh_row >> 2) & 3)) << 4);
+        } else {
+            const int row = 64 + q * 16 + lrow;
+            sofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
+        }
     }
     // fragment read offsets (row = tile*16 + r16, chunk g4)
     int aofs[4], bofs[NT];
@@ -92,7 +105,7 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
     }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int row = 64 + t * 16 + r16;
+        const int row = (SHW ? 0 : 64) + t * 16 + r16;
         bofs[t] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
     }
 
@@ -148,8 +161,13 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
                                       : S + (int64_t)j * BN * p.s_ld + koff_;                      \
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
             DREG[q] = *reinterpret_cast<const u32x4*>(dptr[q] + koff_);                            \
-        _Pragma("unroll") for (int q = 0; q < WL; ++q)                                             \
-            SREG[q] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)(q * 16 + lrow) * sld + lchk * E16); \
+        if constexpr (SHW) {                                                                       \
+            if (sh_active)                                                                         \
+                SREG[0] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)sh_row * sld + sh_chk * E16); \
+        } else {                                                                                   \
+            _Pragma("unroll") for (int q = 0; q < WL; ++q)                                         \
+                SREG[q] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)(q * 16 + lrow) * sld + lchk * E16); \
+        }                                                                                          \
     } while (0)
 
 // All global loads and LDS writes of the pipeline are issued unconditionally (steps
@@ -160,18 +178,24 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
     do {                                                                                           \
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
             *reinterpret_cast<u32x4*>(lds + wofs[q]) = DREG[q];                                    \
-        _Pragma("unroll") for (int q = 0; q < WL; ++q)                                             \
-            *reinterpret_cast<u32x4*>(lds + sofs[q]) = SREG[q];                                    \
+        char* sdst_ = SHW ? wsh + ((IT) & 1) * (BN * 64) : lds;                                     \
+        if constexpr (SHW) {                                                                       \
+            if (sh_active) *reinterpret_cast<u32x4*>(sdst_ + sofs[0]) = SREG[0];                   \
+        } else {                                                                                   \
+            _Pragma("unroll") for (int q = 0; q < WL; ++q)                                         \
+                *reinterpret_cast<u32x4*>(sdst_ + sofs[q]) = SREG[q];                              \
+        }                                                                                          \
         {                                                                                          \
             const int nx_ = (IT) + NST < n_it ? (IT) + NST : n_it - 1;                             \
             SPX_PANEL_ISSUE(nx_, DREG, SREG);                                                      \
         }                                                                                          \
+        if constexpr (SHW) __syncthreads(); /* the S tile of this step is complete */             \
         if ((IT) < n_it) {                                                                         \
             Frag af_[4], bf_[NT];                                                                  \
             _Pragma("unroll") for (int i = 0; i < 4; ++i)                                          \
                 af_[i] = *reinterpret_cast<const Frag*>(lds + aofs[i]);                            \
             _Pragma("unroll") for (int t = 0; t < NT; ++t)                                         \
-                bf_[t] = *reinterpret_cast<const Frag*>(lds + bofs[t]);                            \
+                bf_[t] = *reinterpret_cast<const Frag*>(sdst_ + bofs[t]);                          \
             _Pragma("unroll") for (int i = 0; i < 4; ++i)                                          \
                 _Pragma("unroll") for (int t = 0; t < NT; ++t)                                     \
                     acc[i][t] = SWAP ? MMA::mma(bf_[t], af_[i], acc[i][t])                         \
@@ -263,14 +287,14 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
     }
 }
 
-template <typename T, int BN, int BK, int NST, bool SWAP>
+template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW>
 static int launch_spmm_panel_inst(const SpmmParams& p, int batch, hipStream_t st) {
     const int n_mtiles = (p.Mc + 255) / 256;
     const int nb = p.Nc / BN;
     const int64_t groups = (n_mtiles + kPanelXcd - 1) / kPanelXcd;
     const int64_t nblocks = groups * kPanelXcd * nb;
     if (nblocks > 0x7fffffffLL) return fail(SPX_E_SHAPE, "problem too large for one launch");
-    hipLaunchKernelGGL((spmm_panel_kernel<T, BN, BK, NST, SWAP>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st,
+    hipLaunchKernelGGL((spmm_panel_kernel<T, BN, BK, NST, SWAP, SHW>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st,
                        p, n_mtiles);
     SPX_LAUNCH_CHECK("spmm_panel_kernel");
     return 0;
@@ -283,14 +307,14 @@ bool spmm_panel_supported(int BN, int BK) {
     return BK % kc == 0 && (BN == 16 || BN == 32 || BN == 64);
 }
 
-template <typename T, int NST>
+template <typename T, int NST, bool SHW>
 int launch_spmm_panel_impl(const SpmmParams& p, int BN, int batch, hipStream_t st) {
     const bool swap = p.out_ncontig != 0;
 #define SPX_PANEL_CASE(bn, bk)                                                                  \
     if (BN == bn && p.BK == bk) {                                                               \
         if constexpr (bk % (64 / (int)sizeof(T)) == 0) {                                        \
-            return swap ? launch_spmm_panel_inst<T, bn, bk, NST, true>(p, batch, st)            \
-                        : launch_spmm_panel_inst<T, bn, bk, NST, false>(p, batch, st);          \
+            return swap ? launch_spmm_panel_inst<T, bn, bk, NST, true, SHW>(p, batch, st)       \
+                        : launch_spmm_panel_inst<T, bn, bk, NST, false, SHW>(p, batch, st);     \
         }                                                                                       \
     }
     SPX_PANEL_CASE(16, 16) SPX_PANEL_CASE(16, 32) SPX_PANEL_CASE(16, 64)

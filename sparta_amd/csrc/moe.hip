@@ -325,6 +325,176 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
     }
 }
 
+// ---- gathered GEMM, 256 x 128 tiles with register prefetch ---------------------------
+// Same tile lookup and LDS layout as moe_gemm_kernel; the workgroup tile is 256 token
+// rows x 128 output columns (wave w owns rows 64w .. 64w+63), and the global loads of
+// K-stage s+1 are in flight (in registers) while stage s feeds the MFMAs, so HBM/L2
+// latency overlaps with the matrix cores.  Two workgroups fit on a CU.
+
+// TM x TN: workgroup tile; WGM: wavefronts along the token dimension (4 / WGM along the
+// output dimension); OCC: workgroups per CU the register budget is sized for.
+template <typename T, int TM, int TN, int WGM, int OCC>
+__global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
+    constexpr int MOE2_TM = TM, MOE2_TN = TN;
+    constexpr int WGN = 4 / WGM;
+    constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
+    constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
+    constexpr int A_LOADS = MOE2_TM * 8 / 256;  // 8
+    constexpr int B_LOADS = MOE2_TN * 8 / 256;  // 4
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ __align__(16) char As[MOE2_TM * 128];
+    __shared__ __align__(16) char Bs[MOE2_TN * 128];
+    __shared__ int s_expert, s_row0, s_rows;
+
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const int y = blockIdx.y;
+        int tiles_before = 0;
+        int found_e = -1, found_row0 = 0, found_rows = 0;
+        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
+            const int e = e0 + lane;
+            int cnt = 0, off = 0;
+            if (e < p.n_exp) {
+                off = p.expert_offset[e];
+                cnt = p.expert_offset[e + 1] - off;
+            }
+            const int tiles = (cnt + MOE2_TM - 1) / MOE2_TM;
+            const int inc = wave_inclusive_scan(tiles);
+            const int excl = tiles_before + inc - tiles;
+            const bool mine = y >= excl && y < excl + tiles;
+            const unsigned long long hit = __ballot(mine);
+            if (hit) {
+                const int src = __ffsll((long long)hit) - 1;
+                const int lt = y - __shfl(excl, src, 64);
+                found_e = e0 + src;
+                found_row0 = __shfl(off, src, 64) + lt * MOE2_TM;
+                found_rows = min(MOE2_TM, __shfl(cnt, src, 64) - lt * MOE2_TM);
+            }
+            tiles_before += __shfl(inc, 63, 64);
+        }
+        if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
+    }
+    __syncthreads();
+    const int expert = s_expert;
+    if (expert < 0) return;
+    const int row0 = s_row0, rows = s_rows;
+    const int n0 = blockIdx.x * MOE2_TN;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
+
+    const T* X = reinterpret_cast<const T*>(p.tokens);
+    const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
+
+    // staging map: chunk = tid % 8, rows tid / 8 + 32 q
+    const int chunk = threadIdx.x & 7;
+    const int srow = threadIdx.x >> 3;
+    const T* a_src[A_LOADS];
+    int a_dst[A_LOADS];
+#pragma unroll
+    for (int q = 0; q < A_LOADS; ++q) {
+        const int r = srow + 32 * q;
+        const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
+        a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
+        a_dst[q] = moe_lds_off<T>(r, chunk);
+    }
+    const T* b_src[B_LOADS];
+    int b_dst[B_LOADS];
+#pragma unroll
+    for (int q = 0; q < B_LOADS; ++q) {
+        const int r = srow + 32 * q;
+        const int n = n0 + r < p.N ? n0 + r : p.N - 1;
+        b_src[q] = W + (int64_t)n * p.K + chunk * VE;
+        b_dst[q] = moe_lds_off<T>(r, chunk);
+    }
+
+    f32x4 acc[MT][NTT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < NTT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 ra[A_LOADS], rb[B_LOADS];
+#pragma unroll
+    for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q]);
+#pragma unroll
+    for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q]);
+
+    for (int k0 = 0; k0 < p.K; k0 += KT) {
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) *reinterpret_cast<u32x4*>(As + a_dst[q]) = ra[q];
+#pragma unroll
+        for (int q = 0; q < B_LOADS; ++q) *reinterpret_cast<u32x4*>(Bs + b_dst[q]) = rb[q];
+        // next stage (the last iteration re-reads the final stage; it is not used)
+        const int kn = k0 + KT < p.K ? k0 + KT : k0;
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + kn);
+#pragma unroll
+        for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + kn);
+        __syncthreads();
+        if constexpr (HasMma32<T>::value) {
+#pragma unroll
+            for (int kc = 0; kc < KT; kc += 32) {
+                typename Mma32<T>::frag af[MT], bf[NTT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma32<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < NTT; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma32<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma32<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < KT; kc += 16) {
+                typename Mma16<T>::frag af[MT], bf[NTT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < NTT; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        }
+        __syncthreads();
+    }
+
+    T* out = reinterpret_cast<T*>(p.out);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int r = wrow + i * 16 + r16;
+        if (r >= rows) continue;
+        const int tok = p.token_perm[row0 + r];
+#pragma unroll
+        for (int t = 0; t < NTT; ++t) {
+            const int n = n0 + wcol + t * 16 + g4 * 4;
+            T vals[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
+            T* dst = out + (int64_t)tok * p.N + n;
+            if (n + 4 <= p.N) {
+                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+            } else {
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < p.N) dst[q] = vals[q];
+            }
+        }
+    }
+}
+
 static size_t moe_index_ws(int n_tok, int n_exp) {
     const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
     return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * n_exp * sizeof(int32_t), 256);
@@ -370,7 +540,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    (void)tile_cfg;
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -385,10 +555,32 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     p.expert_offset = expert_offset; p.token_perm = token_perm;
     p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
     p.w_kcontig = weight_layout == 1;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // tile_cfg 0: pick by size; 1: 128x128 tiles, no prefetch (any weight layout);
+    // 2: 256x128 tiles, 3: 128x128 tiles, both with the next K stage prefetched into
+    // registers (k-contiguous weights only).
+    if (tile_cfg == 0 && p.w_kcontig && n_tok >= 1024) tile_cfg = 3;
+    if (tile_cfg >= 2) {
+        SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
+        const int tm = tile_cfg == 2 ? 256 : 128;
+        const int tiles2 = (n_tok + tm - 1) / tm + n_exp;
+        SPX_REQUIRE(tiles2 <= 65535, SPX_E_SHAPE, "too many row tiles for one launch");
+        dim3 grid2((out_dim + 127) / 128, tiles2, 1);
+#define SPX_MOE2(T)                                                                                   \
+        if (tile_cfg == 2) hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 256, 128, 4, 2>), grid2, dim3(256), 0, st, p); \
+        else hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 128, 128, 2, 3>), grid2, dim3(256), 0, st, p);
+        switch (dtype) {
+            case SPX_F32: SPX_MOE2(float) break;
+            case SPX_F16: SPX_MOE2(_Float16) break;
+            default: SPX_MOE2(bf16_t) break;
+        }
+#undef SPX_MOE2
+        SPX_LAUNCH_CHECK("moe_gemm_kernel_v2");
+        return 0;
+    }
     const int max_tiles = (n_tok + MOE_TM - 1) / MOE_TM + n_exp;
     SPX_REQUIRE(max_tiles <= 65535, SPX_E_SHAPE, "too many row tiles for one launch");
     dim3 grid((out_dim + MOE_TN - 1) / MOE_TN, max_tiles, 1);
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const size_t smem = 2 * (size_t)MOE_TM * 128;
     switch (dtype) {
         case SPX_F32: hipLaunchKernelGGL(moe_gemm_kernel<float>, grid, dim3(256), smem, st, p); break;

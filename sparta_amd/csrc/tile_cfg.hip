@@ -17,6 +17,7 @@ static const spx_tile_cfg kSpmmCfgs[] = {
     {4, 256, 0, 4, 2, 16, 7, "direct-256"},
     {5, 256, 0, 4, 2, 16, 7, "panel-256x2"},
     {6, 256, 0, 4, 3, 16, 7, "panel-256x3"},
+    {7, 256, 0, 4, 2, 16, 7, "panel-256-sharedS"},
 };
 static const spx_tile_cfg kDdsCfgs[] = {
     {0, 0, 0, 4, 1, 16, 7, "block-per-workgroup"},
@@ -28,7 +29,10 @@ static const spx_tile_cfg kAttentionCfgs[] = {
     {0, 0, 0, 0, 1, 16, 6, "fused-online-softmax"},
 };
 static const spx_tile_cfg kMoeCfgs[] = {
-    {0, 128, 128, 4, 1, 0, 7, "gather-128x128"},
+    {0, 0, 0, 4, 0, 0, 7, "auto"},
+    {1, 128, 128, 4, 1, 0, 7, "gather-128x128"},
+    {2, 256, 128, 4, 2, 0, 7, "gather-256x128-prefetch"},
+    {3, 128, 128, 4, 2, 0, 7, "gather-128x128-prefetch"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {

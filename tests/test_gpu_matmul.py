@@ -98,7 +98,7 @@ def test_matmul_block_shapes(blocks, mode, gpu):
              batch=2, M=192, K=128, N=256, gran=(16, 16), sparsity=0.8, seed=k)
 
 
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize('mode', ['sdd', 'dsd'])
 @pytest.mark.parametrize('compressed', [False, True])
 @pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 64, 32)),
