@@ -177,6 +177,252 @@ __global__ __launch_bounds__(512) void attention_kernel(AttnParams p) {
     }
 }
 
+// ---- pipelined variant ------------------------------------------------------------------
+// Same mathematics and register layout as attention_kernel, rebuilt around the
+// instruction budget of a block step:
+//  * K and V tiles of the next live block travel global -> registers while the
+//    current one is consumed; with two LDS buffers a step needs one barrier.
+//  * V is staged untransposed ([key][e], 16-byte writes); the keys-contiguous
+//    operand of  O^T += V^T P^T  comes from the LDS transpose read of gfx950
+//    (ds_read_b64_tr_b16: in a 16-lane group, lane i supplies the address of 4
+//    consecutive e of key i/4, and lane j receives element j%4 of lanes
+//    j/4, 4+j/4, 8+j/4, 12+j/4: the 4 keys of column e0 + j).
+//  * P.V runs on 16x16x32 MFMAs: the 8 k-slots of a lane are the 4 keys it holds
+//    of key tile 2i followed by the 4 of key tile 2i+1.
+//  * exp2 with the scale folded into one fma; the row sums come from one more MFMA
+//    (an all-ones tile in place of V^T), and the running maximum is moved lazily.
+//  * workgroups are numbered so that all query blocks of one batch*head entry run
+//    on one XCD and find that entry's K and V in its L2.
+template <typename T> struct AttnPack;
+template <> struct AttnPack<_Float16> {
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    __device__ static f16x8 pack(f32x8 v) { return __builtin_convertvector(v, f16x8); }
+};
+template <> struct AttnPack<bf16_t> {
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    __device__ static bf16x8 pack(f32x8 v) { return __builtin_convertvector(v, bf16x8); }
+};
+
+template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(AttnParams p, int nbr, int batch) {
+    constexpr int NT = 64 * WAVES;
+    constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
+    constexpr int KP = E * 2 + 16;            // K row pitch in bytes
+    constexpr int VP = E * 2 + 32;            // V row pitch in bytes
+    constexpr int TILE = BW * (KP + VP);
+    constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
+    constexpr int VPR = E / 8;                // 16-byte vectors per tile row
+    constexpr int NV = BW * VPR / NT;         // vectors per thread and tile
+    constexpr int RSTEP = NT / VPR;           // tile rows between a thread's vectors
+    static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    // workgroup L runs on XCD L % 8: give each XCD whole batch*head entries
+    const int L = blockIdx.x;
+    const int slot = L >> 3;
+    const int64_t b = (slot / nbr) * 8 + (L & 7);
+    const int br = slot % nbr;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.Nt * E;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    const T* Vg = reinterpret_cast<const T*>(p.v) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    T* O = reinterpret_cast<T*>(p.out) + b * (int64_t)p.Nt * E;
+
+    const int qrow = br * (16 * WAVES) + wave * 16 + r16;
+    Frag qf[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) qf[c] = Mma32<T>::load(Q + (int64_t)qrow * E + c * 32 + g4 * 8);
+
+    f32x4 oacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -1e30f;
+    f32x4 lacc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float c2 = p.inv_t * 1.4426950408889634f;
+    constexpr float RESCALE_LOG2 = 6.f;
+    constexpr short ONE_BITS = sizeof(T) == 2 && Elem<T>::dtype == SPX_F16 ? (short)0x3c00 : (short)0x3f80;
+    const Frag ones = __builtin_bit_cast(Frag, s16x8{ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS});
+
+    // staging map: vector v = tid + i * NT of the (contiguous) tile is row v / VPR, chunk v % VPR
+    const int st_row = threadIdx.x / VPR, st_chunk = threadIdx.x % VPR;
+    const int k_dst = st_row * KP + st_chunk * 16;
+    const int v_dst = BW * KP + st_row * VP + st_chunk * 16;
+    // fragment bases
+    const int k_src = r16 * KP + g4 * 16;
+    const int v_src = BW * KP + (g4 * 4 + (r16 >> 2)) * VP + (r16 & 3) * 8;
+
+    const int e_begin = p.row_ptr[br];
+    const int e_end = p.row_ptr[br + 1];
+    u32x4 kr[NV], vr[NV];
+    int bc = 0;
+    if (e_begin < e_end) {
+        bc = p.bcsr_idx[e_begin] & 0xffff;
+        const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();  // the previous block's fragments are consumed
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + k_dst + i * RSTEP * KP) = kr[i];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
+        const int key0 = bc * BW;
+        // next live block (the last step re-reads its own block; the copy is not used)
+        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        {
+            const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+        }
+        unsigned live[KT];
+        if constexpr (HAS_MASK) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+                live[kt] = *reinterpret_cast<const uint32_t*>(p.mask + (int64_t)qrow * p.Ns + key0 + kt * 16 + g4 * 4);
+        }
+        __syncthreads();
+
+        // ---- S^T tiles: keys x this wave's 16 queries ------------------------------------
+        f32x4 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + c * 64);
+                s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
+            }
+        }
+        float tmax = -1e30f;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if constexpr (HAS_MASK) {
+                    if ((live[kt] >> (8 * q)) & 0xffu) tmax = fmaxf(tmax, s[kt][q]);
+                } else {
+                    tmax = fmaxf(tmax, s[kt][q]);
+                }
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        // The reference point m_run only has to keep exp2 in range, so it moves (and the
+        // accumulators are rescaled) only when some query's maximum outgrows it by more
+        // than 2^RESCALE_LOG2; numerator and denominator always share one reference.
+        if (__builtin_amdgcn_ballot_w64((tmax - m_run) * c2 > RESCALE_LOG2) != 0) {
+            const float m_new = fmaxf(m_run, tmax);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2);
+            m_run = m_new;
+            lacc *= alpha;
+#pragma unroll
+            for (int t = 0; t < ET; ++t) oacc[t] *= alpha;
+        }
+        const float mc = m_run * c2;
+        Frag pf[KT / 2];
+#pragma unroll
+        for (int kp = 0; kp < KT / 2; ++kp) {
+            f32x8 pv;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int kt = 2 * kp + (j >> 2), q = j & 3;
+                float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][q], c2, -mc));
+                if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
+                pv[j] = x;
+            }
+            pf[kp] = AttnPack<T>::pack(pv);
+            // row sums of the rounded probabilities: an all-ones tile in place of V^T
+            lacc = Mma32<T>::mma(ones, pf[kp], lacc);
+        }
+        // ---- O^T[e][query] += V^T P^T ------------------------------------------------------
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int kp = 0; kp < KT / 2; ++kp) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + v_src + (kp * 32) * VP + t * 32));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + v_src + (kp * 32 + 16) * VP + t * 32));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                oacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), pf[kp], oacc[t]);
+            }
+        }
+    }
+
+    // every accumulator row of lacc holds the row sum of query r16
+    const float l_run = lacc[0];
+    const float inv_l = l_run > 0.f ? 1.f / l_run : 0.f;
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T vals[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][q] * inv_l);
+        *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+    }
+}
+
+template <typename T, int BW, int E, int WAVES>
+static int launch_attention_v2_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr int TILE = BW * (E * 4 + 48);
+    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    const int nbr = p.Nt / p.BH;
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (p.mask) {
+        if (smem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_kernel_v2<T, BW, E, WAVES, true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_kernel_v2)");
+        }
+        hipLaunchKernelGGL((attention_kernel_v2<T, BW, E, WAVES, true>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    } else {
+        if (smem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_kernel_v2<T, BW, E, WAVES, false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_kernel_v2)");
+        }
+        hipLaunchKernelGGL((attention_kernel_v2<T, BW, E, WAVES, false>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    }
+    SPX_LAUNCH_CHECK("attention_kernel_v2");
+    return 0;
+}
+
+// The pipelined kernel covers query blocks of 32 / 64 / 128, key blocks of 32 / 64 / 128
+// and head dimensions 64 / 128 (except 128-query blocks with 32 x 64 key tiles).
+static bool attention_v2_supported(int BH, int BW, int E) {
+    return (BH == 32 || BH == 64 || BH == 128) && (BW == 32 || BW == 64 || BW == 128) && (E == 64 || E == 128) &&
+           BW * E / 8 >= BH * 4;  // at least one 16-byte vector of a tile per thread
+}
+
+template <typename T>
+static int launch_attention_v2(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTN2_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_v2_inst<T, bw, e, bh / 16>(p, batch, st);
+    SPX_ATTN2_CASE(32, 32, 64) SPX_ATTN2_CASE(32, 64, 64) SPX_ATTN2_CASE(32, 128, 64)
+    SPX_ATTN2_CASE(32, 32, 128) SPX_ATTN2_CASE(32, 64, 128) SPX_ATTN2_CASE(32, 128, 128)
+    SPX_ATTN2_CASE(64, 32, 64) SPX_ATTN2_CASE(64, 64, 64) SPX_ATTN2_CASE(64, 128, 64)
+    SPX_ATTN2_CASE(64, 32, 128) SPX_ATTN2_CASE(64, 64, 128) SPX_ATTN2_CASE(64, 128, 128)
+    SPX_ATTN2_CASE(128, 64, 64) SPX_ATTN2_CASE(128, 128, 64)
+    SPX_ATTN2_CASE(128, 32, 128) SPX_ATTN2_CASE(128, 64, 128) SPX_ATTN2_CASE(128, 128, 128)
+#undef SPX_ATTN2_CASE
+    return fail(SPX_E_CONFIG, "the pipelined attention kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
 template <typename T, int BW, int E>
 static int launch_attention_inst(const AttnParams& p, int batch, hipStream_t st) {
     const int waves = p.BH / 16;
@@ -211,7 +457,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
                                      int batch, int Nt, int Ns, int E, int BH, int BW,
                                      int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    (void)tile_cfg;
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 2, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
                 "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
     SPX_REQUIRE(q && k && v && out && row_ptr && bcsr_idx, SPX_E_NULL, "a required buffer is NULL");
@@ -229,6 +475,12 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel
+    if (tile_cfg == 0) tile_cfg = attention_v2_supported(BH, BW, E) ? 2 : 1;
+    if (tile_cfg == 2) {
+        if (dtype == SPX_F16) return launch_attention_v2<_Float16>(p, batch, BW, E, st);
+        return launch_attention_v2<bf16_t>(p, batch, BW, E, st);
+    }
     if (dtype == SPX_F16) return launch_attention<_Float16>(p, batch, BW, E, st);
     return launch_attention<bf16_t>(p, batch, BW, E, st);
 }

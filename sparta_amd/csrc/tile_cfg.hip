@@ -26,7 +26,9 @@ static const spx_tile_cfg kSoftmaxCfgs[] = {
     {0, 4, 0, 4, 0, 4, 7, "wave-per-row"},
 };
 static const spx_tile_cfg kAttentionCfgs[] = {
-    {0, 0, 0, 0, 1, 16, 6, "fused-online-softmax"},
+    {0, 0, 0, 0, 1, 16, 6, "auto"},
+    {1, 0, 0, 0, 1, 16, 6, "fused-online-softmax"},
+    {2, 0, 0, 0, 2, 32, 6, "fused-pipelined"},
 };
 static const spx_tile_cfg kMoeCfgs[] = {
     {0, 0, 0, 4, 0, 0, 7, "auto"},

@@ -126,3 +126,37 @@ def test_attention_long_sequence_layout(gpu):
     scores = scores.masked_fill(~live, float('-inf'))
     want = torch.softmax(scores, -1) @ v.float()
     torch.testing.assert_close(fused[:, :blk].float(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('element_mask', [False, True])
+@pytest.mark.parametrize('BH,BW,E', [(64, 64, 64), (32, 32, 64), (32, 128, 64), (64, 32, 128), (128, 64, 64),
+                                     (128, 128, 128), (64, 128, 128), (32, 64, 128), (128, 32, 128)])
+def test_attention_kernel_variants(dtype, element_mask, BH, BW, E, gpu):
+    """Both fused kernels through the C ABI (tile configs 1 and 2) on the same inputs:
+    each against the oracle, batch sizes that do not fill the eight-way workgroup
+    numbering, empty block rows and (element_mask) partly filled blocks."""
+    from sparta_amd import _lib
+    from sparta_amd.tesa import get_bcs_function
+    batch, Nt, Ns = 11, 2 * 128, 3 * 128
+    q_np, q = randn((batch, Nt, E), 21, dtype)
+    k_np, k = randn((batch, Ns, E), 22, dtype)
+    v_np, v = randn((batch, Ns, E), 23, dtype)
+    gran = (1, 1) if element_mask else (BH, BW)
+    mask_np = ops.block_mask((Nt, Ns), gran, 0.7 if element_mask else 0.5, seed=24)
+    mask_np[:BH] = 0  # an empty block row
+    mask = torch.from_numpy(mask_np).to(gpu)
+    indexes = get_bcs_function(BH, BW, True, False).build_indexes(mask)
+    q, k, v = q.to(gpu), k.to(gpu), v.to(gpu)
+    want = ops.attention_reference(q_np, k_np, v_np, mask_np)
+    lib = _lib.load()
+    for cfg in (1, 2):
+        out = torch.full_like(q, float('nan'))
+        rc = lib.spx_attention_forward(
+            _lib.dtype_code(dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
+            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf),
+            _lib.dev_ptr(indexes.raw_mask) if element_mask else None,
+            1.0 / float(np.sqrt(E)), batch, Nt, Ns, E, BH, BW, cfg, _lib.current_stream(q.device))
+        _lib.check(rc, 'spx_attention_forward')
+        assert_close(out, want, dtype, f'attention tile config {cfg} {dtype} {(BH, BW, E)} mask={element_mask}')
+        assert float(out[:, :BH].abs().max()) == 0.0
