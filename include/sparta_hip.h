@@ -132,7 +132,8 @@ int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
  * values with sparse_batch_stride elements between batches; otherwise it is
  * stored dense and the index only selects tiles (a dense DDS output must be
  * zero-filled by the caller; dead tiles are not written).
- * ptr  row_ptr (BCSR) or col_ptr (BCSC); unused for DDS (may be NULL).
+ * ptr  row_ptr (BCSR) or col_ptr (BCSC); optional for DDS: row_ptr lets the launch
+ *           group the live blocks of neighbouring block rows on one XCD (NULL = BCSR order).
  * idx / idx_kind  see spx_idx_kind.  nnz_bound / nnz_dev as in spx_bcs_gather
  *                 (only DDS launches over blocks).
  * sched     optional output of spx_bcs_schedule for `ptr` (NULL = natural order).

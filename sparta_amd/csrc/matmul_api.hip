@@ -17,6 +17,7 @@ static int run_matmul(int mode, int transA, int transB, int compressed,
         DdsParams p;
         p.A = A; p.B = B; p.bias = bias; p.C = C;
         p.idx = reinterpret_cast<const int32_t*>(idx);
+        p.row_ptr = ptr;
         p.nnz_dev = nnz_dev;
         p.M = M; p.K = K; p.N = N;
         p.a_kcontig = !transA; p.a_ld = transA ? M : K;

@@ -16,6 +16,7 @@ struct DdsParams {
     const void* bias;
     void* C;
     const int32_t* idx;      // BCSR_idx (row<<16 | col), one entry per live block
+    const int32_t* row_ptr;  // optional: enables the XCD-aware assignment of blocks to workgroups
     const int32_t* nnz_dev;  // optional: blocks >= *nnz_dev are skipped
     int M, K, N;
     int a_kcontig;           // A[m*a_ld + k] if set, else A[k*a_ld + m]
@@ -36,6 +37,41 @@ template <int MT, int NT> struct DdsWaveGrid {
     static constexpr int WTN = NT / WGN;
 };
 
+// Which live block a workgroup computes.  Workgroup L of a launch runs on XCD L % 8, each
+// with its own L2.  With row_ptr at hand, XCD x takes the blocks of the x-th band of
+// block rows (a contiguous range of the BCSR order) one after the other, so an A panel is
+// fetched into one L2 only and consecutive workgroups of an XCD reuse it; B panels are
+// shared by the blocks of the band.  Every XCD still gets the same number of workgroups:
+// those left over in short bands take the surplus of long ones.  Returns -1 for none.
+template <int BM>
+__device__ __forceinline__ int dds_block_of_workgroup(const DdsParams& p) {
+    const int L = blockIdx.x;
+    if (!p.row_ptr) return (p.nnz_dev && L >= p.nnz_dev[0]) ? -1 : L;
+    const int R = p.M / BM;
+    const int n_pos = gridDim.x;
+    const int x = L & 7, t = L >> 3;
+    int start[9];
+#pragma unroll
+    for (int y = 0; y <= 8; ++y) start[y] = p.row_ptr[(int)((int64_t)y * R / 8)];
+    if (t < start[x + 1] - start[x]) return start[x] + t;
+    int q = t - (start[x + 1] - start[x]);  // rank among the workgroups without a band block
+#pragma unroll
+    for (int y = 0; y < 8; ++y) {
+        const int idle = (n_pos - y + 7) / 8 - (start[y + 1] - start[y]);
+        if (y < x && idle > 0) q += idle;
+    }
+#pragma unroll
+    for (int y = 0; y < 8; ++y) {
+        const int slots = (n_pos - y + 7) / 8;
+        const int surplus = start[y + 1] - start[y] - slots;
+        if (surplus > 0) {
+            if (q < surplus) return start[y] + slots + q;
+            q -= surplus;
+        }
+    }
+    return -1;
+}
+
 template <typename T, int BM, int BN>
 __global__ __launch_bounds__(256) void dds_kernel(DdsParams p) {
     constexpr int MT = BM / 16, NT = BN / 16;
@@ -49,8 +85,8 @@ __global__ __launch_bounds__(256) void dds_kernel(DdsParams p) {
     T* As = reinterpret_cast<T*>(smem);
     T* Bs = As + BM * LDK;
 
-    const int i = blockIdx.x;
-    if (p.nnz_dev && i >= p.nnz_dev[0]) return;
+    const int i = dds_block_of_workgroup<BM>(p);
+    if (i < 0) return;
     const int code = p.idx[i];
     const int bi = (code >> 16) & 0xffff;
     const int bj = code & 0xffff;
@@ -155,6 +191,194 @@ __global__ __launch_bounds__(256) void dds_kernel(DdsParams p) {
     }
 }
 
+// ---- pipelined variant -----------------------------------------------------------------
+// A live block is a skinny product (BM x K by K x BN): almost no arithmetic per byte, so
+// the kernel is a data mover and wants many bytes in flight.  Each thread keeps NST
+// stages of its 16-byte pieces of the A and B panels in registers (issued NST steps
+// ahead, unconditionally, so the compiler keeps them asynchronous), drops the oldest
+// into one of two LDS buffers and the MFMAs read it after a single barrier per stage.
+// Needs k-contiguous A and B and K a multiple of the stage depth.
+template <int BM, int BN> struct DdsPipeCfg {
+    static constexpr int STAGE_BYTES = BM + BN == 128 ? 128 : 256;
+    static constexpr int NST = BM + BN <= 32 ? 4 : (BM + BN == 64 || BM + BN == 128 ? 3 : 2);
+};
+
+template <typename T, int BM, int BN, int NST>
+__global__ __launch_bounds__(256) void dds_pipe_kernel(DdsParams p) {
+    constexpr int MT = BM / 16, NT = BN / 16;
+    typedef DdsWaveGrid<MT, NT> G;
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int SB = DdsPipeCfg<BM, BN>::STAGE_BYTES;  // bytes of k per row and stage
+    constexpr int KT = SB / (int)sizeof(T);
+    constexpr int LDK = KT + VE;
+    constexpr int KW = KT / G::KS;
+    constexpr int CH = SB / 16;                     // 16-byte chunks per row and stage
+    constexpr int RP = 256 / CH;                    // panel rows per pass of the workgroup
+    constexpr int NV = (BM + BN) / RP;              // 16-byte vectors per thread and stage
+    static_assert((BM + BN) % RP == 0, "panel rows do not split over the workgroup");
+    constexpr int BUF = (BM + BN) * LDK * (int)sizeof(T);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) char smem[];
+
+    const int i = dds_block_of_workgroup<BM>(p);
+    if (i < 0) return;
+    const int code = p.idx[i];
+    const int bi = (code >> 16) & 0xffff;
+    const int bj = code & 0xffff;
+    const int64_t b = blockIdx.y;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15;
+    const int g4 = lane >> 4;
+    const int wt = wave % (G::WGM * G::WGN);
+    const int kpart = wave / (G::WGM * G::WGN);
+    const int wgm = wt / G::WGN;
+    const int wgn = wt % G::WGN;
+
+    const T* A = reinterpret_cast<const T*>(p.A) + b * p.a_batch;
+    const T* B = reinterpret_cast<const T*>(p.B) + b * p.b_batch;
+
+    // staging map: vector v = tid + 256 u covers panel row tid / CH + RP u, bytes (tid % CH) * 16;
+    // panel rows 0 .. BM-1 are A rows, the rest B rows
+    const int st_row = threadIdx.x / CH, st_chunk = threadIdx.x % CH;
+    const T* src[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int row = st_row + RP * u;
+        src[u] = (row < BM ? A + ((int64_t)bi * BM + row) * p.a_ld : B + ((int64_t)bj * BN + row - BM) * p.b_ld) + st_chunk * VE;
+    }
+    const int st_dst = (st_row * LDK + st_chunk * VE) * (int)sizeof(T);
+
+    f32x4 acc[G::WTM][G::WTN];
+#pragma unroll
+    for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+        for (int y = 0; y < G::WTN; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int n_st = p.K / KT;
+    // The workgroups of one XCD walk k in step (they share panels through its L2); the
+    // XCDs start at staggered depths, so that at any time the chip reads eight different
+    // column ranges of the row-major operands rather than one (rows are a power of two
+    // apart, which would keep hitting the same memory channels).
+    const int rot = (int)(((int64_t)(blockIdx.x & 7) * n_st) >> 3);
+    u32x4 ring[NST][NV];
+#pragma unroll
+    for (int r = 0; r < NST; ++r) {
+        int st0 = (r < n_st ? r : n_st - 1) + rot;
+        st0 = st0 >= n_st ? st0 - n_st : st0;
+        const int k0 = st0 * KT;
+#pragma unroll
+        for (int u = 0; u < NV; ++u) ring[r][u] = *reinterpret_cast<const u32x4*>(src[u] + k0);
+    }
+    for (int it = 0; it < n_st; it += NST) {
+#pragma unroll
+        for (int r = 0; r < NST; ++r) {
+            const int s = it + r;
+            char* buf = smem + (s & 1) * BUF;
+            if (s < n_st) {
+#pragma unroll
+                for (int u = 0; u < NV; ++u)
+                    *reinterpret_cast<u32x4*>(buf + st_dst + u * RP * LDK * (int)sizeof(T)) = ring[r][u];
+            }
+            {   // refill the slot NST stages ahead (clamped: the extra copies are never used)
+                int st1 = (s + NST < n_st ? s + NST : n_st - 1) + rot;
+                st1 = st1 >= n_st ? st1 - n_st : st1;
+                const int k0 = st1 * KT;
+#pragma unroll
+                for (int u = 0; u < NV; ++u) ring[r][u] = *reinterpret_cast<const u32x4*>(src[u] + k0);
+            }
+            if (s < n_st) {
+                __syncthreads();
+                const T* a_base = reinterpret_cast<const T*>(buf) + (wgm * G::WTM * 16 + r16) * LDK + kpart * KW;
+                const T* b_base = reinterpret_cast<const T*>(buf) + (BM + wgn * G::WTN * 16 + r16) * LDK + kpart * KW;
+                if constexpr (HasMma32<T>::value) {
+#pragma unroll
+                    for (int kc = 0; kc < KW; kc += 32) {
+                        typename Mma32<T>::frag af[G::WTM], bf[G::WTN];
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x) af[x] = Mma32<T>::load(a_base + x * 16 * LDK + kc + g4 * 8);
+#pragma unroll
+                        for (int y = 0; y < G::WTN; ++y) bf[y] = Mma32<T>::load(b_base + y * 16 * LDK + kc + g4 * 8);
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                            for (int y = 0; y < G::WTN; ++y) acc[x][y] = Mma32<T>::mma(af[x], bf[y], acc[x][y]);
+                    }
+                } else {
+#pragma unroll
+                    for (int kc = 0; kc < KW; kc += 16) {
+                        typename Mma16<T>::frag af[G::WTM], bf[G::WTN];
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x) af[x] = Mma16<T>::load(a_base + x * 16 * LDK + kc + g4 * 4);
+#pragma unroll
+                        for (int y = 0; y < G::WTN; ++y) bf[y] = Mma16<T>::load(b_base + y * 16 * LDK + kc + g4 * 4);
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                            for (int y = 0; y < G::WTN; ++y) acc[x][y] = Mma16<T>::mma(af[x], bf[y], acc[x][y]);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();  // all fragments are consumed before the buffers are reused
+
+    // ---- epilogue: partial sums -> LDS fp32 -> sum over k parts, bias, store ----
+    constexpr int LDE = BN + 1;
+    float* Ef = reinterpret_cast<float*>(smem);
+#pragma unroll
+    for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+        for (int y = 0; y < G::WTN; ++y)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int m = (wgm * G::WTM + x) * 16 + g4 * 4 + q;
+                const int n = (wgn * G::WTN + y) * 16 + r16;
+                Ef[(kpart * BM + m) * LDE + n] = acc[x][y][q];
+            }
+    __syncthreads();
+    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
+    T* C = reinterpret_cast<T*>(p.C) + b * p.c_batch;
+    for (int v = threadIdx.x; v < BM * BN; v += 256) {
+        const int m = v / BN;
+        const int n = v - m * BN;
+        float s = 0.f;
+#pragma unroll
+        for (int kp = 0; kp < G::KS; ++kp) s += Ef[(kp * BM + m) * LDE + n];
+        if (biasT) s += Elem<T>::to_float(biasT[bj * BN + n]);
+        const int64_t off = p.compressed ? (int64_t)i * (BM * BN) + v
+                                         : ((int64_t)bi * BM + m) * p.N + (int64_t)bj * BN + n;
+        C[off] = Elem<T>::from_float(s);
+    }
+}
+
+template <typename T, int BM, int BN>
+static int launch_dds_pipe_inst(const DdsParams& p, int nnz_bound, int batch, hipStream_t st) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int KT = DdsPipeCfg<BM, BN>::STAGE_BYTES / (int)sizeof(T);
+    constexpr int NST = DdsPipeCfg<BM, BN>::NST;
+    typedef DdsWaveGrid<BM / 16, BN / 16> G;
+    size_t smem = 2 * (size_t)(BM + BN) * (KT + VE) * sizeof(T);
+    size_t epi = (size_t)G::KS * BM * (BN + 1) * sizeof(float);
+    if (epi > smem) smem = epi;
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_pipe_kernel<T, BM, BN, NST>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(dds_pipe_kernel)");
+    }
+    hipLaunchKernelGGL((dds_pipe_kernel<T, BM, BN, NST>), dim3(nnz_bound, batch, 1), dim3(256), smem, st, p);
+    SPX_LAUNCH_CHECK("dds_pipe_kernel");
+    return 0;
+}
+
+// The pipelined kernel needs k-contiguous operands and K a multiple of its stage depth
+// (256 bytes of k per row; 128 bytes for 64 x 64 blocks).
+template <typename T>
+static bool dds_pipe_ok(const DdsParams& p, int BM, int BN) {
+    const int stage = (BM + BN == 128 ? 128 : 256) / (int)sizeof(T);
+    return p.a_kcontig && p.b_kcontig && p.K % stage == 0;
+}
+
 template <typename T, int BM, int BN>
 static int launch_dds_inst(const DdsParams& p, int nnz_bound, int batch, hipStream_t st) {
     constexpr int VE = 16 / (int)sizeof(T);
@@ -168,10 +392,18 @@ static int launch_dds_inst(const DdsParams& p, int nnz_bound, int batch, hipStre
     return 0;
 }
 
+// tile_cfg: 0 = the pipelined kernel where it applies; 1 = one LDS buffer, no prefetch;
+//           2 = pipelined (register ring + two LDS buffers).
 template <typename T>
-int launch_dds_impl(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, hipStream_t st) {
+int launch_dds_impl(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, int tile_cfg, hipStream_t st) {
+    if (tile_cfg < 0 || tile_cfg > 2) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    if (tile_cfg == 0) tile_cfg = dds_pipe_ok<T>(p, BM, BN) ? 2 : 1;
+    if (tile_cfg == 2 && !dds_pipe_ok<T>(p, BM, BN))
+        return fail(SPX_E_CONFIG, "tile config 2 needs k-contiguous operands and K a multiple of the stage depth");
 #define SPX_DDS_CASE(bm, bn) \
-    if (BM == bm && BN == bn) return launch_dds_inst<T, bm, bn>(p, nnz_bound, batch, st);
+    if (BM == bm && BN == bn) \
+        return tile_cfg == 2 ? launch_dds_pipe_inst<T, bm, bn>(p, nnz_bound, batch, st) \
+                             : launch_dds_inst<T, bm, bn>(p, nnz_bound, batch, st);
     SPX_DDS_CASE(16, 16) SPX_DDS_CASE(16, 32) SPX_DDS_CASE(16, 64)
     SPX_DDS_CASE(32, 16) SPX_DDS_CASE(32, 32) SPX_DDS_CASE(32, 64)
     SPX_DDS_CASE(64, 16) SPX_DDS_CASE(64, 32) SPX_DDS_CASE(64, 64)

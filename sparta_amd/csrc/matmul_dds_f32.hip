@@ -3,7 +3,6 @@
 namespace spx {
 template <>
 int launch_dds<float>(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, int tile_cfg, hipStream_t st) {
-    (void)tile_cfg;
-    return launch_dds_impl<float>(p, BM, BN, nnz_bound, batch, st);
+    return launch_dds_impl<float>(p, BM, BN, nnz_bound, batch, tile_cfg, st);
 }
 }  // namespace spx

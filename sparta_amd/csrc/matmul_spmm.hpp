@@ -221,9 +221,13 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
     const bool panel_ok = kcontig && (p.BK * (int)sizeof(T)) % 64 == 0;
     if (tile_cfg < 0 || tile_cfg > 7) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg == 0) {
-        if (panel_ok && p.Mc >= 512) tile_cfg = p.Mc >= 1024 ? 7 : 5;
-        else if (kcontig) tile_cfg = p.Mc >= 1024 ? 4 : 3;
-        else tile_cfg = p.Mc >= 1024 ? 2 : 1;
+        // 256-row tiles only when they still give every CU a few workgroups; small
+        // problems are latency-bound and want more, shorter workgroups.
+        const int64_t big_tiles = (int64_t)((p.Mc + 255) / 256) * (p.Nc / BN) * batch;
+        const bool fill = big_tiles >= 1024;
+        if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
+        else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
+        else tile_cfg = p.Mc >= 1024 && fill ? 2 : 1;
     }
     if (tile_cfg >= 5) {
         if (!panel_ok) return fail(SPX_E_CONFIG, "tile config %d needs k-contiguous operands and 64-byte block rows", tile_cfg);

@@ -20,7 +20,9 @@ static const spx_tile_cfg kSpmmCfgs[] = {
     {7, 256, 0, 4, 2, 16, 7, "panel-256-sharedS"},
 };
 static const spx_tile_cfg kDdsCfgs[] = {
-    {0, 0, 0, 4, 1, 16, 7, "block-per-workgroup"},
+    {0, 0, 0, 4, 1, 16, 7, "auto"},
+    {1, 0, 0, 4, 1, 16, 7, "block-per-workgroup"},
+    {2, 0, 0, 4, 3, 16, 7, "block-per-workgroup-pipelined"},
 };
 static const spx_tile_cfg kSoftmaxCfgs[] = {
     {0, 4, 0, 4, 0, 4, 7, "wave-per-row"},

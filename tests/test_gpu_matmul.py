@@ -112,6 +112,19 @@ def test_matmul_tile_configs(tile_cfg, mode, compressed, dtype, blocks, gpu):
              sparsity=0.7, seed=11, tile_cfg=tile_cfg)
 
 
+@pytest.mark.parametrize('tile_cfg', [1, 2])
+@pytest.mark.parametrize('K', [128, 640])
+@pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 32, 64)),
+                                          (torch.float32, (16, 32, 16)), (torch.float16, (16, 32, 64)),
+                                          (torch.float32, (64, 32, 32)), (torch.float16, (64, 32, 16)),
+                                          (torch.float32, (32, 32, 32))])
+def test_matmul_dds_tile_configs(tile_cfg, K, dtype, blocks, gpu):
+    """Both sparse-output kernels (single-buffer and pipelined) on k-contiguous operands:
+    stage counts below, equal to and above the depth of the register ring."""
+    run_case(gpu, 'dds', False, True, True, True, dtype, blocks, batch=2, M=192, K=K, N=256,
+             gran=(16, 16), sparsity=0.7, seed=5, tile_cfg=tile_cfg)
+
+
 def test_matmul_all_ones_mask_is_plain_gemm(gpu):
     a_np, a = randn((1, 256, 128), 1, torch.float32)
     b_np, b = randn((1, 64, 128), 2, torch.float32)
