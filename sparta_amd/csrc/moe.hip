@@ -436,6 +436,7 @@ __global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
         for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + kn);
 #pragma unroll
         for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + kn);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the MFMAs that hide them
         __syncthreads();
         if constexpr (HasMma32<T>::value) {
 #pragma unroll
@@ -495,6 +496,209 @@ __global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
     }
 }
 
+// ---- gathered GEMM, 256 x 256 tiles, eight wavefronts, two LDS buffers ------------------
+// On gfx950 a 64 x 64 wavefront tile reads as many LDS bytes per MFMA as the LDS can
+// deliver, and a 128 x 128 workgroup tile pulls twice the operand bytes through L1 that
+// a 256 x 256 one does.  Here each wavefront owns 128 x 64 outputs (12 fragment reads per
+// 32 MFMAs), K-stage s+1 sits in the second LDS buffer and stage s+2 is in flight in
+// registers while stage s feeds the matrix cores; one barrier per stage.
+template <typename T, int TM, int TN, int WAVES, int WGM>
+__global__ __launch_bounds__(64 * WAVES, 1) void moe_gemm_kernel_v4(MoeParams p) {
+    constexpr int NTH = 64 * WAVES;
+    constexpr int WGN = WAVES / WGM;
+    constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
+    constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
+    constexpr int A_LOADS = TM * 8 / NTH;
+    constexpr int B_LOADS = TN * 8 / NTH;
+    constexpr int RSTEP = NTH / 8;        // tile rows between a thread's vectors (a multiple of 8)
+    constexpr int A_BYTES = TM * 128;
+    constexpr int BUF = (TM + TN) * 128;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) char smem[];
+    __shared__ int s_expert, s_row0, s_rows;
+
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const int y = blockIdx.y;
+        int tiles_before = 0;
+        int found_e = -1, found_row0 = 0, found_rows = 0;
+        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
+            const int e = e0 + lane;
+            int cnt = 0, off = 0;
+            if (e < p.n_exp) {
+                off = p.expert_offset[e];
+                cnt = p.expert_offset[e + 1] - off;
+            }
+            const int tiles = (cnt + TM - 1) / TM;
+            const int inc = wave_inclusive_scan(tiles);
+            const int excl = tiles_before + inc - tiles;
+            const bool mine = y >= excl && y < excl + tiles;
+            const unsigned long long hit = __ballot(mine);
+            if (hit) {
+                const int src = __ffsll((long long)hit) - 1;
+                const int lt = y - __shfl(excl, src, 64);
+                found_e = e0 + src;
+                found_row0 = __shfl(off, src, 64) + lt * TM;
+                found_rows = min(TM, __shfl(cnt, src, 64) - lt * TM);
+            }
+            tiles_before += __shfl(inc, 63, 64);
+        }
+        if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
+    }
+    __syncthreads();
+    const int expert = s_expert;
+    if (expert < 0) return;
+    const int row0 = s_row0, rows = s_rows;
+    const int n0 = blockIdx.x * TN;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
+
+    const T* X = reinterpret_cast<const T*>(p.tokens);
+    const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
+
+    // staging map: chunk = tid % 8, rows tid / 8 + RSTEP q (the swizzle only sees row % 8)
+    const int chunk = threadIdx.x & 7;
+    const int srow = threadIdx.x >> 3;
+    const int st_dst = moe_lds_off<T>(srow, chunk);
+    const T* a_src[A_LOADS];
+#pragma unroll
+    for (int q = 0; q < A_LOADS; ++q) {
+        const int r = srow + RSTEP * q;
+        const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
+        a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
+    }
+    const T* b_src[B_LOADS];
+#pragma unroll
+    for (int q = 0; q < B_LOADS; ++q) {
+        const int r = srow + RSTEP * q;
+        const int n = n0 + r < p.N ? n0 + r : p.N - 1;
+        b_src[q] = W + (int64_t)n * p.K + chunk * VE;
+    }
+
+    f32x4 acc[MT][NTT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < NTT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int n_st = p.K / KT;
+    u32x4 ra[A_LOADS], rb[B_LOADS];
+#pragma unroll
+    for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q]);
+#pragma unroll
+    for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q]);
+#pragma unroll
+    for (int q = 0; q < A_LOADS; ++q) *reinterpret_cast<u32x4*>(smem + st_dst + q * RSTEP * 128) = ra[q];
+#pragma unroll
+    for (int q = 0; q < B_LOADS; ++q) *reinterpret_cast<u32x4*>(smem + A_BYTES + st_dst + q * RSTEP * 128) = rb[q];
+    {
+        const int k1 = (1 < n_st ? 1 : 0) * KT;
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + k1);
+#pragma unroll
+        for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + k1);
+    }
+    __syncthreads();
+
+    for (int s = 0; s < n_st; ++s) {
+        const char* cur = smem + (s & 1) * BUF;
+        char* nxt = smem + ((s + 1) & 1) * BUF;
+        if (s + 1 < n_st) {
+#pragma unroll
+            for (int q = 0; q < A_LOADS; ++q) *reinterpret_cast<u32x4*>(nxt + st_dst + q * RSTEP * 128) = ra[q];
+#pragma unroll
+            for (int q = 0; q < B_LOADS; ++q) *reinterpret_cast<u32x4*>(nxt + A_BYTES + st_dst + q * RSTEP * 128) = rb[q];
+        }
+        {   // stage s + 2 (clamped: the extra copies are never used)
+            const int k2 = (s + 2 < n_st ? s + 2 : n_st - 1) * KT;
+#pragma unroll
+            for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + k2);
+#pragma unroll
+            for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + k2);
+        }
+        // keep the loads ahead of the MFMAs: sunk below them they would be waited for at
+        // the top of the next stage with nothing left to hide their latency
+        __builtin_amdgcn_sched_barrier(0);
+        const char* As = cur;
+        const char* Bs = cur + A_BYTES;
+        if constexpr (HasMma32<T>::value) {
+#pragma unroll
+            for (int kc = 0; kc < KT; kc += 32) {
+                typename Mma32<T>::frag af[MT], bf[NTT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma32<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < NTT; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma32<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma32<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < KT; kc += 16) {
+                typename Mma16<T>::frag af[MT], bf[NTT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < NTT; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        }
+        __syncthreads();
+    }
+
+    T* out = reinterpret_cast<T*>(p.out);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int r = wrow + i * 16 + r16;
+        if (r >= rows) continue;
+        const int tok = p.token_perm[row0 + r];
+#pragma unroll
+        for (int t = 0; t < NTT; ++t) {
+            const int n = n0 + wcol + t * 16 + g4 * 4;
+            T vals[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
+            T* dst = out + (int64_t)tok * p.N + n;
+            if (n + 4 <= p.N) {
+                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+            } else {
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < p.N) dst[q] = vals[q];
+            }
+        }
+    }
+}
+
+template <typename T>
+static int launch_moe_v4(const MoeParams& p, hipStream_t st) {
+    constexpr int TM = 256, TN = 256;
+    const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp;
+    if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
+    const int smem = 2 * (TM + TN) * 128;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel_v4<T, TM, TN, 8, 2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_kernel_v4)");
+    hipLaunchKernelGGL((moe_gemm_kernel_v4<T, TM, TN, 8, 2>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(512), smem, st, p);
+    SPX_LAUNCH_CHECK("moe_gemm_kernel_v4");
+    return 0;
+}
+
 static size_t moe_index_ws(int n_tok, int n_exp) {
     const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
     return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * n_exp * sizeof(int32_t), 256);
@@ -540,7 +744,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -556,10 +760,19 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
     p.w_kcontig = weight_layout == 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    // tile_cfg 0: pick by size; 1: 128x128 tiles, no prefetch (any weight layout);
+    // tile_cfg 0: default (1); 1: 128x128 tiles, no prefetch (any weight layout);
     // 2: 256x128 tiles, 3: 128x128 tiles, both with the next K stage prefetched into
-    // registers (k-contiguous weights only).
-    if (tile_cfg == 0 && p.w_kcontig && n_tok >= 1024) tile_cfg = 3;
+    // registers; 4: 256x256 tiles with two LDS buffers (2..4: k-contiguous weights only).
+    if (tile_cfg == 0) tile_cfg = 1;  // measured best on the benchmark shapes; the others stay selectable
+    if (tile_cfg == 4) {
+        // 256x256 tiles, eight wavefronts, two LDS buffers (k-contiguous weights only)
+        SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
+        switch (dtype) {
+            case SPX_F32: return launch_moe_v4<float>(p, st);
+            case SPX_F16: return launch_moe_v4<_Float16>(p, st);
+            default: return launch_moe_v4<bf16_t>(p, st);
+        }
+    }
     if (tile_cfg >= 2) {
         SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
         const int tm = tile_cfg == 2 ? 256 : 128;

@@ -37,6 +37,7 @@ static const spx_tile_cfg kMoeCfgs[] = {
     {1, 128, 128, 4, 1, 0, 7, "gather-128x128"},
     {2, 256, 128, 4, 2, 0, 7, "gather-256x128-prefetch"},
     {3, 128, 128, 4, 2, 0, 7, "gather-128x128-prefetch"},
+    {4, 256, 256, 8, 3, 0, 7, "gather-256x256-two-buffers"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {

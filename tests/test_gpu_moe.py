@@ -112,3 +112,27 @@ def test_moe_weight_layouts_agree(gpu):
                                      _lib.current_stream(gpu))
     _lib.check(rc, 'spx_moe_forward')
     assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4])
+@pytest.mark.parametrize('dtype,n_tok,in_dims,out_dims', [
+    (torch.float16, 3000, 256, 520), (torch.bfloat16, 1500, 128, 256), (torch.float32, 700, 96, 136),
+    (torch.float16, 5, 64, 64)])
+def test_moe_tile_configs(tile_cfg, dtype, n_tok, in_dims, out_dims, gpu):
+    """Every gathered-GEMM variant through the C ABI on the same routing (one stage, two
+    stages and more; ragged last tiles in both directions; an empty expert)."""
+    from sparta_amd import _lib
+    n_exp = 5
+    moe, w = make_moe(n_exp, in_dims, out_dims, dtype, gpu)
+    ids_np = np.random.default_rng(n_tok).choice([0, 1, 2, 4], size=n_tok, p=[0.6, 0.2, 0.15, 0.05]).astype(np.int32)
+    x = torch.from_numpy(np.random.default_rng(1).random((n_tok, in_dims), dtype=np.float32)).to(dtype)
+    xg = x.to(gpu)
+    moe(xg, torch.from_numpy(ids_np).to(gpu))  # builds the index and the [E, out, in] weight copy
+    out = torch.full((n_tok, out_dims), float('nan'), dtype=dtype, device=gpu)
+    rc = _lib.load().spx_moe_forward(_lib.dtype_code(dtype), _lib.dev_ptr(xg), _lib.dev_ptr(moe._weight_nk), 1,
+                                     _lib.dev_ptr(out), _lib.dev_ptr(moe.expert_offset),
+                                     _lib.dev_ptr(moe.sparse_index), n_tok, in_dims, out_dims, n_exp, tile_cfg,
+                                     _lib.current_stream(gpu))
+    _lib.check(rc, 'spx_moe_forward')
+    want = ops.moe_reference(x.to(torch.float64).numpy(), w, ids_np)
+    assert_close(out, want, dtype, f'moe tile config {tile_cfg} {dtype}')
