@@ -182,6 +182,8 @@ __global__ __launch_bounds__(512) void attention_kernel(AttnParams p) {
 // instruction budget of a block step:
 //  * K and V tiles of the next live block travel global -> registers while the
 //    current one is consumed; with two LDS buffers a step needs one barrier.
+//  * K is staged with its 16-byte chunks XOR-swizzled by the row (padding the pitch
+//    instead halves the rate of 16-byte LDS reads on this chip).
 //  * V is staged untransposed ([key][e], 16-byte writes); the keys-contiguous
 //    operand of  O^T += V^T P^T  comes from the LDS transpose read of gfx950
 //    (ds_read_b64_tr_b16: in a 16-lane group, lane i supplies the address of 4
@@ -207,7 +209,7 @@ template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(AttnParams p, int nbr, int batch) {
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
-    constexpr int KP = E * 2 + 16;            // K row pitch in bytes
+    constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
     constexpr int VP = E * 2 + 32;            // V row pitch in bytes
     constexpr int TILE = BW * (KP + VP);
     constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
@@ -255,10 +257,11 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
 
     // staging map: vector v = tid + i * NT of the (contiguous) tile is row v / VPR, chunk v % VPR
     const int st_row = threadIdx.x / VPR, st_chunk = threadIdx.x % VPR;
-    const int k_dst = st_row * KP + st_chunk * 16;
+    const int k_dst = st_row * KP + (st_chunk ^ (st_row & 7)) * 16;  // rows of one thread are 8 apart or more
     const int v_dst = BW * KP + st_row * VP + st_chunk * 16;
     // fragment bases
-    const int k_src = r16 * KP + g4 * 16;
+    const int k_src = r16 * KP;
+    const int k_sw = r16 & 7;
     const int v_src = BW * KP + (g4 * 4 + (r16 >> 2)) * VP + (r16 & 3) * 8;
 
     const int e_begin = p.row_ptr[br];
@@ -305,7 +308,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
             s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < EC; ++c) {
-                const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + c * 64);
+                const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + (((c * 4 + g4) ^ k_sw) * 16));
                 s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
             }
         }
@@ -378,7 +381,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
 
 template <typename T, int BW, int E, int WAVES>
 static int launch_attention_v2_inst(const AttnParams& p, int batch, hipStream_t st) {
-    constexpr int TILE = BW * (E * 4 + 48);
+    constexpr int TILE = BW * (E * 4 + 32);
     constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
     const int nbr = p.Nt / p.BH;
     const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;

@@ -224,7 +224,7 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
         // 256-row tiles only when they still give every CU a few workgroups; small
         // problems are latency-bound and want more, shorter workgroups.
         const int64_t big_tiles = (int64_t)((p.Mc + 255) / 256) * (p.Nc / BN) * batch;
-        const bool fill = big_tiles >= 1024;
+        const bool fill = big_tiles >= 512;
         if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
         else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
         else tile_cfg = p.Mc >= 1024 && fill ? 2 : 1;
