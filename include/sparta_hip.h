@@ -156,8 +156,13 @@ int spx_matmul(int mode, int dtype, int transA, int transB, int compressed,
  *   grad_x = inv_temperature * (y*grad_y - y * sum_live(y*grad_y))
  * x / y are [batch,H,W] (compressed == 0; only entries of live blocks are
  * written, the caller zero-fills y) or [batch, nnz*BH*BW] (compressed != 0;
- * every entry is written).  mask is uint8 in the same layout as one batch of x.
+ * every entry is written).  mask is uint8 in the same layout as one batch of x;
+ * NULL means that every entry of a live block takes part.
  * batch_stride: elements between batches of x / y.
+ * tile_cfg: 0 = pick; 1 = one entry per access; 2 = 16-byte accesses, one
+ * wavefront per row; 3 = 16-byte accesses, sixteen lanes per row (for rows of
+ * at most 512 live 16-bit entries; longer rows stay correct).  2 and 3 need BW
+ * a multiple of 16 bytes of entries and 16-byte aligned tensors.
  * ------------------------------------------------------------------------ */
 int spx_softmax_forward(int dtype, int compressed, const void* x, void* y,
                         const int32_t* row_ptr, const int32_t* bcsr_idx,

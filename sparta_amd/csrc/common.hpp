@@ -88,6 +88,26 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
     }
     return v;
 }
+// Reductions over each aligned group of 16 lanes (a DPP "row"): four data-parallel
+// steps on the VALU, no LDS traffic.  Every lane of the group gets the result.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row16_reduce_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
+    v = fmaxf(v, dpp_move<0x140>(v));  // row_mirror
+    return v;
+}
+__device__ __forceinline__ float row16_reduce_sum(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);
+    return v;
+}
+
 __device__ __forceinline__ float wave_reduce_max(float v) {
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) v = fmaxf(v, __shfl_xor(v, d, 64));

@@ -72,6 +72,55 @@ __device__ __forceinline__ int dds_block_of_workgroup(const DdsParams& p) {
     return -1;
 }
 
+// Epilogue shared by both kernels: the accumulators meet in LDS as fp32 (one copy per
+// k part), each thread then sums, adds the bias and stores 16 bytes of one output row.
+template <typename T, int BM, int BN, typename Acc>
+__device__ __forceinline__ void dds_epilogue(const DdsParams& p, const Acc& acc, float* Ef, int i, int bi, int bj,
+                                             int64_t b, int wgm, int wgn, int kpart, int r16, int g4) {
+    typedef DdsWaveGrid<BM / 16, BN / 16> G;
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int LDE = BN + 4;  // keeps 16-byte alignment of a row, shifts rows by four banks
+#pragma unroll
+    for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+        for (int y = 0; y < G::WTN; ++y)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int m = (wgm * G::WTM + x) * 16 + g4 * 4 + q;
+                const int n = (wgn * G::WTN + y) * 16 + r16;
+                Ef[(kpart * BM + m) * LDE + n] = acc[x][y][q];
+            }
+    __syncthreads();
+    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
+    T* C = reinterpret_cast<T*>(p.C) + b * p.c_batch;
+    constexpr int VPR = BN / VE;  // 16-byte vectors per output row
+    for (int v = threadIdx.x; v < BM * VPR; v += 256) {
+        const int m = v / VPR;
+        const int n = (v - m * VPR) * VE;
+        float s[VE];
+#pragma unroll
+        for (int e = 0; e < VE; ++e) s[e] = 0.f;
+#pragma unroll
+        for (int kp = 0; kp < G::KS; ++kp) {
+#pragma unroll
+            for (int e = 0; e < VE; e += 4) {
+                const f32x4 part = *reinterpret_cast<const f32x4*>(Ef + (kp * BM + m) * LDE + n + e);
+                s[e] += part[0]; s[e + 1] += part[1]; s[e + 2] += part[2]; s[e + 3] += part[3];
+            }
+        }
+        if (biasT) {
+#pragma unroll
+            for (int e = 0; e < VE; ++e) s[e] += Elem<T>::to_float(biasT[bj * BN + n + e]);
+        }
+        union { vec16 q; T t[VE]; } u;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) u.t[e] = Elem<T>::from_float(s[e]);
+        const int64_t off = p.compressed ? (int64_t)i * (BM * BN) + m * BN + n
+                                         : ((int64_t)bi * BM + m) * p.N + (int64_t)bj * BN + n;
+        *reinterpret_cast<vec16*>(C + off) = u.q;
+    }
+}
+
 template <typename T, int BM, int BN>
 __global__ __launch_bounds__(256) void dds_kernel(DdsParams p) {
     constexpr int MT = BM / 16, NT = BN / 16;
@@ -162,33 +211,7 @@ __global__ __launch_bounds__(256) void dds_kernel(DdsParams p) {
         __syncthreads();
     }
 
-    // ---- epilogue: partial sums -> LDS fp32 -> sum over k parts, bias, store ----
-    constexpr int LDE = BN + 1;
-    float* Ef = reinterpret_cast<float*>(smem);
-#pragma unroll
-    for (int x = 0; x < G::WTM; ++x)
-#pragma unroll
-        for (int y = 0; y < G::WTN; ++y)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int m = (wgm * G::WTM + x) * 16 + g4 * 4 + q;
-                const int n = (wgn * G::WTN + y) * 16 + r16;
-                Ef[(kpart * BM + m) * LDE + n] = acc[x][y][q];
-            }
-    __syncthreads();
-    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
-    T* C = reinterpret_cast<T*>(p.C) + b * p.c_batch;
-    for (int v = threadIdx.x; v < BM * BN; v += 256) {
-        const int m = v / BN;
-        const int n = v - m * BN;
-        float s = 0.f;
-#pragma unroll
-        for (int kp = 0; kp < G::KS; ++kp) s += Ef[(kp * BM + m) * LDE + n];
-        if (biasT) s += Elem<T>::to_float(biasT[bj * BN + n]);
-        const int64_t off = p.compressed ? (int64_t)i * (BM * BN) + v
-                                         : ((int64_t)bi * BM + m) * p.N + (int64_t)bj * BN + n;
-        C[off] = Elem<T>::from_float(s);
-    }
+    dds_epilogue<T, BM, BN>(p, acc, reinterpret_cast<float*>(smem), i, bi, bj, b, wgm, wgn, kpart, r16, g4);
 }
 
 // ---- pipelined variant -----------------------------------------------------------------
@@ -323,33 +346,7 @@ __global__ __launch_bounds__(256) void dds_pipe_kernel(DdsParams p) {
     }
     __syncthreads();  // all fragments are consumed before the buffers are reused
 
-    // ---- epilogue: partial sums -> LDS fp32 -> sum over k parts, bias, store ----
-    constexpr int LDE = BN + 1;
-    float* Ef = reinterpret_cast<float*>(smem);
-#pragma unroll
-    for (int x = 0; x < G::WTM; ++x)
-#pragma unroll
-        for (int y = 0; y < G::WTN; ++y)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int m = (wgm * G::WTM + x) * 16 + g4 * 4 + q;
-                const int n = (wgn * G::WTN + y) * 16 + r16;
-                Ef[(kpart * BM + m) * LDE + n] = acc[x][y][q];
-            }
-    __syncthreads();
-    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
-    T* C = reinterpret_cast<T*>(p.C) + b * p.c_batch;
-    for (int v = threadIdx.x; v < BM * BN; v += 256) {
-        const int m = v / BN;
-        const int n = v - m * BN;
-        float s = 0.f;
-#pragma unroll
-        for (int kp = 0; kp < G::KS; ++kp) s += Ef[(kp * BM + m) * LDE + n];
-        if (biasT) s += Elem<T>::to_float(biasT[bj * BN + n]);
-        const int64_t off = p.compressed ? (int64_t)i * (BM * BN) + v
-                                         : ((int64_t)bi * BM + m) * p.N + (int64_t)bj * BN + n;
-        C[off] = Elem<T>::from_float(s);
-    }
+    dds_epilogue<T, BM, BN>(p, acc, reinterpret_cast<float*>(smem), i, bi, bj, b, wgm, wgn, kpart, r16, g4);
 }
 
 template <typename T, int BM, int BN>
@@ -359,7 +356,7 @@ static int launch_dds_pipe_inst(const DdsParams& p, int nnz_bound, int batch, hi
     constexpr int NST = DdsPipeCfg<BM, BN>::NST;
     typedef DdsWaveGrid<BM / 16, BN / 16> G;
     size_t smem = 2 * (size_t)(BM + BN) * (KT + VE) * sizeof(T);
-    size_t epi = (size_t)G::KS * BM * (BN + 1) * sizeof(float);
+    size_t epi = (size_t)G::KS * BM * (BN + 4) * sizeof(float);
     if (epi > smem) smem = epi;
     if (smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_pipe_kernel<T, BM, BN, NST>),
@@ -385,7 +382,7 @@ static int launch_dds_inst(const DdsParams& p, int nnz_bound, int batch, hipStre
     constexpr int KT = sizeof(T) == 2 ? 128 : 64;
     typedef DdsWaveGrid<BM / 16, BN / 16> G;
     size_t smem = (size_t)(BM + BN) * (KT + VE) * sizeof(T);
-    size_t epi = (size_t)G::KS * BM * (BN + 1) * sizeof(float);
+    size_t epi = (size_t)G::KS * BM * (BN + 4) * sizeof(float);
     if (epi > smem) smem = epi;
     hipLaunchKernelGGL((dds_kernel<T, BM, BN>), dim3(nnz_bound, batch, 1), dim3(256), smem, st, p);
     SPX_LAUNCH_CHECK("dds_kernel");

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
             cache[t] = 0.f;
             if (e < rv.n) {
                 const int64_t off = entry_offset(p, rv, e);
-                if (p.mask[off]) {
+                if (!p.mask || p.mask[off]) {
                     cache[t] = Elem<T>::to_float(x[off]);
                     live_bits |= 1u << t;
                     vmax = fmaxf(vmax, cache[t]);
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
         }
         for (int e = lane + 64 * SM_CACHE; e < rv.n; e += 64) {
             const int64_t off = entry_offset(p, rv, e);
-            if (p.mask[off]) vmax = fmaxf(vmax, Elem<T>::to_float(x[off]));
+            if (!p.mask || p.mask[off]) vmax = fmaxf(vmax, Elem<T>::to_float(x[off]));
         }
         vmax = wave_reduce_max(vmax);
         float sum = 0.f;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
         }
         for (int e = lane + 64 * SM_CACHE; e < rv.n; e += 64) {
             const int64_t off = entry_offset(p, rv, e);
-            if (p.mask[off]) sum += __expf((Elem<T>::to_float(x[off]) - vmax) * p.inv_t);
+            if (!p.mask || p.mask[off]) sum += __expf((Elem<T>::to_float(x[off]) - vmax) * p.inv_t);
         }
         sum = wave_reduce_sum(sum);
         const float inv = sum > 0.f ? 1.f / sum : 0.f;
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
         for (int e = lane + 64 * SM_CACHE; e < rv.n; e += 64) {
             const int64_t off = entry_offset(p, rv, e);
             float v = 0.f;
-            if (p.mask[off]) v = __expf((Elem<T>::to_float(x[off]) - vmax) * p.inv_t) * inv;
+            if (!p.mask || p.mask[off]) v = __expf((Elem<T>::to_float(x[off]) - vmax) * p.inv_t) * inv;
             out[off] = Elem<T>::from_float(v);
         }
     } else {
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
             ycache[t] = 0.f;
             if (e < rv.n) {
                 const int64_t off = entry_offset(p, rv, e);
-                if (p.mask[off]) {
+                if (!p.mask || p.mask[off]) {
                     ycache[t] = Elem<T>::to_float(yin[off]);
                     cache[t] = ycache[t] * Elem<T>::to_float(x[off]);
                     dot += cache[t];
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
         }
         for (int e = lane + 64 * SM_CACHE; e < rv.n; e += 64) {
             const int64_t off = entry_offset(p, rv, e);
-            if (p.mask[off]) dot += Elem<T>::to_float(yin[off]) * Elem<T>::to_float(x[off]);
+            if (!p.mask || p.mask[off]) dot += Elem<T>::to_float(yin[off]) * Elem<T>::to_float(x[off]);
         }
         dot = wave_reduce_sum(dot);
 #pragma unroll
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
         for (int e = lane + 64 * SM_CACHE; e < rv.n; e += 64) {
             const int64_t off = entry_offset(p, rv, e);
             float v = 0.f;
-            if (p.mask[off]) {
+            if (!p.mask || p.mask[off]) {
                 const float yv = Elem<T>::to_float(yin[off]);
                 v = p.inv_t * (yv * Elem<T>::to_float(x[off]) - yv * dot);
             }
@@ -153,12 +153,235 @@ __global__ __launch_bounds__(64 * SM_ROWS) void softmax_kernel(SoftmaxParams p) 
     }
 }
 
+// ---- vectorized variant -------------------------------------------------------------------
+// Same row-per-wavefront scheme with 16-byte accesses: a lane owns whole vectors of VE
+// consecutive entries of one live block row (VE = 8 for 16-bit types, 4 for fp32), reads
+// the VE mask bytes as one word and keeps up to SMV_CACHE vectors in registers, so a row
+// of up to 64 * SMV_CACHE * VE candidate entries moves through HBM once each way.  A NULL
+// mask means that every entry of a live block takes part.  Needs BW % VE == 0.
+constexpr int SMV_CACHE = 4;
+constexpr int SMV_ROWS = 4;
+
+template <typename T> struct SmVec;
+template <> struct SmVec<float> {
+    static constexpr int VE = 4;
+    typedef uint32_t mask_t;
+    __device__ static void unpack(const vec16& v, float* f) {
+        f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+    }
+    __device__ static vec16 pack(const float* f) {
+        return vec16{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+    }
+};
+template <> struct SmVec<_Float16> {
+    static constexpr int VE = 8;
+    typedef uint64_t mask_t;
+    __device__ static void unpack(const vec16& v, float* f) {
+        union { vec16 q; _Float16 h[8]; } u; u.q = v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)u.h[i];
+    }
+    __device__ static vec16 pack(const float* f) {
+        union { vec16 q; _Float16 h[8]; } u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u.h[i] = (_Float16)f[i];
+        return u.q;
+    }
+};
+template <> struct SmVec<bf16_t> {
+    static constexpr int VE = 8;
+    typedef uint64_t mask_t;
+    __device__ static void unpack(const vec16& v, float* f) {
+        f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+        f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+        f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+        f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+    }
+    __device__ static vec16 pack(const float* f) {
+        vec16 r;
+        r.x = (uint32_t)float_to_bf16(f[0]) | ((uint32_t)float_to_bf16(f[1]) << 16);
+        r.y = (uint32_t)float_to_bf16(f[2]) | ((uint32_t)float_to_bf16(f[3]) << 16);
+        r.z = (uint32_t)float_to_bf16(f[4]) | ((uint32_t)float_to_bf16(f[5]) << 16);
+        r.w = (uint32_t)float_to_bf16(f[6]) | ((uint32_t)float_to_bf16(f[7]) << 16);
+        return r;
+    }
+};
+
+// element offset of vector v (VE entries) of the row
+template <int VE>
+__device__ __forceinline__ int64_t vector_offset(const SoftmaxParams& p, const RowView& rv, int v, int log_vpb) {
+    const int bo = v >> log_vpb;
+    const int c = (v & ((1 << log_vpb) - 1)) * VE;
+    if (p.compressed) return (((int64_t)(rv.first + bo) << p.log_bh) + rv.rr) * p.BW + c;
+    const int bc = p.bcsr_idx[rv.first + bo] & 0xffff;
+    return (int64_t)rv.row * p.W + (int64_t)bc * p.BW + c;
+}
+
+// LPR lanes share a row (16: four rows per wavefront, for rows of up to 16 * SMV_CACHE
+// vectors; 64: one row per wavefront, any length).
+template <int LPR> __device__ __forceinline__ float group_reduce_max(float v) {
+    v = row16_reduce_max(v);
+    if constexpr (LPR == 64) {
+        v = fmaxf(v, __shfl_xor(v, 16, 64));
+        v = fmaxf(v, __shfl_xor(v, 32, 64));
+    }
+    return v;
+}
+template <int LPR> __device__ __forceinline__ float group_reduce_sum(float v) {
+    v = row16_reduce_sum(v);
+    if constexpr (LPR == 64) {
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+    }
+    return v;
+}
+
+template <typename T, bool BACKWARD, int LPR>
+__global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParams p) {
+    constexpr int VE = SmVec<T>::VE;
+    constexpr int RPW = 64 / LPR;
+    typedef typename SmVec<T>::mask_t mask_t;
+    const int lane = lane_id() % LPR;
+    const int wave = threadIdx.x >> 6;
+    RowView rv;
+    rv.row = (blockIdx.x * SMV_ROWS + wave) * RPW + lane_id() / LPR;
+    if (rv.row >= p.H) return;
+    rv.br = rv.row >> p.log_bh;
+    rv.rr = rv.row & (p.BH - 1);
+    rv.first = p.row_ptr[rv.br];
+    rv.nblk = p.row_ptr[rv.br + 1] - rv.first;
+    const int log_vpb = p.log_bw - (VE == 8 ? 3 : 2);  // vectors per block row
+    const int nvec = rv.nblk << log_vpb;
+    rv.n = nvec;
+    if (nvec == 0) return;
+
+    const int64_t boff = (int64_t)blockIdx.y * p.batch_stride;
+    const T* x = reinterpret_cast<const T*>(p.x) + boff;
+    const T* yin = BACKWARD ? reinterpret_cast<const T*>(p.y_in) + boff : nullptr;
+    T* out = reinterpret_cast<T*>(p.out) + boff;
+
+    float cache[SMV_CACHE][VE];
+    float ycache[BACKWARD ? SMV_CACHE : 1][VE];
+    mask_t live[SMV_CACHE];
+    int64_t offs[SMV_CACHE];
+#pragma unroll
+    for (int t = 0; t < SMV_CACHE; ++t) {
+        const int v = lane + LPR * t;
+        live[t] = 0;
+        offs[t] = 0;
+        if (v < nvec) {
+            offs[t] = vector_offset<VE>(p, rv, v, log_vpb);
+            live[t] = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + offs[t]) : ~(mask_t)0;
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + offs[t]), cache[t]);
+            if (BACKWARD) SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + offs[t]), ycache[t]);
+        }
+    }
+    if (!BACKWARD) {
+        float vmax = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < SMV_CACHE; ++t)
+#pragma unroll
+            for (int i = 0; i < VE; ++i)
+                if ((live[t] >> (8 * i)) & 0xff) vmax = fmaxf(vmax, cache[t][i]);
+        for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
+            const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
+            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            float f[VE];
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), f);
+#pragma unroll
+            for (int i = 0; i < VE; ++i)
+                if ((m >> (8 * i)) & 0xff) vmax = fmaxf(vmax, f[i]);
+        }
+        vmax = group_reduce_max<LPR>(vmax);
+        float sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < SMV_CACHE; ++t)
+#pragma unroll
+            for (int i = 0; i < VE; ++i) {
+                cache[t][i] = ((live[t] >> (8 * i)) & 0xff) ? __expf((cache[t][i] - vmax) * p.inv_t) : 0.f;
+                sum += cache[t][i];
+            }
+        for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
+            const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
+            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            float f[VE];
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), f);
+#pragma unroll
+            for (int i = 0; i < VE; ++i)
+                if ((m >> (8 * i)) & 0xff) sum += __expf((f[i] - vmax) * p.inv_t);
+        }
+        sum = group_reduce_sum<LPR>(sum);
+        const float inv = sum > 0.f ? 1.f / sum : 0.f;
+#pragma unroll
+        for (int t = 0; t < SMV_CACHE; ++t) {
+            if (lane + LPR * t < nvec) {
+#pragma unroll
+                for (int i = 0; i < VE; ++i) cache[t][i] *= inv;
+                *reinterpret_cast<vec16*>(out + offs[t]) = SmVec<T>::pack(cache[t]);
+            }
+        }
+        for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
+            const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
+            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            float f[VE];
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), f);
+#pragma unroll
+            for (int i = 0; i < VE; ++i)
+                f[i] = ((m >> (8 * i)) & 0xff) ? __expf((f[i] - vmax) * p.inv_t) * inv : 0.f;
+            *reinterpret_cast<vec16*>(out + off) = SmVec<T>::pack(f);
+        }
+    } else {
+        // cache holds grad_y, ycache holds y; grad_x = inv_t * y * (grad_y - sum(y * grad_y))
+        float dot = 0.f;
+#pragma unroll
+        for (int t = 0; t < SMV_CACHE; ++t)
+#pragma unroll
+            for (int i = 0; i < VE; ++i) {
+                const bool on = (live[t] >> (8 * i)) & 0xff;
+                ycache[t][i] = on ? ycache[t][i] : 0.f;
+                cache[t][i] = on ? ycache[t][i] * cache[t][i] : 0.f;
+                dot += cache[t][i];
+            }
+        for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
+            const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
+            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            float g[VE], yv[VE];
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), g);
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + off), yv);
+#pragma unroll
+            for (int i = 0; i < VE; ++i)
+                if ((m >> (8 * i)) & 0xff) dot += yv[i] * g[i];
+        }
+        dot = group_reduce_sum<LPR>(dot);
+#pragma unroll
+        for (int t = 0; t < SMV_CACHE; ++t) {
+            if (lane + LPR * t < nvec) {
+#pragma unroll
+                for (int i = 0; i < VE; ++i) cache[t][i] = p.inv_t * (cache[t][i] - ycache[t][i] * dot);
+                *reinterpret_cast<vec16*>(out + offs[t]) = SmVec<T>::pack(cache[t]);
+            }
+        }
+        for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
+            const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
+            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            float g[VE], yv[VE];
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), g);
+            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + off), yv);
+#pragma unroll
+            for (int i = 0; i < VE; ++i)
+                g[i] = ((m >> (8 * i)) & 0xff) ? p.inv_t * (yv[i] * g[i] - yv[i] * dot) : 0.f;
+            *reinterpret_cast<vec16*>(out + off) = SmVec<T>::pack(g);
+        }
+    }
+}
+
 template <bool BACKWARD>
 static int launch_softmax(int dtype, int compressed, const void* x, const void* y_in, void* out,
                           const int32_t* row_ptr, const int32_t* bcsr_idx, const uint8_t* mask,
                           float inv_t, int batch, int H, int W, int BH, int BW,
-                          int64_t batch_stride, hipStream_t st) {
-    SPX_REQUIRE(x && out && row_ptr && bcsr_idx && mask, SPX_E_NULL, "a required buffer is NULL");
+                          int64_t batch_stride, int tile_cfg, hipStream_t st) {
+    SPX_REQUIRE(x && out && row_ptr && bcsr_idx, SPX_E_NULL, "a required buffer is NULL");
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(!BACKWARD || y_in, SPX_E_NULL, "y is required for the backward pass");
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(valid_block_edge(BH) && valid_block_edge(BW), SPX_E_CONFIG,
@@ -173,6 +396,32 @@ static int launch_softmax(int dtype, int compressed, const void* x, const void* 
     p.inv_t = inv_t;
     p.H = H; p.W = W; p.BH = BH; p.BW = BW; p.log_bh = ilog2(BH); p.log_bw = ilog2(BW);
     p.compressed = compressed; p.batch_stride = batch_stride;
+    // tile_cfg 0: pick; 1: one entry per access; 2: 16-byte accesses, a wavefront per row;
+    // 3: 16-byte accesses, sixteen lanes per row (best when rows hold at most
+    // 16 * SMV_CACHE vectors of live entries; longer rows stay correct).  The live length of
+    // a row is only known on the device, so the default goes by the full width.
+    const int ve = dtype == SPX_F32 ? 4 : 8;
+    const bool vec_ok = BW % ve == 0 && aligned(x, 16) && aligned(out, 16) && (!y_in || aligned(y_in, 16)) &&
+                        (!mask || aligned(mask, 8)) && batch_stride % ve == 0;
+    if (tile_cfg == 0) tile_cfg = vec_ok ? (W / ve <= 16 * SMV_CACHE ? 3 : 2) : 1;
+    if (tile_cfg >= 2) {
+        SPX_REQUIRE(vec_ok, SPX_E_CONFIG, "tile configs 2 and 3 need BW %% %d == 0 and 16-byte aligned tensors", ve);
+        const bool narrow = tile_cfg == 3;
+        const int rows_per_group = SMV_ROWS * (narrow ? 4 : 1);
+        dim3 vgrid((H + rows_per_group - 1) / rows_per_group, batch, 1);
+        dim3 vblock(64 * SMV_ROWS);
+#define SPX_SMV(T) \
+        if (narrow) hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 16>), vgrid, vblock, 0, st, p); \
+        else hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 64>), vgrid, vblock, 0, st, p);
+        switch (dtype) {
+            case SPX_F32: SPX_SMV(float) break;
+            case SPX_F16: SPX_SMV(_Float16) break;
+            default: SPX_SMV(bf16_t) break;
+        }
+#undef SPX_SMV
+        SPX_LAUNCH_CHECK("softmax_vec_kernel");
+        return 0;
+    }
     dim3 grid((H + SM_ROWS - 1) / SM_ROWS, batch, 1);
     dim3 block(64 * SM_ROWS);
     switch (dtype) {
@@ -191,9 +440,8 @@ extern "C" int spx_softmax_forward(int dtype, int compressed, const void* x, voi
                                    const uint8_t* mask, float inv_temperature,
                                    int batch, int H, int W, int BH, int BW,
                                    int64_t batch_stride, int tile_cfg, spx_stream_t stream) {
-    (void)tile_cfg;
     return spx::launch_softmax<false>(dtype, compressed, x, nullptr, y, row_ptr, bcsr_idx, mask,
-                                      inv_temperature, batch, H, W, BH, BW, batch_stride,
+                                      inv_temperature, batch, H, W, BH, BW, batch_stride, tile_cfg,
                                       reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -202,8 +450,7 @@ extern "C" int spx_softmax_backward(int dtype, int compressed, const void* grad_
                                     const uint8_t* mask, float inv_temperature,
                                     int batch, int H, int W, int BH, int BW,
                                     int64_t batch_stride, int tile_cfg, spx_stream_t stream) {
-    (void)tile_cfg;
     return spx::launch_softmax<true>(dtype, compressed, grad_y, y, grad_x, row_ptr, bcsr_idx, mask,
-                                     inv_temperature, batch, H, W, BH, BW, batch_stride,
+                                     inv_temperature, batch, H, W, BH, BW, batch_stride, tile_cfg,
                                      reinterpret_cast<hipStream_t>(stream));
 }

@@ -25,7 +25,10 @@ static const spx_tile_cfg kDdsCfgs[] = {
     {2, 0, 0, 4, 3, 16, 7, "block-per-workgroup-pipelined"},
 };
 static const spx_tile_cfg kSoftmaxCfgs[] = {
-    {0, 4, 0, 4, 0, 4, 7, "wave-per-row"},
+    {0, 4, 0, 4, 0, 4, 7, "auto"},
+    {1, 4, 0, 4, 0, 4, 7, "wave-per-row"},
+    {2, 4, 0, 4, 0, 8, 7, "wave-per-row-16-byte"},
+    {3, 16, 0, 4, 0, 8, 7, "16-lanes-per-row-16-byte"},
 };
 static const spx_tile_cfg kAttentionCfgs[] = {
     {0, 0, 0, 0, 1, 16, 6, "auto"},

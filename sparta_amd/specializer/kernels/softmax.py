@@ -28,6 +28,8 @@ class SparseSoftmaxKernel(KernelBase):
         for name in ('BATCH_SIZE', 'GLOBAL_H_VALUE', 'GLOBAL_W_VALUE'):
             self._add_parameter(name)
         self._add_parameter('COMPRESSED', value=self._compressed)
+        # gfx950 kernel variant (0 = chosen by the library); outside the search space
+        self._add_parameter('TILE_CFG', value=0)
 
     def set_parameters(self, params: Dict[str, Any]):
         super().set_parameters(params)
@@ -50,13 +52,24 @@ class SparseSoftmaxKernel(KernelBase):
         BH, BW = self.get_block_shape()
         indexes = self.ports['y'].indexes
         mask = indexes.raw_mask
+        tile_cfg = int(self.get_parameter('TILE_CFG') or 0)
         if self._compressed:
-            mask = indexes.convert(mask)
             shape = (batch_size, indexes.block_nnz * BH * BW)
         else:
             shape = (batch_size, H, W)
+        # A mask that is uniform inside its blocks needs no per-entry test: the kernel
+        # takes NULL for "every entry of a live block takes part" (one synchronising
+        # comparison per index build).
+        if not self.ports['y'].at_capacity and indexes.is_block_uniform():
+            mask = None
+        elif self._compressed:
+            mask = indexes.convert(mask)
         stride = int(np.prod(shape[1:]))
-        return batch_size, H, W, BH, BW, indexes, mask, shape, stride
+        if tile_cfg == 0 and not self.ports['y'].at_capacity and BW % 8 == 0:
+            # short rows (known from the live block count): sixteen lanes per row
+            if indexes.block_nnz * BW <= 410 * max(indexes.row_num, 1):
+                tile_cfg = 3
+        return batch_size, H, W, BH, BW, indexes, mask, shape, stride, tile_cfg
 
     def _mask_and_compress(self, tensors: List[torch.Tensor], positions: List[int]):
         mask = self.ports['y'].mask
@@ -76,7 +89,7 @@ class SparseSoftmaxForwardKernel(SparseSoftmaxKernel):
         self.ports['x'].connect(self, 'y')
 
     def update_func(self):
-        batch_size, H, W, BH, BW, indexes, mask, shape, stride = self._launch_state()
+        batch_size, H, W, BH, BW, indexes, mask, shape, stride, tile_cfg = self._launch_state()
         compressed = int(self._compressed)
         alloc = torch.empty if self._compressed else torch.zeros
         row_ptr, idx = indexes.row_ptr, indexes._bcsr_buf
@@ -84,10 +97,12 @@ class SparseSoftmaxForwardKernel(SparseSoftmaxKernel):
 
         def softmax_forward_func(x: torch.Tensor, T: np.float32):
             y = alloc(shape, dtype=x.dtype, device=x.device)
+            if y.numel() == 0:  # no live block: nothing to compute
+                return y
             rc = lib.spx_softmax_forward(
                 _lib.dtype_code(x.dtype), compressed, _lib.dev_ptr(x.contiguous()), _lib.dev_ptr(y),
                 _lib.dev_ptr(row_ptr), _lib.dev_ptr(idx), _lib.dev_ptr(mask), float(T),
-                batch_size, H, W, BH, BW, stride, 0, _lib.current_stream(x.device))
+                batch_size, H, W, BH, BW, stride, tile_cfg, _lib.current_stream(x.device))
             _lib.check(rc, 'spx_softmax_forward')
             return y
 
@@ -114,7 +129,7 @@ class SparseSoftmaxBackwardKernel(SparseSoftmaxKernel):
         self.ports['grad_y'].connect(self, 'grad_x')
 
     def update_func(self):
-        batch_size, H, W, BH, BW, indexes, mask, shape, stride = self._launch_state()
+        batch_size, H, W, BH, BW, indexes, mask, shape, stride, tile_cfg = self._launch_state()
         compressed = int(self._compressed)
         alloc = torch.empty if self._compressed else torch.zeros
         row_ptr, idx = indexes.row_ptr, indexes._bcsr_buf
@@ -122,11 +137,13 @@ class SparseSoftmaxBackwardKernel(SparseSoftmaxKernel):
 
         def softmax_backward_func(grad_y: torch.Tensor, y: torch.Tensor, T: np.float32):
             grad_x = alloc(shape, dtype=grad_y.dtype, device=grad_y.device)
+            if grad_x.numel() == 0:
+                return grad_x
             rc = lib.spx_softmax_backward(
                 _lib.dtype_code(grad_y.dtype), compressed, _lib.dev_ptr(grad_y.contiguous()),
                 _lib.dev_ptr(y.contiguous()), _lib.dev_ptr(grad_x),
                 _lib.dev_ptr(row_ptr), _lib.dev_ptr(idx), _lib.dev_ptr(mask), float(T),
-                batch_size, H, W, BH, BW, stride, 0, _lib.current_stream(grad_y.device))
+                batch_size, H, W, BH, BW, stride, tile_cfg, _lib.current_stream(grad_y.device))
             _lib.check(rc, 'spx_softmax_backward')
             return grad_x
 

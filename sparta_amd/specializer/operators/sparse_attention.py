@@ -71,7 +71,7 @@ class SparseAttention(OperatorBase):
         if self._fused_mask_key is not indexes:
             # A mask that is uniform inside its blocks needs no per-element test in the
             # kernel; decided once per index build (one synchronising comparison).
-            block_level = torch.equal(indexes.get_mask(), indexes.raw_mask != 0)
+            block_level = indexes.is_block_uniform()
             self._fused_mask = None if block_level else indexes.raw_mask
             self._fused_mask_key = indexes
         lead = query.shape[:-2]

@@ -85,6 +85,16 @@ class BCSIndexes(TeSAIndexes):
         grid[rows, cols] = 1
         return grid
 
+    def is_block_uniform(self) -> bool:
+        """True when every element of every live block is set in the raw mask, i.e. the
+        element mask carries no information beyond the block index.  Computed once per
+        index (one synchronising comparison) and cached."""
+        cached = self.__dict__.get('_block_uniform')
+        if cached is None:
+            cached = bool(torch.equal(self.get_mask() != 0, self.raw_mask != 0))
+            self.__dict__['_block_uniform'] = cached
+        return cached
+
     def get_mask(self) -> torch.Tensor:
         grid = self.get_block_mask()
         full = grid.repeat_interleave(self.block_H, dim=0).repeat_interleave(self.block_W, dim=1)
