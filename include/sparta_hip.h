@@ -191,6 +191,23 @@ int spx_attention_forward(int dtype, const void* q, const void* k, const void* v
                           int tile_cfg, spx_stream_t stream);
 
 /* ------------------------------------------------------------------------ *
+ * Sequence-length attention: q, k, v, out are [batch, heads, N, E]; batch b
+ * attends over its first seqlens[b] positions only (int32 [batch], on the
+ * device; values are clamped to [0, N]):
+ *   out[b,h,i,:] = softmax_{j < L}(q_i . k_j * inv_temperature) v_j   for i < L,
+ *   out[b,h,i,:] = 0                                                    for i >= L.
+ * fp32, fp16 and bf16; N and E multiples of 32, E in {32, 64, 96, 128}.
+ * Replaces seqlen_dynamic_sparse_attention_cpp.forward(Q, K, V, inter_result,
+ * seqlens, head_num) (csrc/seqlen_dynamic_sparse_attention_forward.cpp:7-26);
+ * the reference applies no temperature (pass 1.0f) and needs a [B*H*N*N] fp32
+ * scratch that this entry point does not.
+ * ------------------------------------------------------------------------ */
+int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const void* v, void* out,
+                                 const int32_t* seqlens, float inv_temperature,
+                                 int batch, int heads, int N, int E,
+                                 int tile_cfg, spx_stream_t stream);
+
+/* ------------------------------------------------------------------------ *
  * MoE sparse forward: out[t,:] = tokens[t,:] . W[exp_ids[t]].
  * Replace sparse_moe_cpp.convert_index / forward
  * (csrc/moe_sparse_forward.cpp:7-25, csrc/moe_sparse_forward_kernel.cu.j2:58-116,

@@ -452,6 +452,173 @@ static int launch_attention(const AttnParams& p, int batch, int BW, int E, hipSt
     return fail(SPX_E_CONFIG, "fused attention supports key blocks of 16/32/64/128 and head dims 32/64/128 (got %d, %d)", BW, E);
 }
 
+// ---- sequence-length attention ------------------------------------------------------------
+// out[b,h,i,:] = softmax_j<L(q_i . k_j * inv_t) v_j  for i < L = seqlens[b], zero rows for
+// i >= L: the per-batch "mask" is a prefix square, so the key loop simply stops at L and
+// no index or score scratch is needed.  fp32 as well as the 16-bit types (16x16 MFMAs with
+// k = 16 for both products; the fp32 one is four 16x16x4 steps).
+// Replaces seqlen_dynamic_sparse_attention_cpp.forward
+// (csrc/seqlen_dynamic_sparse_attention_forward.cpp:7-26 and the three kernels of
+// csrc/seqlen_dynamic_sparse_attention_forward_kernel.cu:511-583), whose softmax uses
+// no temperature (SPARSE_SOFTMAX, :305-377) and whose rows past the length stay zero.
+template <> struct AttnMma<float> {
+    typedef f32x4 pfrag;
+    __device__ static pfrag pack(float a, float b, float c, float d) { return pfrag{a, b, c, d}; }
+};
+
+struct SeqlenParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* out;
+    const int32_t* seqlens;
+    float inv_t;
+    int heads, N;
+};
+
+// TB queries and TB keys per step, E head dimension; TB / 16 wavefronts.
+template <typename T, int TB, int E>
+__global__ __launch_bounds__(TB * 4) void attention_seqlen_kernel(SeqlenParams p) {
+    constexpr int WAVES = TB / 16;
+    constexpr int NT = 64 * WAVES;
+    constexpr int KT = TB / 16;     // key tiles per step
+    constexpr int ET = E / 16;      // 16-wide chunks of the head dimension
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int LDK = E + VE;     // K tile row pitch (elements)
+    constexpr int LDV = TB + VE;    // V^T tile row pitch
+    typedef typename Mma16<T>::frag Frag;
+    typedef typename AttnMma<T>::pfrag PFrag;
+    extern __shared__ __align__(16) char smem[];
+    T* Ks = reinterpret_cast<T*>(smem);        // [TB][LDK]
+    T* Vt = Ks + TB * LDK;                     // [E][LDV]
+
+    const int br = blockIdx.x;
+    const int64_t b = blockIdx.y;              // batch * heads + head
+    const int L = min(max(p.seqlens[b / p.heads], 0), p.N);
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.N * E;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + b * (int64_t)p.N * E;
+    const T* Vg = reinterpret_cast<const T*>(p.v) + b * (int64_t)p.N * E;
+    T* O = reinterpret_cast<T*>(p.out) + b * (int64_t)p.N * E;
+
+    const int qrow = br * TB + wave * 16 + r16;
+    Frag qf[ET];
+#pragma unroll
+    for (int c = 0; c < ET; ++c) qf[c] = Mma16<T>::load(Q + (int64_t)qrow * E + c * 16 + g4 * 4);
+
+    f32x4 oacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -1e30f, l_run = 0.f;
+
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const int n_steps = br * TB < L ? (L + TB - 1) / TB : 0;   // query blocks past the length do nothing
+    for (int step = 0; step < n_steps; ++step) {
+        const int key0 = step * TB;
+        __syncthreads();  // the previous step's fragments are consumed
+        for (int v = threadIdx.x; v < TB * (E / VE); v += NT) {
+            const int key = v / (E / VE), c = v % (E / VE);
+            *reinterpret_cast<u32x4*>(Ks + key * LDK + c * VE) =
+                *reinterpret_cast<const u32x4*>(Kg + (int64_t)(key0 + key) * E + c * VE);
+        }
+        for (int v = threadIdx.x; v < TB * (E / VE); v += NT) {
+            const int key = v / (E / VE), c = v % (E / VE);
+            union { u32x4 v4; T e[VE]; } a;
+            a.v4 = *reinterpret_cast<const u32x4*>(Vg + (int64_t)(key0 + key) * E + c * VE);
+#pragma unroll
+            for (int i = 0; i < VE; ++i) Vt[(c * VE + i) * LDV + key] = a.e[i];
+        }
+        __syncthreads();
+
+        f32x4 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < ET; ++c) {
+                const Frag kf = Mma16<T>::load(Ks + (kt * 16 + r16) * LDK + c * 16 + g4 * 4);
+                s[kt] = Mma16<T>::mma(kf, qf[c], s[kt]);
+            }
+        }
+        // lane holds s[kt][q] = score(query r16, key key0 + kt*16 + g4*4 + q); keys >= L are out
+        float tmax = -1e30f;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (key0 + kt * 16 + g4 * 4 + q < L) tmax = fmaxf(tmax, s[kt][q]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = __expf((m_run - m_new) * p.inv_t);
+        float psum = 0.f;
+        PFrag pf[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            float pv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                pv[q] = key0 + kt * 16 + g4 * 4 + q < L ? __expf((s[kt][q] - m_new) * p.inv_t) : 0.f;
+                psum += pv[q];
+            }
+            pf[kt] = AttnMma<T>::pack(pv[0], pv[1], pv[2], pv[3]);
+        }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+            oacc[t] *= alpha;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const Frag vf = Mma16<T>::load(Vt + (t * 16 + r16) * LDV + kt * 16 + g4 * 4);
+                oacc[t] = Mma16<T>::mma(vf, pf[kt], oacc[t]);
+            }
+        }
+    }
+
+    // lane holds O^T[e = t*16 + g4*4 + q][query r16]; queries at or past the length give 0
+    const float inv_l = (qrow < L && l_run > 0.f) ? 1.f / l_run : 0.f;
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T vals[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][q] * inv_l);
+        T* dst = O + (int64_t)qrow * E + t * 16 + g4 * 4;
+        if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+        else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+    }
+}
+
+template <typename T, int TB, int E>
+static int launch_attention_seqlen_inst(const SeqlenParams& p, int batch_heads, hipStream_t st) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    const size_t smem = ((size_t)TB * (E + VE) + (size_t)E * (TB + VE)) * sizeof(T);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_seqlen_kernel<T, TB, E>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_seqlen_kernel)");
+    }
+    hipLaunchKernelGGL((attention_seqlen_kernel<T, TB, E>), dim3(p.N / TB, batch_heads, 1), dim3(TB * 4), smem, st, p);
+    SPX_LAUNCH_CHECK("attention_seqlen_kernel");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_seqlen(const SeqlenParams& p, int batch_heads, int E, hipStream_t st) {
+    const int TB = p.N % 64 == 0 ? 64 : 32;
+#define SPX_SEQ_CASE(tb, e) \
+    if (TB == tb && E == e) return launch_attention_seqlen_inst<T, tb, e>(p, batch_heads, st);
+    SPX_SEQ_CASE(64, 32) SPX_SEQ_CASE(64, 64) SPX_SEQ_CASE(64, 96) SPX_SEQ_CASE(64, 128)
+    SPX_SEQ_CASE(32, 32) SPX_SEQ_CASE(32, 64) SPX_SEQ_CASE(32, 96) SPX_SEQ_CASE(32, 128)
+#undef SPX_SEQ_CASE
+    return fail(SPX_E_CONFIG, "sequence-length attention supports head dims 32 / 64 / 96 / 128 (got %d)", E);
+}
+
 }  // namespace spx
 
 extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, const void* v, void* out,
@@ -486,4 +653,29 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     }
     if (dtype == SPX_F16) return launch_attention<_Float16>(p, batch, BW, E, st);
     return launch_attention<bf16_t>(p, batch, BW, E, st);
+}
+
+extern "C" int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const void* v, void* out,
+                                            const int32_t* seqlens, float inv_temperature,
+                                            int batch, int heads, int N, int E,
+                                            int tile_cfg, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(tile_cfg == 0, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
+    SPX_REQUIRE(batch >= 0 && heads > 0 && N > 0 && N % 32 == 0 && E > 0 && E % 32 == 0, SPX_E_SHAPE,
+                "need N %% 32 == 0 and E %% 32 == 0 (got batch=%d heads=%d N=%d E=%d)", batch, heads, N, E);
+    SPX_REQUIRE((int64_t)batch * heads <= 65535, SPX_E_SHAPE, "batch * heads = %lld out of range", (long long)batch * heads);
+    if (batch == 0) return 0;
+    SPX_REQUIRE(q && k && v && out && seqlens, SPX_E_NULL, "a required buffer is NULL");
+    SPX_REQUIRE(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 16), SPX_E_ALIGN,
+                "q, k, v, out must be 16-byte aligned");
+    SeqlenParams p;
+    p.q = q; p.k = k; p.v = v; p.out = out; p.seqlens = seqlens;
+    p.inv_t = inv_temperature; p.heads = heads; p.N = N;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case SPX_F32: return launch_attention_seqlen<float>(p, batch * heads, E, st);
+        case SPX_F16: return launch_attention_seqlen<_Float16>(p, batch * heads, E, st);
+        default: return launch_attention_seqlen<bf16_t>(p, batch * heads, E, st);
+    }
 }

@@ -1,3 +1,4 @@
 from sparta_amd.specializer.operators import (
     OperatorBase, SparseLinear, SparseBatchMatMul, SparseSoftmax, SparseAttention, DynamicSparseMoE,
+    SeqlenDynamicSparseAttention,
 )
