@@ -214,11 +214,14 @@ int launch_spmm_panel(const SpmmParams& p, int BN, int batch, int nst, hipStream
 //   3 / 4  register-direct kernel, 64 / 256-row workgroup tiles (k-contiguous operands);
 //   5 / 6  panel kernel, 256-row workgroup tiles, 2 / 3 load stages (k-contiguous
 //          operands, block depth a multiple of 64 bytes);
-//   7      panel kernel whose four wavefronts share the sparse block through LDS.
+//   7      panel kernel whose four wavefronts share the sparse block through LDS (the
+//          sparse operand may be stored with n contiguous: it is transposed on the way).
 template <typename T>
 int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipStream_t st) {
     const bool kcontig = p.d_kcontig && p.s_kcontig;
     const bool panel_ok = kcontig && (p.BK * (int)sizeof(T)) % 64 == 0;
+    // the shared-S panel variant transposes an n-contiguous sparse block while staging it
+    const bool panel7_ok = p.d_kcontig && (p.BK * (int)sizeof(T)) % 64 == 0;
     if (tile_cfg < 0 || tile_cfg > 7) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg == 0) {
         // 256-row tiles only when they still give every CU a few workgroups; small
@@ -226,11 +229,13 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
         const int64_t big_tiles = (int64_t)((p.Mc + 255) / 256) * (p.Nc / BN) * batch;
         const bool fill = big_tiles >= 512;
         if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
+        else if (panel7_ok && p.Mc >= 512 && fill) tile_cfg = 7;
         else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
         else tile_cfg = p.Mc >= 1024 && fill ? 2 : 1;
     }
     if (tile_cfg >= 5) {
-        if (!panel_ok) return fail(SPX_E_CONFIG, "tile config %d needs k-contiguous operands and 64-byte block rows", tile_cfg);
+        if (!(tile_cfg == 7 ? panel7_ok : panel_ok))
+            return fail(SPX_E_CONFIG, "tile config %d needs k-contiguous operands and 64-byte block rows", tile_cfg);
         return launch_spmm_panel<T>(p, BN, batch, tile_cfg == 6 ? 3 : tile_cfg == 7 ? 12 : 2, st);
     }
     if (tile_cfg >= 3) {

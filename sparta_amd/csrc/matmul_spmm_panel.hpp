@@ -83,10 +83,14 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
         wofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
     }
     int sofs[WL];
-    // shared S tile: this wave stages chunks wave*BN .. wave*BN+BN-1 of the BN*4 chunks
+    // shared S tile: this wave stages chunks wave*BN .. wave*BN+BN-1 of the BN*4 chunks.
+    // k-contiguous S: chunk = (n row, 16-byte piece of its 64 bytes of k); otherwise S is
+    // stored with n contiguous, a chunk is 16 bytes of n at one k and is transposed on
+    // its way into LDS.
     const int sh_chunk = wave * BN + lane;
     const int sh_row = sh_chunk >> 2, sh_chk = sh_chunk & 3;
     const bool sh_active = lane < BN;
+    const int sh_k = sh_chunk / (BN / E16), sh_n0 = (sh_chunk % (BN / E16)) * E16;
 #pragma unroll
     for (int q = 0; q < WL; ++q) {
         if constexpr (SHW) {
@@ -118,7 +122,8 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
     const int e_begin = p.ptr[j];
     const int n_blk = p.ptr[j + 1] - e_begin;
     const int n_it = n_blk * CH;
-    const int64_t sld = p.compressed ? BK : p.s_ld;
+    const int64_t sld = p.compressed ? (p.s_kcontig ? BK : BN) : p.s_ld;
+    const int64_t sh_toff = p.s_kcontig ? (int64_t)sh_row * sld + sh_chk * E16 : (int64_t)sh_k * sld + sh_n0;
 
     // The first 64 index entries of the block-column live in one VGPR pair (lane l
     // holds entry l) and are broadcast with readlane, which keeps the index fetch
@@ -157,13 +162,14 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
             slot_ = e_begin + er_;                                                                 \
         }                                                                                          \
         const int koff_ = kb_ * BK + ch_ * KC;                                                     \
-        const T* sblk_ = p.compressed ? S + slot_ * (int64_t)(BK * BN) + ch_ * KC                  \
-                                      : S + (int64_t)j * BN * p.s_ld + koff_;                      \
+        const T* sblk_ = p.compressed ? S + slot_ * (int64_t)(BK * BN) + (p.s_kcontig ? ch_ * KC : ch_ * KC * BN) \
+                                      : (p.s_kcontig ? S + (int64_t)j * BN * p.s_ld + koff_        \
+                                                     : S + (int64_t)koff_ * p.s_ld + (int64_t)j * BN); \
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
             DREG[q] = *reinterpret_cast<const u32x4*>(dptr[q] + koff_);                            \
         if constexpr (SHW) {                                                                       \
             if (sh_active)                                                                         \
-                SREG[0] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)sh_row * sld + sh_chk * E16); \
+                SREG[0] = *reinterpret_cast<const u32x4*>(sblk_ + sh_toff);                        \
         } else {                                                                                   \
             _Pragma("unroll") for (int q = 0; q < WL; ++q)                                         \
                 SREG[q] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)(q * 16 + lrow) * sld + lchk * E16); \
@@ -180,7 +186,19 @@ __global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mti
             *reinterpret_cast<u32x4*>(lds + wofs[q]) = DREG[q];                                    \
         char* sdst_ = SHW ? wsh + ((IT) & 1) * (BN * 64) : lds;                                     \
         if constexpr (SHW) {                                                                       \
-            if (sh_active) *reinterpret_cast<u32x4*>(sdst_ + sofs[0]) = SREG[0];                   \
+            if (sh_active) {                                                                       \
+                if (p.s_kcontig) {                                                                 \
+                    *reinterpret_cast<u32x4*>(sdst_ + sofs[0]) = SREG[0];                          \
+                } else {                                                                           \
+                    union { u32x4 v4; T e[E16]; } u_;                                              \
+                    u_.v4 = SREG[0];                                                               \
+                    _Pragma("unroll") for (int i = 0; i < E16; ++i) {                              \
+                        const int n_ = sh_n0 + i;                                                  \
+                        *reinterpret_cast<T*>(sdst_ + n_ * 64 + (((sh_k / E16) ^ ((n_ >> 2) & 3)) << 4) + \
+                                              (sh_k % E16) * (int)sizeof(T)) = u_.e[i];            \
+                    }                                                                              \
+                }                                                                                  \
+            }                                                                                      \
         } else {                                                                                   \
             _Pragma("unroll") for (int q = 0; q < WL; ++q)                                         \
                 *reinterpret_cast<u32x4*>(sdst_ + sofs[q]) = SREG[q];                              \
