@@ -95,6 +95,7 @@ def tune_sparse_module(module: OperatorBase, name: str, sample_inputs: List[torc
     upper_size = math.prod(len(space._value) for space in upper_space.values())
     trials_per_kernel = int(math.ceil(max_trials / upper_size)) if upper_size else 0
     best_lower: Dict[str, Dict[str, Dict[str, Any]]] = {}
+    best_lower_latency: Dict[str, float] = {}
 
     def lower_search(upper_idx: int, upper_params: Dict[int, Any]) -> float:
         _logger.info(f'[{name}][Upper Search Space] #{upper_idx}: {list(upper_params.values())}')
@@ -124,7 +125,13 @@ def tune_sparse_module(module: OperatorBase, name: str, sample_inputs: List[torc
                     best_latency = tuner.best_result
             chosen[kernel_name] = best_params
             total_latency += best_latency * weight
-        best_lower[str(upper_params)] = chosen
+        # Random search may draw the same upper point twice: keep the better of the two
+        # lower results, so that the point the upper tuner remembers and the kernel
+        # configs returned for it belong to the same trial.
+        key = str(upper_params)
+        if key not in best_lower or total_latency < best_lower_latency[key]:
+            best_lower[key] = chosen
+            best_lower_latency[key] = total_latency
         return total_latency
 
     upper_tuner = tuner_cls(upper_space, lower_search, upper_size)

@@ -80,10 +80,13 @@ class PortConfig:
         """Make `kernel.ports[port_name]` an alias of this port."""
         other = kernel.ports[port_name]
         assert self.is_sparse == other.is_sparse, 'cannot connect a sparse port with a dense one'
+        formats = (self.BCSR, self.BCSC)
         self.BCSR = self.BCSR or other.BCSR
         self.BCSC = self.BCSC or other.BCSC
         self.at_capacity = self.at_capacity or other.at_capacity
         kernel.ports[port_name] = self
+        if self.indexes is not None and formats != (self.BCSR, self.BCSC):
+            self._update_indexes()  # the index built so far lacks a format the new consumer reads
 
 
 class KernelBase(abc.ABC):

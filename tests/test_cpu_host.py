@@ -247,3 +247,56 @@ def test_search_space_filtering_by_fixed_params():
     assert OpenAISparseMatMulKernel(mode='dsd').get_search_space({'BLOCK_SIZE_K_VALUE': 32}) is None
     assert OpenAISparseMatMulKernel(mode='dsd').get_search_space({'BLOCK_SIZE_K_VALUE': 64}) is not None
     k.set_parameters({'_impl': 'sparta', '_name': 'x', 'THREAD_SIZE_M_VALUE': 4})  # tolerated keys
+
+
+# ---- tuned-config tables (the reference's test/bench/*/params/*.csv format) --------------
+def test_config_table_round_trip(tmp_path):
+    from sparta_amd.common import config_table as ct
+    cfg_a = {'forward:C': {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 32},
+             'backward:A': {'_impl': 'openai'}}
+    cfg_b = {'forward:C': {'_impl': 'openai', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 32,
+                           'TILE_CFG': 7}}
+    path = tmp_path / 'params' / 'default.csv'
+    ct.save_config_table(str(path), ['granularity', 'sparsity'],
+                         [({'granularity': 8, 'sparsity': 0.9}, cfg_a), ({'granularity': 32, 'sparsity': 0.95}, cfg_b)])
+    header = path.read_text().splitlines()[0].split(',')
+    assert header[:2] == ['granularity', 'sparsity'] and 'forward:C;_impl' in header and 'forward:C;TILE_CFG' in header
+    table = ct.load_config_table(str(path.parent), device_name='no such device')   # falls back to default.csv
+    assert ct.lookup_config(table, granularity=8, sparsity=0.9) == cfg_a             # absent TILE_CFG (0) is dropped
+    assert ct.lookup_config(table, granularity=32, sparsity=0.95) == cfg_b
+    with pytest.raises(KeyError):
+        ct.lookup_config(table, granularity=1, sparsity=0.5)
+    # a device-specific file wins over default.csv
+    ct.save_config_table(str(path.parent / 'My GPU.csv'), ['granularity', 'sparsity'],
+                         [({'granularity': 8, 'sparsity': 0.9}, cfg_b)])
+    table = ct.load_config_table(str(path.parent), device_name='My GPU')
+    assert ct.lookup_config(table, granularity=8, sparsity=0.9) == cfg_b
+    with pytest.raises(FileNotFoundError):
+        ct.load_config_table(str(tmp_path / 'nowhere'))
+
+
+def test_config_table_reads_reference_style_rows():
+    """A row laid out like the reference's default.csv: zeros mean 'not set', _impl is text."""
+    from sparta_amd.common import config_table as ct
+    row = {'granularity': '1', 'sparsity': '0.0', 'forward:C;BLOCK_SIZE_M_VALUE': '0', 'forward:C;BLOCK_SIZE_K_VALUE': '0',
+           'backward:A;BLOCK_SIZE_M_VALUE': '64', 'backward:A;BLOCK_SIZE_K_VALUE': '32.0',
+           'forward:C;_impl': 'openai', 'backward:A;_impl': 'sparta'}
+    assert ct.unflatten_config(row) == {'forward:C': {'_impl': 'openai'},
+                                        'backward:A': {'BLOCK_SIZE_M_VALUE': 64, 'BLOCK_SIZE_K_VALUE': 32, '_impl': 'sparta'}}
+
+
+@pytest.mark.parametrize('op,kernels', [('matmul', {'forward:C', 'backward:A', 'backward:B'}),
+                                        ('attention', {'qk/forward:C', 'sm/forward:y', 'out/forward:C', 'qk/backward:A',
+                                                       'qk/backward:B', 'sm/backward:x', 'out/backward:A', 'out/backward:B'})])
+def test_packaged_config_tables_cover_the_sweep(op, kernels):
+    """The tables shipped for gfx950 hold one buildable config per (granularity, sparsity)
+    point of the reference's sweeps (test/bench/matmul/matmul.py:16-17)."""
+    from sparta_amd.common import config_table as ct
+    table = ct.load_config_table(ct.packaged_table_dir(op), device_name='some other GPU')
+    for g in (1, 8, 32):
+        for s in (0, 0.2, 0.4, 0.6, 0.8, 0.9, 0.95, 0.99, 0.995, 0.999, 0.9995, 0.9999):
+            config = ct.lookup_config(table, granularity=g, sparsity=s)
+            assert set(config) == kernels
+            for params in config.values():
+                assert params['_impl'] in ('sparta', 'openai')
+                assert all(isinstance(v, int) and v > 0 for k, v in params.items() if k != '_impl')
