@@ -34,7 +34,7 @@ template <typename T> struct PanelMma {
 // wavefronts fetches a quarter - into a double-buffered shared LDS tile, at the price
 // of one workgroup barrier per step; otherwise every wavefront loads it privately.
 template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW>
-__global__ __launch_bounds__(256) void spmm_panel_kernel(SpmmParams p, int n_mtiles) {
+__global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_panel_kernel(SpmmParams p, int n_mtiles) {
     typedef typename PanelMma<T>::M MMA;
     typedef typename MMA::frag Frag;
     constexpr int KC = PanelMma<T>::KC;
