@@ -368,12 +368,190 @@ static int launch_dds_pipe_inst(const DdsParams& p, int nnz_bound, int batch, hi
     return 0;
 }
 
-// The pipelined kernel needs k-contiguous operands and K a multiple of its stage depth
-// (256 bytes of k per row; 128 bytes for 64 x 64 blocks).
+// ---- pipelined variant for operands stored the other way round ---------------------------
+// A is [K, M] and B is [K, N] (m / n contiguous): the layout of the weight gradient
+// grad_W = grad_y^T x.  Same register ring and two LDS buffers; a stage keeps KT k-rows
+// of the A and of the B panel as they are in memory ([k][m], [k][n]), and the
+// k-contiguous MFMA fragments come from the LDS transpose read of gfx950 for the 16-bit
+// types (lane i of a 16-lane group addresses 4 entries of k-row i/4, lane j receives
+// column j of the four rows) or from four 4-byte reads for fp32.
+template <typename T, int BM, int BN, int NST>
+__global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
+    constexpr int MT = BM / 16, NT = BN / 16;
+    typedef DdsWaveGrid<MT, NT> G;
+    constexpr int ES = (int)sizeof(T);
+    constexpr int VE = 16 / ES;
+    constexpr int KT = DdsPipeCfg<BM, BN>::STAGE_BYTES / ES;   // k-rows per stage
+    constexpr int KW = KT / G::KS;
+    constexpr int LDA = BM + VE, LDB = BN + VE;                // row pitches (elements)
+    constexpr int A_BYTES = KT * LDA * ES;
+    constexpr int BUF = KT * (LDA + LDB) * ES;
+    constexpr int CA = BM / VE, CB = BN / VE;                  // 16-byte chunks per k-row
+    constexpr int NA = KT * CA;                                // chunks of the A part
+    constexpr int NV = KT * (CA + CB) / 256;
+    static_assert(KT * (CA + CB) % 256 == 0, "stage does not split over the workgroup");
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    const int i = dds_block_of_workgroup<BM>(p);
+    if (i < 0) return;
+    const int code = p.idx[i];
+    const int bi = (code >> 16) & 0xffff;
+    const int bj = code & 0xffff;
+    const int64_t b = blockIdx.y;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15;
+    const int g4 = lane >> 4;
+    const int wt = wave % (G::WGM * G::WGN);
+    const int kpart = wave / (G::WGM * G::WGN);
+    const int wgm = wt / G::WGN;
+    const int wgn = wt % G::WGN;
+
+    const T* A = reinterpret_cast<const T*>(p.A) + b * p.a_batch + (int64_t)bi * BM;
+    const T* B = reinterpret_cast<const T*>(p.B) + b * p.b_batch + (int64_t)bj * BN;
+
+    // staging map: chunk v = tid + 256 u; the first NA chunks are (k-row, piece) of A, the rest of B
+    const T* src[NV];
+    int64_t sstep[NV];
+    int dst[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int v = threadIdx.x + 256 * u;
+        if (v < NA) {
+            const int k = v / CA, c = v % CA;
+            src[u] = A + (int64_t)k * p.a_ld + c * VE;
+            sstep[u] = (int64_t)KT * p.a_ld;
+            dst[u] = (k * LDA + c * VE) * ES;
+        } else {
+            const int w = v - NA;
+            const int k = w / CB, c = w % CB;
+            src[u] = B + (int64_t)k * p.b_ld + c * VE;
+            sstep[u] = (int64_t)KT * p.b_ld;
+            dst[u] = A_BYTES + (k * LDB + c * VE) * ES;
+        }
+    }
+
+    f32x4 acc[G::WTM][G::WTN];
+#pragma unroll
+    for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+        for (int y = 0; y < G::WTN; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int n_st = p.K / KT;
+    const int rot = (int)(((int64_t)(blockIdx.x & 7) * n_st) >> 3);  // XCDs start at staggered depths
+    u32x4 ring[NST][NV];
+#pragma unroll
+    for (int r = 0; r < NST; ++r) {
+        int st0 = (r < n_st ? r : n_st - 1) + rot;
+        st0 = st0 >= n_st ? st0 - n_st : st0;
+#pragma unroll
+        for (int u = 0; u < NV; ++u) ring[r][u] = *reinterpret_cast<const u32x4*>(src[u] + st0 * sstep[u]);
+    }
+    // fragment bases inside a buffer (bytes)
+    const int a_tr = ((g4 * 8 + (r16 >> 2)) * LDA + (wgm * G::WTM * 16 + (r16 & 3) * 4)) * ES;
+    const int b_tr = A_BYTES + ((g4 * 8 + (r16 >> 2)) * LDB + (wgn * G::WTN * 16 + (r16 & 3) * 4)) * ES;
+    const int a_f32 = ((g4 * 4) * LDA + wgm * G::WTM * 16 + r16) * ES;
+    const int b_f32 = A_BYTES + ((g4 * 4) * LDB + wgn * G::WTN * 16 + r16) * ES;
+    for (int it = 0; it < n_st; it += NST) {
+#pragma unroll
+        for (int r = 0; r < NST; ++r) {
+            const int s = it + r;
+            char* buf = smem + (s & 1) * BUF;
+            if (s < n_st) {
+#pragma unroll
+                for (int u = 0; u < NV; ++u) *reinterpret_cast<u32x4*>(buf + dst[u]) = ring[r][u];
+            }
+            {   // refill the slot NST stages ahead (clamped: the extra copies are never used)
+                int st1 = (s + NST < n_st ? s + NST : n_st - 1) + rot;
+                st1 = st1 >= n_st ? st1 - n_st : st1;
+#pragma unroll
+                for (int u = 0; u < NV; ++u) ring[r][u] = *reinterpret_cast<const u32x4*>(src[u] + st1 * sstep[u]);
+            }
+            if (s < n_st) {
+                __syncthreads();
+                if constexpr (HasMma32<T>::value) {
+                    typedef typename Mma32<T>::frag Frag;
+#pragma unroll
+                    for (int kc = 0; kc < KW; kc += 32) {
+                        const int kb = kpart * KW + kc;
+                        Frag af[G::WTM], bf[G::WTN];
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x) {
+                            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + a_tr + (kb * LDA + x * 16) * ES));
+                            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + a_tr + ((kb + 4) * LDA + x * 16) * ES));
+                            af[x] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                        }
+#pragma unroll
+                        for (int y = 0; y < G::WTN; ++y) {
+                            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + b_tr + (kb * LDB + y * 16) * ES));
+                            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + b_tr + ((kb + 4) * LDB + y * 16) * ES));
+                            bf[y] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                        }
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                            for (int y = 0; y < G::WTN; ++y) acc[x][y] = Mma32<T>::mma(af[x], bf[y], acc[x][y]);
+                    }
+                } else {
+#pragma unroll
+                    for (int kc = 0; kc < KW; kc += 16) {
+                        const int kb = kpart * KW + kc;
+                        typename Mma16<T>::frag af[G::WTM], bf[G::WTN];
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                af[x][j] = *reinterpret_cast<const float*>(buf + a_f32 + ((kb + j) * LDA + x * 16) * ES);
+#pragma unroll
+                        for (int y = 0; y < G::WTN; ++y)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                bf[y][j] = *reinterpret_cast<const float*>(buf + b_f32 + ((kb + j) * LDB + y * 16) * ES);
+#pragma unroll
+                        for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                            for (int y = 0; y < G::WTN; ++y) acc[x][y] = Mma16<T>::mma(af[x], bf[y], acc[x][y]);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();  // all fragments are consumed before the buffers are reused
+    dds_epilogue<T, BM, BN>(p, acc, reinterpret_cast<float*>(smem), i, bi, bj, b, wgm, wgn, kpart, r16, g4);
+}
+
+template <typename T, int BM, int BN>
+static int launch_dds_pipe_t_inst(const DdsParams& p, int nnz_bound, int batch, hipStream_t st) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int KT = DdsPipeCfg<BM, BN>::STAGE_BYTES / (int)sizeof(T);
+    constexpr int NST = DdsPipeCfg<BM, BN>::NST;
+    typedef DdsWaveGrid<BM / 16, BN / 16> G;
+    size_t smem = 2 * (size_t)KT * (BM + BN + 2 * VE) * sizeof(T);
+    size_t epi = (size_t)G::KS * BM * (BN + 4) * sizeof(float);
+    if (epi > smem) smem = epi;
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_pipe_t_kernel<T, BM, BN, NST>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(dds_pipe_t_kernel)");
+    }
+    hipLaunchKernelGGL((dds_pipe_t_kernel<T, BM, BN, NST>), dim3(nnz_bound, batch, 1), dim3(256), smem, st, p);
+    SPX_LAUNCH_CHECK("dds_pipe_t_kernel");
+    return 0;
+}
+
+// The pipelined kernels need both operands stored the same way round (both k-contiguous,
+// or A as [K, M] and B as [K, N]) and K a multiple of the stage depth (256 bytes of k per
+// row; 128 bytes for 64 x 64 blocks).  Returns 0 (no), 1 (k-contiguous) or 2.
 template <typename T>
-static bool dds_pipe_ok(const DdsParams& p, int BM, int BN) {
+static int dds_pipe_ok(const DdsParams& p, int BM, int BN) {
     const int stage = (BM + BN == 128 ? 128 : 256) / (int)sizeof(T);
-    return p.a_kcontig && p.b_kcontig && p.K % stage == 0;
+    if (p.K % stage != 0) return 0;
+    if (p.a_kcontig && p.b_kcontig) return 1;
+    if (!p.a_kcontig && !p.b_kcontig) return 2;
+    return 0;
 }
 
 template <typename T, int BM, int BN>
@@ -394,13 +572,15 @@ static int launch_dds_inst(const DdsParams& p, int nnz_bound, int batch, hipStre
 template <typename T>
 int launch_dds_impl(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, int tile_cfg, hipStream_t st) {
     if (tile_cfg < 0 || tile_cfg > 2) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
-    if (tile_cfg == 0) tile_cfg = dds_pipe_ok<T>(p, BM, BN) ? 2 : 1;
-    if (tile_cfg == 2 && !dds_pipe_ok<T>(p, BM, BN))
-        return fail(SPX_E_CONFIG, "tile config 2 needs k-contiguous operands and K a multiple of the stage depth");
+    const int pipe = dds_pipe_ok<T>(p, BM, BN);
+    if (tile_cfg == 0) tile_cfg = pipe ? 2 : 1;
+    if (tile_cfg == 2 && !pipe)
+        return fail(SPX_E_CONFIG, "tile config 2 needs both operands stored the same way round and K a multiple of the stage depth");
 #define SPX_DDS_CASE(bm, bn) \
     if (BM == bm && BN == bn) \
-        return tile_cfg == 2 ? launch_dds_pipe_inst<T, bm, bn>(p, nnz_bound, batch, st) \
-                             : launch_dds_inst<T, bm, bn>(p, nnz_bound, batch, st);
+        return tile_cfg != 2 ? launch_dds_inst<T, bm, bn>(p, nnz_bound, batch, st) \
+             : pipe == 1 ? launch_dds_pipe_inst<T, bm, bn>(p, nnz_bound, batch, st) \
+                         : launch_dds_pipe_t_inst<T, bm, bn>(p, nnz_bound, batch, st);
     SPX_DDS_CASE(16, 16) SPX_DDS_CASE(16, 32) SPX_DDS_CASE(16, 64)
     SPX_DDS_CASE(32, 16) SPX_DDS_CASE(32, 32) SPX_DDS_CASE(32, 64)
     SPX_DDS_CASE(64, 16) SPX_DDS_CASE(64, 32) SPX_DDS_CASE(64, 64)

@@ -118,10 +118,12 @@ def test_matmul_tile_configs(tile_cfg, mode, compressed, dtype, blocks, gpu):
                                           (torch.float32, (16, 32, 16)), (torch.float16, (16, 32, 64)),
                                           (torch.float32, (64, 32, 32)), (torch.float16, (64, 32, 16)),
                                           (torch.float32, (32, 32, 32))])
-def test_matmul_dds_tile_configs(tile_cfg, K, dtype, blocks, gpu):
-    """Both sparse-output kernels (single-buffer and pipelined) on k-contiguous operands:
-    stage counts below, equal to and above the depth of the register ring."""
-    run_case(gpu, 'dds', False, True, True, True, dtype, blocks, batch=2, M=192, K=K, N=256,
+@pytest.mark.parametrize('tA,tB', [(False, True), (True, False)])
+def test_matmul_dds_tile_configs(tile_cfg, K, dtype, blocks, tA, tB, gpu):
+    """Both sparse-output kernels (single-buffer and pipelined) on operands stored the same
+    way round (k-contiguous, or [K, M] / [K, N] as in a weight gradient): stage counts
+    below, equal to and above the depth of the register ring."""
+    run_case(gpu, 'dds', tA, tB, True, True, dtype, blocks, batch=2, M=192, K=K, N=256,
              gran=(16, 16), sparsity=0.7, seed=5, tile_cfg=tile_cfg)
 
 
