@@ -221,7 +221,9 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
     const bool kcontig = p.d_kcontig && p.s_kcontig;
     const bool panel_ok = kcontig && (p.BK * (int)sizeof(T)) % 64 == 0;
     // the shared-S panel variant transposes an n-contiguous sparse block while staging it
-    const bool panel7_ok = p.d_kcontig && (p.BK * (int)sizeof(T)) % 64 == 0;
+    // ... and reads a dense operand stored with m contiguous through LDS transpose reads
+    const bool panel7_ok = (p.BK * (int)sizeof(T)) % 64 == 0 &&
+                           (p.d_kcontig || (p.Mc % (16 / (int)sizeof(T)) == 0 && p.d_ld % (16 / (int)sizeof(T)) == 0));
     if (tile_cfg < 0 || tile_cfg > 7) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg == 0) {
         // 256-row tiles only when they still give every CU a few workgroups; small

@@ -30,10 +30,35 @@ template <typename T> struct PanelMma {
     static constexpr int KC = 64 / (int)sizeof(T);  // k per step
 };
 
+// One MFMA fragment of the dense operand from the private LDS region: a plain 16-byte
+// read of the [row][k] layout, or - for an operand kept as [k][m] - two transpose reads
+// (16-bit: four k-rows each, 4 k-rows apart) / four 4-byte reads one k-row apart (fp32).
+template <typename T, bool DT, typename Frag>
+__device__ __forceinline__ Frag panel_dfrag(const char* at) {
+    if constexpr (!DT) {
+        return *reinterpret_cast<const Frag*>(at);
+    } else if constexpr (sizeof(T) == 2) {
+        typedef short s16x8_t __attribute__((ext_vector_type(8)));
+        typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at + 4 * 128));
+        return __builtin_bit_cast(Frag, (s16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    } else {
+        Frag f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) f[j] = *reinterpret_cast<const float*>(at + j * 256);
+        return f;
+    }
+}
+
 // SHW: the S (sparse) block of a step is loaded once per workgroup - each of the four
 // wavefronts fetches a quarter - into a double-buffered shared LDS tile, at the price
 // of one workgroup barrier per step; otherwise every wavefront loads it privately.
-template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW>
+// DT: the dense operand is stored with m contiguous (D[k * d_ld + m]).  A step then loads
+// KC k-rows of 64 contiguous m per wavefront (fully coalesced), keeps them as [k][m] in
+// the private LDS region and builds the k-contiguous MFMA fragments with the LDS transpose
+// read of gfx950 (16-bit types) or 4-byte reads (fp32).
+template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW, bool DT = false>
 __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_panel_kernel(SpmmParams p, int n_mtiles) {
     typedef typename PanelMma<T>::M MMA;
     typedef typename MMA::frag Frag;
@@ -74,13 +99,33 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
     const int lchk = lane & 3;
     const T* dptr[4];
     int wofs[4];  // LDS byte offsets of this lane's chunk for the 4 row groups of D
+    constexpr int DT_CPR = 64 / E16;        // DT: 16-byte pieces per k-row of 64 m (8 or 16)
+    constexpr int DT_RPL = 64 / DT_CPR;     // DT: k-rows covered by one wave load (8 or 4)
+    constexpr int DT_PITCH = 64 * (int)sizeof(T);  // DT: bytes per k-row in LDS
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const int row = q * 16 + lrow;
-        int m = m0 + row;
-        if (m >= p.Mc) m = p.Mc - 1;  // rows past the end re-read the last row; never stored
-        dptr[q] = D + (int64_t)m * p.d_ld + lchk * E16;
-        wofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
+        if constexpr (DT) {
+            // lane -> (k-row lane / DT_CPR + DT_RPL q of the step, piece lane % DT_CPR of its 64 m)
+            const int kr = lane / DT_CPR + DT_RPL * q;
+            const int pc = lane % DT_CPR;
+            int m = m0 + pc * E16;
+            if (m >= p.Mc) m = 0;  // columns past the end re-read valid data; never stored
+            dptr[q] = D + (int64_t)kr * p.d_ld + m;
+            if constexpr (sizeof(T) == 2) {
+                // 32-byte units (16 m) XOR-swizzled by bits 1 and 3 of the k-row
+                const int f = ((kr >> 1) & 1) | (((kr >> 3) & 1) << 1);
+                wofs[q] = kr * DT_PITCH + ((((pc >> 1) ^ f) & 3) << 5) + ((pc & 1) << 4);
+            } else {
+                // 64-byte units (16 m) XOR-swizzled by bits 2..3 of the k-row
+                wofs[q] = kr * DT_PITCH + ((((pc >> 2) ^ (kr >> 2)) & 3) << 6) + ((pc & 3) << 4);
+            }
+        } else {
+            const int row = q * 16 + lrow;
+            int m = m0 + row;
+            if (m >= p.Mc) m = p.Mc - 1;  // rows past the end re-read the last row; never stored
+            dptr[q] = D + (int64_t)m * p.d_ld + lchk * E16;
+            wofs[q] = row * 64 + ((lchk ^ ((row >> 2) & 3)) << 4);
+        }
     }
     int sofs[WL];
     // shared S tile: this wave stages chunks wave*BN .. wave*BN+BN-1 of the BN*4 chunks.
@@ -104,8 +149,18 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
     int aofs[4], bofs[NT];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int row = i * 16 + r16;
-        aofs[i] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
+        if constexpr (DT && sizeof(T) == 2) {
+            // transpose read: this lane addresses k-row g4*8 + r16/4 (and +4), m = i*16 + (r16%4)*4
+            const int kr = g4 * 8 + (r16 >> 2);
+            const int f = ((kr >> 1) & 1) | (((kr >> 3) & 1) << 1);
+            aofs[i] = kr * DT_PITCH + (((i ^ f) & 3) << 5) + ((r16 & 3) << 3);
+        } else if constexpr (DT) {
+            // fp32: element (k = g4*4 + j, m = i*16 + r16); j adds DT_PITCH
+            aofs[i] = (g4 * 4) * DT_PITCH + (((i ^ g4) & 3) << 6) + (r16 << 2);
+        } else {
+            const int row = i * 16 + r16;
+            aofs[i] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
+        }
     }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -166,7 +221,7 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
                                       : (p.s_kcontig ? S + (int64_t)j * BN * p.s_ld + koff_        \
                                                      : S + (int64_t)koff_ * p.s_ld + (int64_t)j * BN); \
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
-            DREG[q] = *reinterpret_cast<const u32x4*>(dptr[q] + koff_);                            \
+            DREG[q] = *reinterpret_cast<const u32x4*>(dptr[q] + (DT ? (int64_t)koff_ * p.d_ld : (int64_t)koff_)); \
         if constexpr (SHW) {                                                                       \
             if (sh_active)                                                                         \
                 SREG[0] = *reinterpret_cast<const u32x4*>(sblk_ + sh_toff);                        \
@@ -211,7 +266,7 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
         if ((IT) < n_it) {                                                                         \
             Frag af_[4], bf_[NT];                                                                  \
             _Pragma("unroll") for (int i = 0; i < 4; ++i)                                          \
-                af_[i] = *reinterpret_cast<const Frag*>(lds + aofs[i]);                            \
+                af_[i] = panel_dfrag<T, DT, Frag>(lds + aofs[i]);                                  \
             _Pragma("unroll") for (int t = 0; t < NT; ++t)                                         \
                 bf_[t] = *reinterpret_cast<const Frag*>(sdst_ + bofs[t]);                          \
             _Pragma("unroll") for (int i = 0; i < 4; ++i)                                          \
@@ -305,14 +360,14 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
     }
 }
 
-template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW>
+template <typename T, int BN, int BK, int NST, bool SWAP, bool SHW, bool DT = false>
 static int launch_spmm_panel_inst(const SpmmParams& p, int batch, hipStream_t st) {
     const int n_mtiles = (p.Mc + 255) / 256;
     const int nb = p.Nc / BN;
     const int64_t groups = (n_mtiles + kPanelXcd - 1) / kPanelXcd;
     const int64_t nblocks = groups * kPanelXcd * nb;
     if (nblocks > 0x7fffffffLL) return fail(SPX_E_SHAPE, "problem too large for one launch");
-    hipLaunchKernelGGL((spmm_panel_kernel<T, BN, BK, NST, SWAP, SHW>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st,
+    hipLaunchKernelGGL((spmm_panel_kernel<T, BN, BK, NST, SWAP, SHW, DT>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st,
                        p, n_mtiles);
     SPX_LAUNCH_CHECK("spmm_panel_kernel");
     return 0;
@@ -325,14 +380,14 @@ bool spmm_panel_supported(int BN, int BK) {
     return BK % kc == 0 && (BN == 16 || BN == 32 || BN == 64);
 }
 
-template <typename T, int NST, bool SHW>
+template <typename T, int NST, bool SHW, bool DT = false>
 int launch_spmm_panel_impl(const SpmmParams& p, int BN, int batch, hipStream_t st) {
     const bool swap = p.out_ncontig != 0;
 #define SPX_PANEL_CASE(bn, bk)                                                                  \
     if (BN == bn && p.BK == bk) {                                                               \
         if constexpr (bk % (64 / (int)sizeof(T)) == 0) {                                        \
-            return swap ? launch_spmm_panel_inst<T, bn, bk, NST, true, SHW>(p, batch, st)       \
-                        : launch_spmm_panel_inst<T, bn, bk, NST, false, SHW>(p, batch, st);     \
+            return swap ? launch_spmm_panel_inst<T, bn, bk, NST, true, SHW, DT>(p, batch, st)   \
+                        : launch_spmm_panel_inst<T, bn, bk, NST, false, SHW, DT>(p, batch, st); \
         }                                                                                       \
     }
     SPX_PANEL_CASE(16, 16) SPX_PANEL_CASE(16, 32) SPX_PANEL_CASE(16, 64)

@@ -129,14 +129,16 @@ def test_matmul_dds_tile_configs(tile_cfg, K, dtype, blocks, tA, tB, gpu):
 
 @pytest.mark.parametrize('tile_cfg', [0, 7])
 @pytest.mark.parametrize('compressed', [False, True])
-@pytest.mark.parametrize('mode,tA,tB', [('dsd', False, False), ('sdd', True, True)])
+@pytest.mark.parametrize('mode,tA,tB', [('dsd', False, False), ('sdd', True, True), ('dsd', True, True), ('dsd', True, False),
+                                        ('sdd', False, False), ('sdd', True, False)])
 @pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 64, 16)),
                                           (torch.float32, (16, 32, 64)), (torch.float16, (16, 64, 64))])
 def test_matmul_panel_with_transposed_sparse_operand(tile_cfg, compressed, mode, tA, tB, dtype, blocks, gpu):
-    """Dense operand k-contiguous, sparse operand stored the other way round (the layouts
-    of SparseLinear's input gradient): large enough for the panel kernel to be chosen."""
+    """Every storage order of the two operands other than the all-k-contiguous one (the
+    layouts of the backward kernels and of products with a [K, N] matrix), large and
+    ragged enough for the panel kernel to be chosen and to clamp its last tile."""
     run_case(gpu, mode, tA, tB, True, compressed, dtype, blocks, batch=2,
-             M=1088 if mode == 'dsd' else 128, K=128, N=128 if mode == 'dsd' else 1088, gran=(16, 16),
+             M=1096 if mode == 'dsd' else 128, K=128, N=128 if mode == 'dsd' else 1096, gran=(16, 16),
              sparsity=0.6, seed=13, tile_cfg=tile_cfg)
 
 
