@@ -166,7 +166,7 @@ def main():
     ap.add_argument('--tune', type=int, default=0, help='tune every point with this many trials per kernel')
     ap.add_argument('--warmups', type=int, default=20)
     ap.add_argument('--iters', type=int, default=50)
-    ap.add_argument('--out', default=os.path.join(ROOT, 'gpurun_out'))
+    ap.add_argument('--out', default=os.path.join(ROOT, 'sweep_out'), help='directory for the result CSVs')
     args = ap.parse_args()
 
     import torch
