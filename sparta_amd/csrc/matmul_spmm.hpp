@@ -208,12 +208,16 @@ template <typename T>
 int launch_spmm_direct(const SpmmParams& p, int BN, int batch, int wm, hipStream_t st);
 template <typename T>
 int launch_spmm_panel(const SpmmParams& p, int BN, int batch, int nst, hipStream_t st);
+template <typename T>
+int launch_spmm_ksplit(const SpmmParams& p, int BN, int batch, hipStream_t st);
 
 // tile_cfg: 0 = pick by layout and size;
 //   1 / 2  LDS-staged kernel, 64 / 128-row workgroup tiles (any layout);
 //   3 / 4  register-direct kernel, 64 / 256-row workgroup tiles (k-contiguous operands);
 //   5 / 6  panel kernel, 256-row workgroup tiles, 2 / 3 load stages (k-contiguous
 //          operands, block depth a multiple of 64 bytes);
+//   8      K-split panel kernel: 64-row workgroup tiles, the four wavefronts split the
+//          live blocks of a block-column (k-contiguous operands, BN <= 32): few rows.
 //   7      panel kernel whose four wavefronts share the sparse block through LDS (the
 //          sparse operand may be stored with n contiguous: it is transposed on the way).
 template <typename T>
@@ -224,16 +228,22 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
     // ... and reads a dense operand stored with m contiguous through LDS transpose reads
     const bool panel7_ok = (p.BK * (int)sizeof(T)) % 64 == 0 &&
                            (p.d_kcontig || (p.Mc % (16 / (int)sizeof(T)) == 0 && p.d_ld % (16 / (int)sizeof(T)) == 0));
-    if (tile_cfg < 0 || tile_cfg > 7) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    if (tile_cfg < 0 || tile_cfg > 8) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    const bool ksplit_ok = panel_ok && BN <= 32;
     if (tile_cfg == 0) {
         // 256-row tiles only when they still give every CU a few workgroups; small
         // problems are latency-bound and want more, shorter workgroups.
         const int64_t big_tiles = (int64_t)((p.Mc + 255) / 256) * (p.Nc / BN) * batch;
         const bool fill = big_tiles >= 512;
         if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
+        else if (ksplit_ok && !fill && p.K / p.BK >= 8) tile_cfg = 8;  // few tiles, long block-columns
         else if (panel7_ok && p.Mc >= 512 && fill) tile_cfg = 7;
         else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
         else tile_cfg = p.Mc >= 1024 && fill ? 2 : 1;
+    }
+    if (tile_cfg == 8) {
+        if (!ksplit_ok) return fail(SPX_E_CONFIG, "tile config 8 needs k-contiguous operands, 64-byte block rows and BN <= 32");
+        return launch_spmm_ksplit<T>(p, BN, batch, st);
     }
     if (tile_cfg >= 5) {
         if (!(tile_cfg == 7 ? panel7_ok : panel_ok))

@@ -18,6 +18,7 @@ static const spx_tile_cfg kSpmmCfgs[] = {
     {5, 256, 0, 4, 2, 16, 7, "panel-256x2"},
     {6, 256, 0, 4, 3, 16, 7, "panel-256x3"},
     {7, 256, 0, 4, 2, 16, 7, "panel-256-sharedS"},
+    {8, 64, 0, 4, 2, 16, 7, "panel-64-ksplit"},
 };
 static const spx_tile_cfg kDdsCfgs[] = {
     {0, 0, 0, 4, 1, 16, 7, "auto"},

@@ -98,7 +98,7 @@ def test_matmul_block_shapes(blocks, mode, gpu):
              batch=2, M=192, K=128, N=256, gran=(16, 16), sparsity=0.8, seed=k)
 
 
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize('mode', ['sdd', 'dsd'])
 @pytest.mark.parametrize('compressed', [False, True])
 @pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 64, 32)),
@@ -107,6 +107,8 @@ def test_matmul_block_shapes(blocks, mode, gpu):
 def test_matmul_tile_configs(tile_cfg, mode, compressed, dtype, blocks, gpu):
     """Every kernel family behind TILE_CFG gives the same masked-dense result
     (k-contiguous layout, which all of them accept); M is ragged on purpose."""
+    if tile_cfg == 8 and (blocks[2] if mode == 'dsd' else blocks[0]) > 32:
+        pytest.skip('the K-split kernel covers sparse-side block widths up to 32')
     run_case(gpu, mode, False, True, True, compressed, dtype, blocks, batch=2,
              M=320 if mode == 'dsd' else 192, K=256, N=192 if mode == 'dsd' else 328, gran=(16, 16),
              sparsity=0.7, seed=11, tile_cfg=tile_cfg)
