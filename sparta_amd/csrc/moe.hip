@@ -503,7 +503,7 @@ __global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
 // 32 MFMAs), K-stage s+1 sits in the second LDS buffer and stage s+2 is in flight in
 // registers while stage s feeds the matrix cores; one barrier per stage.
 template <typename T, int TM, int TN, int WAVES, int WGM>
-__global__ __launch_bounds__(64 * WAVES, 1) void moe_gemm_kernel_v4(MoeParams p) {
+__global__ __launch_bounds__(64 * WAVES, (TM + TN) > 256 ? 1 : 2) void moe_gemm_kernel_v4(MoeParams p) {
     constexpr int NTH = 64 * WAVES;
     constexpr int WGN = WAVES / WGM;
     constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
@@ -685,16 +685,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void moe_gemm_kernel_v4(MoeParams p)
     }
 }
 
-template <typename T>
+template <typename T, int TM, int TN, int WAVES>
 static int launch_moe_v4(const MoeParams& p, hipStream_t st) {
-    constexpr int TM = 256, TN = 256;
     const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp;
     if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
     const int smem = 2 * (TM + TN) * 128;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel_v4<T, TM, TN, 8, 2>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel_v4<T, TM, TN, WAVES, 2>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_kernel_v4)");
-    hipLaunchKernelGGL((moe_gemm_kernel_v4<T, TM, TN, 8, 2>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(512), smem, st, p);
+    hipLaunchKernelGGL((moe_gemm_kernel_v4<T, TM, TN, WAVES, 2>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
     SPX_LAUNCH_CHECK("moe_gemm_kernel_v4");
     return 0;
 }
@@ -744,7 +743,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -764,13 +763,21 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     // 2: 256x128 tiles, 3: 128x128 tiles, both with the next K stage prefetched into
     // registers; 4: 256x256 tiles with two LDS buffers (2..4: k-contiguous weights only).
     if (tile_cfg == 0) tile_cfg = 1;  // measured best on the benchmark shapes; the others stay selectable
-    if (tile_cfg == 4) {
-        // 256x256 tiles, eight wavefronts, two LDS buffers (k-contiguous weights only)
+    if (tile_cfg == 4 || tile_cfg == 5) {
+        // two LDS buffers, one barrier per stage (k-contiguous weights only):
+        // 4: 256x256 tiles, eight wavefronts; 5: 128x128 tiles, four wavefronts, two workgroups per CU
         SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
+        if (tile_cfg == 4) {
+            switch (dtype) {
+                case SPX_F32: return launch_moe_v4<float, 256, 256, 8>(p, st);
+                case SPX_F16: return launch_moe_v4<_Float16, 256, 256, 8>(p, st);
+                default: return launch_moe_v4<bf16_t, 256, 256, 8>(p, st);
+            }
+        }
         switch (dtype) {
-            case SPX_F32: return launch_moe_v4<float>(p, st);
-            case SPX_F16: return launch_moe_v4<_Float16>(p, st);
-            default: return launch_moe_v4<bf16_t>(p, st);
+            case SPX_F32: return launch_moe_v4<float, 128, 128, 4>(p, st);
+            case SPX_F16: return launch_moe_v4<_Float16, 128, 128, 4>(p, st);
+            default: return launch_moe_v4<bf16_t, 128, 128, 4>(p, st);
         }
     }
     if (tile_cfg >= 2) {

@@ -42,6 +42,7 @@ static const spx_tile_cfg kMoeCfgs[] = {
     {2, 256, 128, 4, 2, 0, 7, "gather-256x128-prefetch"},
     {3, 128, 128, 4, 2, 0, 7, "gather-128x128-prefetch"},
     {4, 256, 256, 8, 3, 0, 7, "gather-256x256-two-buffers"},
+    {5, 128, 128, 4, 3, 0, 7, "gather-128x128-two-buffers"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {
