@@ -302,6 +302,39 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
 
     // ---- scatter the rows back: lane holds out[m = i*16 + r16][n = t*16 + g4*4 .. +3] -----
     T* out = reinterpret_cast<T*>(p.out);
+    if constexpr (sizeof(T) == 2) {
+        // 16-bit outputs leave through LDS (free after the last barrier): the wavefront's
+        // 64 x 64 tile is laid out as 64 rows of 128 bytes (chunks XOR-swizzled by the
+        // row), then every store instruction writes eight complete 128-byte row segments
+        // instead of sixteen 32-byte pieces.
+        char* ep = smem + wave * (64 * 128);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                T vals[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
+                const int row = i * 16 + r16;
+                const int chunk = t * 2 + (g4 >> 1);
+                *reinterpret_cast<uint64_t*>(ep + row * 128 + ((chunk ^ (row & 7)) << 4) + (g4 & 1) * 8) =
+                    *reinterpret_cast<const uint64_t*>(vals);
+            }
+        // LDS operations of one wavefront complete in order: no barrier needed
+        const int c = lane & 7;
+        const int n = n0 + wn * 64 + c * 8;
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass) {
+            const int row = pass * 8 + (lane >> 3);
+            const int r = wm * 64 + row;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * 128 + ((c ^ (row & 7)) << 4));
+            if (r < rows && n < p.N) {
+                const int tok = p.token_perm[row0 + r];
+                *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int r = wm * 64 + i * 16 + r16;
@@ -333,16 +366,17 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
 
 // TM x TN: workgroup tile; WGM: wavefronts along the token dimension (4 / WGM along the
 // output dimension); OCC: workgroups per CU the register budget is sized for.
-template <typename T, int TM, int TN, int WGM, int OCC>
-__global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
+template <typename T, int TM, int TN, int WGM, int OCC, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES, OCC) void moe_gemm_kernel_v2(MoeParams p) {
     constexpr int MOE2_TM = TM, MOE2_TN = TN;
-    constexpr int WGN = 4 / WGM;
+    constexpr int WGN = WAVES / WGM;
     constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
     constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
     constexpr int VE = 16 / (int)sizeof(T);
     constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
-    constexpr int A_LOADS = MOE2_TM * 8 / 256;  // 8
-    constexpr int B_LOADS = MOE2_TN * 8 / 256;  // 4
+    constexpr int A_LOADS = MOE2_TM * 8 / (64 * WAVES);
+    constexpr int B_LOADS = MOE2_TN * 8 / (64 * WAVES);
+    constexpr int RSTEP2 = 8 * WAVES;   // tile rows between a thread's vectors
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     __shared__ __align__(16) char As[MOE2_TM * 128];
     __shared__ __align__(16) char Bs[MOE2_TN * 128];
@@ -398,7 +432,7 @@ __global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
     int a_dst[A_LOADS];
 #pragma unroll
     for (int q = 0; q < A_LOADS; ++q) {
-        const int r = srow + 32 * q;
+        const int r = srow + RSTEP2 * q;
         const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
         a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
         a_dst[q] = moe_lds_off<T>(r, chunk);
@@ -407,7 +441,7 @@ __global__ __launch_bounds__(256, OCC) void moe_gemm_kernel_v2(MoeParams p) {
     int b_dst[B_LOADS];
 #pragma unroll
     for (int q = 0; q < B_LOADS; ++q) {
-        const int r = srow + 32 * q;
+        const int r = srow + RSTEP2 * q;
         const int n = n0 + r < p.N ? n0 + r : p.N - 1;
         b_src[q] = W + (int64_t)n * p.K + chunk * VE;
         b_dst[q] = moe_lds_off<T>(r, chunk);
@@ -743,7 +777,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 6, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -788,6 +822,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
         dim3 grid2((out_dim + 127) / 128, tiles2, 1);
 #define SPX_MOE2(T)                                                                                   \
         if (tile_cfg == 2) hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 256, 128, 4, 2>), grid2, dim3(256), 0, st, p); \
+        else if (tile_cfg == 6) hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 128, 128, 2, 2, 8>), grid2, dim3(512), 0, st, p); \
         else hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 128, 128, 2, 3>), grid2, dim3(256), 0, st, p);
         switch (dtype) {
             case SPX_F32: SPX_MOE2(float) break;
