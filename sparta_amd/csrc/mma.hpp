@@ -55,6 +55,24 @@ template <> struct Mma32<bf16_t> {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
 };
+// 32 x 32 x 16 MFMA (2-byte types): lane l holds k = (l/32)*8 .. +7 of row (column) l % 32
+// of the A (B) operand; accumulator register j of lane l is D[8*(j/4) + 4*(l/32) + j%4][l % 32].
+// On gfx950 this shape sustains about twice the FLOP rate of the 16 x 16 x 32 one (both
+// issue every ~32 cycles per SIMD), so MFMA-bound loops should be built from it.
+template <typename T> struct MmaW;
+template <> struct MmaW<_Float16> {
+    typedef f16x8 frag;
+    __device__ static f32x16 mma(frag a, frag b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct MmaW<bf16_t> {
+    typedef bf16x8 frag;
+    __device__ static f32x16 mma(frag a, frag b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
 template <typename T> struct HasMma32 { static constexpr bool value = true; };
 template <> struct HasMma32<float> { static constexpr bool value = false; };
 

@@ -219,11 +219,21 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
         a_tok[q] = p.token_perm[row0 + (r < rows ? r : rows - 1)];
     }
 
-    f32x4 acc[4][4];
+    // 2-byte types: 2 x 2 tiles of 32 x 32 (accw); fp32: 4 x 4 tiles of 16 x 16 (acc)
+    constexpr bool WIDE = HasMma32<T>::value;
+    f32x4 acc[WIDE ? 1 : 4][WIDE ? 1 : 4];
+    f32x16 accw[WIDE ? 2 : 1][WIDE ? 2 : 1];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < (WIDE ? 1 : 4); ++i)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < (WIDE ? 1 : 4); ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < (WIDE ? 2 : 1); ++i)
+#pragma unroll
+        for (int t = 0; t < (WIDE ? 2 : 1); ++t)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) accw[i][t][j] = 0.f;
+    const int l32 = lane & 31, h2 = lane >> 5;
 
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     for (int k0 = 0; k0 < p.K; k0 += MOE_KT) {
@@ -266,20 +276,20 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
         }
         __syncthreads();
         // ---- MFMA over the stage -----------------------------------------------------------
-        if constexpr (HasMma32<T>::value) {
+        if constexpr (WIDE) {
 #pragma unroll
-            for (int kc = 0; kc < MOE_KT; kc += 32) {
-                typename Mma32<T>::frag af[4], bf[4];
+            for (int kc = 0; kc < MOE_KT; kc += 16) {
+                typename MmaW<T>::frag af[2], bf[2];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    af[i] = *reinterpret_cast<const typename Mma32<T>::frag*>(As + moe_lds_off<T>(wm * 64 + i * 16 + r16, kc / VE + g4));
+                for (int i = 0; i < 2; ++i)
+                    af[i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + moe_lds_off<T>(wm * 64 + i * 32 + l32, kc / VE + h2));
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    bf[t] = *reinterpret_cast<const typename Mma32<T>::frag*>(Bs + moe_lds_off<T>(wn * 64 + t * 16 + r16, kc / VE + g4));
+                for (int t = 0; t < 2; ++t)
+                    bf[t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + moe_lds_off<T>(wn * 64 + t * 32 + l32, kc / VE + h2));
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < 2; ++i)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[i][t] = Mma32<T>::mma(bf[t], af[i], acc[i][t]);
+                    for (int t = 0; t < 2; ++t) accw[i][t] = MmaW<T>::mma(bf[t], af[i], accw[i][t]);
             }
         } else {
 #pragma unroll
@@ -300,26 +310,29 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
         __syncthreads();
     }
 
-    // ---- scatter the rows back: lane holds out[m = i*16 + r16][n = t*16 + g4*4 .. +3] -----
+    // ---- scatter the rows back (fp32: lane holds out[m = i*16 + r16][n = t*16 + g4*4 .. +3]) ----
     T* out = reinterpret_cast<T*>(p.out);
     if constexpr (sizeof(T) == 2) {
         // 16-bit outputs leave through LDS (free after the last barrier): the wavefront's
         // 64 x 64 tile is laid out as 64 rows of 128 bytes (chunks XOR-swizzled by the
         // row), then every store instruction writes eight complete 128-byte row segments
         // instead of sixteen 32-byte pieces.
+        // lane holds out[m = i*32 + lane%32][n = t*32 + 8*jj + 4*(lane/32) + q] in accw[i][t][4*jj + q]
         char* ep = smem + wave * (64 * 128);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                T vals[4];
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
-                const int row = i * 16 + r16;
-                const int chunk = t * 2 + (g4 >> 1);
-                *reinterpret_cast<uint64_t*>(ep + row * 128 + ((chunk ^ (row & 7)) << 4) + (g4 & 1) * 8) =
-                    *reinterpret_cast<const uint64_t*>(vals);
-            }
+                for (int jj = 0; jj < 4; ++jj) {
+                    T vals[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(accw[i][t][4 * jj + q]);
+                    const int row = i * 32 + l32;
+                    const int chunk = t * 4 + jj;
+                    *reinterpret_cast<uint64_t*>(ep + row * 128 + ((chunk ^ (row & 7)) << 4) + h2 * 8) =
+                        *reinterpret_cast<const uint64_t*>(vals);
+                }
         // LDS operations of one wavefront complete in order: no barrier needed
         const int c = lane & 7;
         const int n = n0 + wn * 64 + c * 8;
@@ -333,8 +346,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
                 *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
             }
         }
-        return;
-    }
+    } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int r = wm * 64 + i * 16 + r16;
@@ -355,6 +367,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
                     if (n + q < p.N) dst[q] = vals[q];
             }
         }
+    }
     }
 }
 
@@ -615,11 +628,22 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) > 256 ? 1 : 2) void moe_gemm_
         b_src[q] = W + (int64_t)n * p.K + chunk * VE;
     }
 
-    f32x4 acc[MT][NTT];
+    // 2-byte types: 32 x 32 x 16 MFMAs (twice the sustained rate of the 16 x 16 x 32 ones)
+    constexpr bool WIDE = HasMma32<T>::value;
+    constexpr int MTW = TM / WGM / 32, NTW = TN / WGN / 32;
+    const int l32 = lane & 31, h2 = lane >> 5;
+    f32x4 acc[WIDE ? 1 : MT][WIDE ? 1 : NTT];
+    f32x16 accw[WIDE ? MTW : 1][WIDE ? NTW : 1];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < (WIDE ? 1 : MT); ++i)
 #pragma unroll
-        for (int t = 0; t < NTT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < (WIDE ? 1 : NTT); ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < (WIDE ? MTW : 1); ++i)
+#pragma unroll
+        for (int t = 0; t < (WIDE ? NTW : 1); ++t)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) accw[i][t][j] = 0.f;
 
     const int n_st = p.K / KT;
     u32x4 ra[A_LOADS], rb[B_LOADS];
@@ -661,20 +685,20 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) > 256 ? 1 : 2) void moe_gemm_
         __builtin_amdgcn_sched_barrier(0);
         const char* As = cur;
         const char* Bs = cur + A_BYTES;
-        if constexpr (HasMma32<T>::value) {
+        if constexpr (WIDE) {
 #pragma unroll
-            for (int kc = 0; kc < KT; kc += 32) {
-                typename Mma32<T>::frag af[MT], bf[NTT];
+            for (int kc = 0; kc < KT; kc += 16) {
+                typename MmaW<T>::frag af[MTW], bf[NTW];
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
-                    af[i] = *reinterpret_cast<const typename Mma32<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+                for (int i = 0; i < MTW; ++i)
+                    af[i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + moe_lds_off<T>(wrow + i * 32 + l32, kc / VE + h2));
 #pragma unroll
-                for (int t = 0; t < NTT; ++t)
-                    bf[t] = *reinterpret_cast<const typename Mma32<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+                for (int t = 0; t < NTW; ++t)
+                    bf[t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 32 + l32, kc / VE + h2));
 #pragma unroll
-                for (int i = 0; i < MT; ++i)
+                for (int i = 0; i < MTW; ++i)
 #pragma unroll
-                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma32<T>::mma(bf[t], af[i], acc[i][t]);
+                    for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[t], af[i], accw[i][t]);
             }
         } else {
 #pragma unroll
@@ -696,6 +720,41 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) > 256 ? 1 : 2) void moe_gemm_
     }
 
     T* out = reinterpret_cast<T*>(p.out);
+    if constexpr (WIDE) {
+        // the wavefront's (TM / WGM) x 64 tile leaves through LDS (free after the last
+        // barrier) as rows of 128 bytes, chunks XOR-swizzled by the row; every store
+        // instruction then writes eight complete 128-byte row segments.
+        // lane holds out[m = i*32 + lane%32][n = t*32 + 8*jj + 4*(lane/32) + q] in accw[i][t][4*jj + q]
+        static_assert(!WIDE || TN / WGN == 64, "epilogue assumes 64 output columns per wavefront");
+        constexpr int WR = TM / WGM;
+        char* ep = smem + wave * (WR * 128);
+#pragma unroll
+        for (int i = 0; i < MTW; ++i)
+#pragma unroll
+            for (int t = 0; t < NTW; ++t)
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    T vals[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(accw[i][t][4 * jj + q]);
+                    const int row = i * 32 + l32;
+                    const int ch = t * 4 + jj;
+                    *reinterpret_cast<uint64_t*>(ep + row * 128 + ((ch ^ (row & 7)) << 4) + h2 * 8) =
+                        *reinterpret_cast<const uint64_t*>(vals);
+                }
+        const int c = lane & 7;
+        const int n = n0 + wcol + c * 8;
+#pragma unroll
+        for (int pass = 0; pass < WR / 8; ++pass) {
+            const int row = pass * 8 + (lane >> 3);
+            const int r = wrow + row;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * 128 + ((c ^ (row & 7)) << 4));
+            if (r < rows && n < p.N) {
+                const int tok = p.token_perm[row0 + r];
+                *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
+            }
+        }
+    } else {
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int r = wrow + i * 16 + r16;
@@ -709,13 +768,13 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) > 256 ? 1 : 2) void moe_gemm_
             for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
             T* dst = out + (int64_t)tok * p.N + n;
             if (n + 4 <= p.N) {
-                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
-                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+                *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
             } else {
                 for (int q = 0; q < 4; ++q)
                     if (n + q < p.N) dst[q] = vals[q];
             }
         }
+    }
     }
 }
 
@@ -729,6 +788,251 @@ static int launch_moe_v4(const MoeParams& p, hipStream_t st) {
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_kernel_v4)");
     hipLaunchKernelGGL((moe_gemm_kernel_v4<T, TM, TN, WAVES, 2>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
     SPX_LAUNCH_CHECK("moe_gemm_kernel_v4");
+    return 0;
+}
+
+// ---- gathered GEMM with LDS-direct loads ------------------------------------------------
+// Same tiles as moe_gemm_kernel_v4, but the operands go from global memory straight into
+// LDS (global_load_lds_dwordx4: each wavefront instruction writes 64 x 16 bytes to
+// consecutive LDS addresses starting at M0), so no registers or LDS-store instructions
+// are spent on staging.  NBUF LDS buffers hold stages s .. s + NBUF - 1; one barrier per
+// stage.  The loads are issued through inline assembly, which keeps the compiler from
+// serialising them against the fragment reads of the other buffers.
+__device__ __forceinline__ void lds_direct_load16(const void* g, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(g) : "memory", "m0");
+}
+
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
+__global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void moe_gemm_kernel_v5(MoeParams p) {
+    constexpr int NTH = 64 * WAVES;
+    constexpr int WGN = WAVES / WGM;
+    constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
+    constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
+    constexpr int A_LOADS = TM * 8 / NTH;
+    constexpr int B_LOADS = TN * 8 / NTH;
+    constexpr int RSTEP = NTH / 8;        // tile rows between a thread's vectors (a multiple of 8)
+    constexpr int A_BYTES = TM * 128;
+    constexpr int BUF = (TM + TN) * 128;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) char smem[];
+    __shared__ int s_expert, s_row0, s_rows;
+
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        const int y = blockIdx.y;
+        int tiles_before = 0;
+        int found_e = -1, found_row0 = 0, found_rows = 0;
+        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
+            const int e = e0 + lane;
+            int cnt = 0, off = 0;
+            if (e < p.n_exp) {
+                off = p.expert_offset[e];
+                cnt = p.expert_offset[e + 1] - off;
+            }
+            const int tiles = (cnt + TM - 1) / TM;
+            const int inc = wave_inclusive_scan(tiles);
+            const int excl = tiles_before + inc - tiles;
+            const bool mine = y >= excl && y < excl + tiles;
+            const unsigned long long hit = __ballot(mine);
+            if (hit) {
+                const int src = __ffsll((long long)hit) - 1;
+                const int lt = y - __shfl(excl, src, 64);
+                found_e = e0 + src;
+                found_row0 = __shfl(off, src, 64) + lt * TM;
+                found_rows = min(TM, __shfl(cnt, src, 64) - lt * TM);
+            }
+            tiles_before += __shfl(inc, 63, 64);
+        }
+        if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
+    }
+    __syncthreads();
+    const int expert = s_expert;
+    if (expert < 0) return;
+    const int row0 = s_row0, rows = s_rows;
+    const int n0 = blockIdx.x * TN;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
+
+    const T* X = reinterpret_cast<const T*>(p.tokens);
+    const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
+
+    // staging map: every wavefront instruction fills 8 consecutive LDS rows (1 KB); lane l
+    // lands at position l % 8 of row l / 8, so it fetches the chunk that the swizzle
+    // keeps at that position: (l % 8) ^ (row % 8)
+    const int srow = threadIdx.x >> 3;
+    const int chunk = (threadIdx.x & 7) ^ (srow & 7);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    const uint32_t st_dst = __builtin_amdgcn_readfirstlane(lds_base + (wave * 8) * 128);
+    const T* a_src[A_LOADS];
+#pragma unroll
+    for (int q = 0; q < A_LOADS; ++q) {
+        const int r = srow + RSTEP * q;
+        const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
+        a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
+    }
+    const T* b_src[B_LOADS];
+#pragma unroll
+    for (int q = 0; q < B_LOADS; ++q) {
+        const int r = srow + RSTEP * q;
+        const int n = n0 + r < p.N ? n0 + r : p.N - 1;
+        b_src[q] = W + (int64_t)n * p.K + chunk * VE;
+    }
+    auto issue_stage = [&](int s) {
+        const uint32_t dst = st_dst + (uint32_t)((s % NBUF) * BUF);
+        const int k = s * KT;
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) lds_direct_load16(a_src[q] + k, dst + q * RSTEP * 128);
+#pragma unroll
+        for (int q = 0; q < B_LOADS; ++q) lds_direct_load16(b_src[q] + k, dst + A_BYTES + q * RSTEP * 128);
+    };
+
+    // 2-byte types: 32 x 32 x 16 MFMAs (twice the sustained rate of the 16 x 16 x 32 ones)
+    constexpr bool WIDE = HasMma32<T>::value;
+    constexpr int MTW = TM / WGM / 32, NTW = TN / WGN / 32;
+    const int l32 = lane & 31, h2 = lane >> 5;
+    f32x4 acc[WIDE ? 1 : MT][WIDE ? 1 : NTT];
+    f32x16 accw[WIDE ? MTW : 1][WIDE ? NTW : 1];
+#pragma unroll
+    for (int i = 0; i < (WIDE ? 1 : MT); ++i)
+#pragma unroll
+        for (int t = 0; t < (WIDE ? 1 : NTT); ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < (WIDE ? MTW : 1); ++i)
+#pragma unroll
+        for (int t = 0; t < (WIDE ? NTW : 1); ++t)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) accw[i][t][j] = 0.f;
+
+    const int n_st = p.K / KT;
+    constexpr int L = A_LOADS + B_LOADS;   // loads per thread and stage
+    issue_stage(0);
+    if (NBUF > 2 && n_st > 1) issue_stage(1);
+
+    for (int s = 0; s < n_st; ++s) {
+        // stage s has landed once at most the loads of the stages after it are outstanding
+        if (NBUF > 2 && s + 1 < n_st) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();   // everyone's part of stage s is in LDS; the buffer of stage s - 1 is free
+        if (s + NBUF - 1 < n_st) issue_stage(s + NBUF - 1);
+        const char* cur = smem + (s % NBUF) * BUF;
+        const char* As = cur;
+        const char* Bs = cur + A_BYTES;
+        if constexpr (WIDE) {
+            // fragments of k-step c + 1 are read while the MFMAs of step c run
+            constexpr int KSTEPS = KT / 16;
+            typename MmaW<T>::frag af[2][MTW], bf[2][NTW];
+            auto read_frags = [&](int c, int slot) {
+#pragma unroll
+                for (int i = 0; i < MTW; ++i)
+                    af[slot][i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + moe_lds_off<T>(wrow + i * 32 + l32, c * 2 + h2));
+#pragma unroll
+                for (int t = 0; t < NTW; ++t)
+                    bf[slot][t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 32 + l32, c * 2 + h2));
+            };
+            read_frags(0, 0);
+#pragma unroll
+            for (int c = 0; c < KSTEPS; ++c) {
+                if (c + 1 < KSTEPS) read_frags(c + 1, (c + 1) & 1);
+                __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of this step's MFMAs
+#pragma unroll
+                for (int i = 0; i < MTW; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < KT; kc += 16) {
+                typename Mma16<T>::frag af[MT], bf[NTT];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int t = 0; t < NTT; ++t)
+                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
+            }
+        }
+    }
+    __syncthreads();   // the epilogue reuses the LDS buffers
+
+    T* out = reinterpret_cast<T*>(p.out);
+    if constexpr (WIDE) {
+        // the wavefront's (TM / WGM) x 64 tile leaves through LDS (free after the last
+        // barrier) as rows of 128 bytes, chunks XOR-swizzled by the row; every store
+        // instruction then writes eight complete 128-byte row segments.
+        // lane holds out[m = i*32 + lane%32][n = t*32 + 8*jj + 4*(lane/32) + q] in accw[i][t][4*jj + q]
+        static_assert(!WIDE || TN / WGN == 64, "epilogue assumes 64 output columns per wavefront");
+        constexpr int WR = TM / WGM;
+        char* ep = smem + wave * (WR * 128);
+#pragma unroll
+        for (int i = 0; i < MTW; ++i)
+#pragma unroll
+            for (int t = 0; t < NTW; ++t)
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    T vals[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(accw[i][t][4 * jj + q]);
+                    const int row = i * 32 + l32;
+                    const int ch = t * 4 + jj;
+                    *reinterpret_cast<uint64_t*>(ep + row * 128 + ((ch ^ (row & 7)) << 4) + h2 * 8) =
+                        *reinterpret_cast<const uint64_t*>(vals);
+                }
+        const int c = lane & 7;
+        const int n = n0 + wcol + c * 8;
+#pragma unroll
+        for (int pass = 0; pass < WR / 8; ++pass) {
+            const int row = pass * 8 + (lane >> 3);
+            const int r = wrow + row;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * 128 + ((c ^ (row & 7)) << 4));
+            if (r < rows && n < p.N) {
+                const int tok = p.token_perm[row0 + r];
+                *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
+            }
+        }
+    } else {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int r = wrow + i * 16 + r16;
+        if (r >= rows) continue;
+        const int tok = p.token_perm[row0 + r];
+#pragma unroll
+        for (int t = 0; t < NTT; ++t) {
+            const int n = n0 + wcol + t * 16 + g4 * 4;
+            T vals[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
+            T* dst = out + (int64_t)tok * p.N + n;
+            if (n + 4 <= p.N) {
+                *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+            } else {
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < p.N) dst[q] = vals[q];
+            }
+        }
+    }
+    }
+}
+
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
+static int launch_moe_v5(const MoeParams& p, hipStream_t st) {
+    const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp;
+    if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
+    const int smem = NBUF * (TM + TN) * 128;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel_v5<T, TM, TN, WAVES, WGM, NBUF>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_kernel_v5)");
+    hipLaunchKernelGGL((moe_gemm_kernel_v5<T, TM, TN, WAVES, WGM, NBUF>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
+    SPX_LAUNCH_CHECK("moe_gemm_kernel_v5");
     return 0;
 }
 
@@ -777,7 +1081,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 6, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 8, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -793,10 +1097,24 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
     p.w_kcontig = weight_layout == 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    // tile_cfg 0: default (1); 1: 128x128 tiles, no prefetch (any weight layout);
-    // 2: 256x128 tiles, 3: 128x128 tiles, both with the next K stage prefetched into
-    // registers; 4: 256x256 tiles with two LDS buffers (2..4: k-contiguous weights only).
-    if (tile_cfg == 0) tile_cfg = 1;  // measured best on the benchmark shapes; the others stay selectable
+    // tile_cfg 0: 7 for k-contiguous weights, else 1; 1: 128x128 tiles, no prefetch (any
+    // weight layout); 2: 256x128 tiles, 3 and 6: 128x128 tiles with the next K stage
+    // prefetched into registers; 4, 5: 256x256 and 128x128 tiles with two LDS buffers;
+    // 7, 8: 128x128 and 256x256 tiles filled by LDS-direct loads (2..8: k-contiguous
+    // weights only).  7 measured best on the benchmark shapes; the others stay selectable.
+    if (tile_cfg == 0) tile_cfg = p.w_kcontig ? 7 : 1;
+    if (tile_cfg >= 7) {
+        SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
+#define SPX_MOE5(T)                                                             \
+        if (tile_cfg == 7) return launch_moe_v5<T, 128, 128, 4, 2, 2>(p, st);   \
+        return launch_moe_v5<T, 256, 256, 8, 2, 2>(p, st);
+        switch (dtype) {
+            case SPX_F32: SPX_MOE5(float)
+            case SPX_F16: SPX_MOE5(_Float16)
+            default: SPX_MOE5(bf16_t)
+        }
+#undef SPX_MOE5
+    }
     if (tile_cfg == 4 || tile_cfg == 5) {
         // two LDS buffers, one barrier per stage (k-contiguous weights only):
         // 4: 256x256 tiles, eight wavefronts; 5: 128x128 tiles, four wavefronts, two workgroups per CU
