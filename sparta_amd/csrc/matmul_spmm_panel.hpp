@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
     // they stay in VGPRs.
     u32x4 d0[4], s0[WL], d1[4], s1[WL], d2[4], s2[WL];
 
-#define SPX_PANEL_ISSUE(IT, DREG, SREG)                                                            \
+#define SPX_PANEL_ISSUE(IT, LIVE, DREG, SREG)                                                          \
     do {                                                                                           \
         const int er_ = (IT) / CH;                                                                 \
         const int ch_ = (IT) % CH;                                                                 \
@@ -221,18 +221,19 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
                                       : (p.s_kcontig ? S + (int64_t)j * BN * p.s_ld + koff_        \
                                                      : S + (int64_t)koff_ * p.s_ld + (int64_t)j * BN); \
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                              \
-            DREG[q] = *reinterpret_cast<const u32x4*>(dptr[q] + (DT ? (int64_t)koff_ * p.d_ld : (int64_t)koff_)); \
+            DREG[q] = *reinterpret_cast<const u32x4*>((LIVE) ? dptr[q] + (DT ? (int64_t)koff_ * p.d_ld : (int64_t)koff_) : D); \
         if constexpr (SHW) {                                                                       \
             if (sh_active)                                                                         \
-                SREG[0] = *reinterpret_cast<const u32x4*>(sblk_ + sh_toff);                        \
+                SREG[0] = *reinterpret_cast<const u32x4*>((LIVE) ? sblk_ + sh_toff : S);           \
         } else {                                                                                   \
             _Pragma("unroll") for (int q = 0; q < WL; ++q)                                         \
-                SREG[q] = *reinterpret_cast<const u32x4*>(sblk_ + (int64_t)(q * 16 + lrow) * sld + lchk * E16); \
+                SREG[q] = *reinterpret_cast<const u32x4*>((LIVE) ? sblk_ + (int64_t)(q * 16 + lrow) * sld + lchk * E16 : S); \
         }                                                                                          \
     } while (0)
 
 // All global loads and LDS writes of the pipeline are issued unconditionally (steps
-// past the end re-load the last step and are not accumulated): with no branch
+// past the end load the first 16 bytes of each operand in every lane - one cache line
+// per instruction - and are not accumulated): with no branch
 // around a memory instruction the number of loads in flight is the same on every
 // path, so each wait only covers the oldest stage and NST-1 stages stay in flight.
 #define SPX_PANEL_STEP(IT, DREG, SREG)                                                             \
@@ -259,8 +260,9 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
                 *reinterpret_cast<u32x4*>(sdst_ + sofs[q]) = SREG[q];                              \
         }                                                                                          \
         {                                                                                          \
-            const int nx_ = (IT) + NST < n_it ? (IT) + NST : n_it - 1;                             \
-            SPX_PANEL_ISSUE(nx_, DREG, SREG);                                                      \
+            const bool live_ = (IT) + NST < n_it;                                                  \
+            const int nx_ = live_ ? (IT) + NST : n_it - 1;                                         \
+            SPX_PANEL_ISSUE(nx_, live_, DREG, SREG);                                               \
         }                                                                                          \
         if constexpr (SHW) __syncthreads(); /* the S tile of this step is complete */             \
         if ((IT) < n_it) {                                                                         \
@@ -277,9 +279,9 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
     } while (0)
 
     if (n_it > 0) {
-        SPX_PANEL_ISSUE(0, d0, s0);
-        SPX_PANEL_ISSUE((1 < n_it ? 1 : n_it - 1), d1, s1);
-        if (NST > 2) SPX_PANEL_ISSUE((2 < n_it ? 2 : n_it - 1), d2, s2);
+        SPX_PANEL_ISSUE(0, true, d0, s0);
+        SPX_PANEL_ISSUE((1 < n_it ? 1 : n_it - 1), 1 < n_it, d1, s1);
+        if (NST > 2) SPX_PANEL_ISSUE((2 < n_it ? 2 : n_it - 1), 2 < n_it, d2, s2);
         for (int it = 0; it < n_it; it += NST) {
             SPX_PANEL_STEP(it, d0, s0);
             SPX_PANEL_STEP(it + 1, d1, s1);
