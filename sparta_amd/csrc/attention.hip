@@ -426,6 +426,246 @@ static int launch_attention_v2(const AttnParams& p, int batch, int BW, int E, hi
     return fail(SPX_E_CONFIG, "the pipelined attention kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
 }
 
+// ---- pipelined variant on 32 x 32 x 16 MFMAs ---------------------------------------------
+// The 32 x 32 x 16 MFMA sustains about twice the rate of the 16 x 16 x 32 one on gfx950,
+// so here a wavefront owns 32 queries and every product runs on the wide shape:
+//   S^T[key][query] (A = K rows from LDS, B = Q from registers): lane l holds, for query
+//   l % 32, the keys 8a + 4(l / 32) + b (a, b = 0..3) of a 32-key tile in s[4a + b];
+//   O^T[e][query] += V^T P^T in 16-key steps: k-slot i of half h = l / 32 is key
+//   16u + 8(i / 4) + 4h + i % 4, which is s[8(u % 2) + i] of tile u / 2 - the probabilities go
+//   from the accumulator straight into the B operand - and for V^T two LDS transpose reads
+//   (keys 16u + 4h .. +3 and 16u + 8 + 4h .. +3 of column e).
+// Staging, LDS layout, lazy rescaling and the XCD mapping are those of attention_kernel_v2;
+// the row sums are kept per lane (two lanes per query, joined at the end).
+template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
+__global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams p, int nbr, int batch) {
+    constexpr int NT = 64 * WAVES;
+    constexpr int KT = BW / 32, EC = E / 16, ET = E / 32, KS = BW / 16;
+    constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
+    constexpr int VP = E * 2 + 32;            // V row pitch in bytes
+    constexpr int TILE = BW * (KP + VP);
+    constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
+    constexpr int VPR = E / 8;                // 16-byte vectors per tile row
+    constexpr int NV = BW * VPR / NT;         // vectors per thread and tile
+    constexpr int RSTEP = NT / VPR;           // tile rows between a thread's vectors
+    static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && NV >= 1 && NV <= 8, "tile does not split over the workgroup");
+    typedef typename MmaW<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    // workgroup L runs on XCD L % 8: give each XCD whole batch*head entries
+    const int L = blockIdx.x;
+    const int slot = L >> 3;
+    const int64_t b = (slot / nbr) * 8 + (L & 7);
+    const int br = slot % nbr;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, h2 = lane >> 5;
+
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.Nt * E;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    const T* Vg = reinterpret_cast<const T*>(p.v) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    T* O = reinterpret_cast<T*>(p.out) + b * (int64_t)p.Nt * E;
+
+    const int qrow = br * (32 * WAVES) + wave * 32 + l32;
+    Frag qf[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) qf[c] = *reinterpret_cast<const Frag*>(Q + (int64_t)qrow * E + c * 16 + h2 * 8);
+
+    f32x16 oacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) oacc[t][j] = 0.f;
+    float m_run = -1e30f, l_part = 0.f;
+    const float c2 = p.inv_t * 1.4426950408889634f;
+    constexpr float RESCALE_LOG2 = 6.f;
+
+    // staging map: vector v = tid + i * NT of the (contiguous) tile is row v / VPR, chunk v % VPR
+    const int st_row = threadIdx.x / VPR, st_chunk = threadIdx.x % VPR;
+    int k_dst[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int row = st_row + i * RSTEP;
+        k_dst[i] = row * KP + (st_chunk ^ (row & 7)) * 16;
+    }
+    const int v_dst = BW * KP + st_row * VP + st_chunk * 16;
+    // fragment bases
+    const int k_src = l32 * KP;
+    const int k_sw = l32 & 7;
+    const int i16 = lane & 15;
+    const int v_src = BW * KP + (h2 * 4 + (i16 >> 2)) * VP + (((lane >> 4) & 1) * 16 + (i16 & 3) * 4) * 2;
+
+    const int e_begin = p.row_ptr[br];
+    const int e_end = p.row_ptr[br + 1];
+    u32x4 kr[NV], vr[NV];
+    int bc = 0;
+    if (e_begin < e_end) {
+        bc = p.bcsr_idx[e_begin] & 0xffff;
+        const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();  // the previous block's fragments are consumed
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + k_dst[i]) = kr[i];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
+        const int key0 = bc * BW;
+        // next live block (the last step re-reads its own block; the copy is not used)
+        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        {
+            const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+        }
+        unsigned live[KT][4];
+        if constexpr (HAS_MASK) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+                    live[kt][a] = *reinterpret_cast<const uint32_t*>(p.mask + (int64_t)qrow * p.Ns + key0 + kt * 32 + a * 8 + h2 * 4);
+        }
+        __syncthreads();
+
+        // ---- S^T tiles: 32 keys x this wave's 32 queries ------------------------------------
+        f32x16 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s[kt][j] = 0.f;
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 32 * KP + (((c * 2 + h2) ^ k_sw) * 16));
+                s[kt] = MmaW<T>::mma(kf, qf[c], s[kt]);
+            }
+        }
+        float tmax = -1e30f;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                if constexpr (HAS_MASK) {
+                    if ((live[kt][j >> 2] >> (8 * (j & 3))) & 0xffu) tmax = fmaxf(tmax, s[kt][j]);
+                } else {
+                    tmax = fmaxf(tmax, s[kt][j]);
+                }
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        // m_run only has to keep exp2 in range: it moves (and the accumulators are rescaled)
+        // only when some query's maximum outgrows it by more than 2^RESCALE_LOG2
+        if (__builtin_amdgcn_ballot_w64((tmax - m_run) * c2 > RESCALE_LOG2) != 0) {
+            const float m_new = fmaxf(m_run, tmax);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2);
+            m_run = m_new;
+            l_part *= alpha;
+#pragma unroll
+            for (int t = 0; t < ET; ++t) oacc[t] *= alpha;
+        }
+        const float mc = m_run * c2;
+        Frag pf[KS];
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+            f32x8 pv;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int kt = u >> 1, j = 8 * (u & 1) + i;
+                float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][j], c2, -mc));
+                if constexpr (HAS_MASK) x = ((live[kt][j >> 2] >> (8 * (j & 3))) & 0xffu) ? x : 0.f;
+                pv[i] = x;
+                l_part += x;
+            }
+            pf[u] = AttnPack<T>::pack(pv);
+        }
+        // ---- O^T[e][query] += V^T P^T ------------------------------------------------------
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int u = 0; u < KS; ++u) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + v_src + (u * 16) * VP + t * 64));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + v_src + (u * 16 + 8) * VP + t * 64));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                oacc[t] = MmaW<T>::mma(__builtin_bit_cast(Frag, both), pf[u], oacc[t]);
+            }
+        }
+    }
+
+    // lane holds O^T[e = t*32 + 8*(j/4) + 4*h2 + j%4][query l32]; rows with no live entry give 0
+    const float l_run = l_part + __shfl_xor(l_part, 32, 64);
+    const float inv_l = l_run > 0.f ? 1.f / l_run : 0.f;
+#pragma unroll
+    for (int t = 0; t < ET; ++t)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            T vals[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][4 * a + q] * inv_l);
+            *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 32 + a * 8 + h2 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+        }
+}
+
+template <typename T, int BW, int E, int WAVES>
+static int launch_attention_v3_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr int TILE = BW * (E * 4 + 32);
+    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    const int nbr = p.Nt / p.BH;
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (p.mask) {
+        if (smem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_kernel_v3<T, BW, E, WAVES, true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_kernel_v3)");
+        }
+        hipLaunchKernelGGL((attention_kernel_v3<T, BW, E, WAVES, true>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    } else {
+        if (smem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_kernel_v3<T, BW, E, WAVES, false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_kernel_v3)");
+        }
+        hipLaunchKernelGGL((attention_kernel_v3<T, BW, E, WAVES, false>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    }
+    SPX_LAUNCH_CHECK("attention_kernel_v3");
+    return 0;
+}
+
+// The wide-MFMA kernel covers query blocks of 32 / 64 / 128 (one wavefront per 32 queries),
+// key blocks of 32 / 64 / 128 and head dimensions 64 / 128, as long as a thread stages one
+// to eight 16-byte vectors of each tile.
+static bool attention_v3_supported(int BH, int BW, int E) {
+    if (!((BH == 32 || BH == 64 || BH == 128) && (BW == 32 || BW == 64 || BW == 128) && (E == 64 || E == 128))) return false;
+    const int nt = BH * 2, vecs = BW * E / 8;
+    return vecs % nt == 0 && vecs / nt >= 1 && vecs / nt <= 8;
+}
+
+template <typename T>
+static int launch_attention_v3(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTN3_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_v3_inst<T, bw, e, bh / 32>(p, batch, st);
+    SPX_ATTN3_CASE(32, 32, 64) SPX_ATTN3_CASE(32, 64, 64) SPX_ATTN3_CASE(32, 32, 128)
+    SPX_ATTN3_CASE(64, 32, 64) SPX_ATTN3_CASE(64, 64, 64) SPX_ATTN3_CASE(64, 128, 64)
+    SPX_ATTN3_CASE(64, 32, 128) SPX_ATTN3_CASE(64, 64, 128)
+    SPX_ATTN3_CASE(128, 32, 64) SPX_ATTN3_CASE(128, 64, 64) SPX_ATTN3_CASE(128, 128, 64)
+    SPX_ATTN3_CASE(128, 32, 128) SPX_ATTN3_CASE(128, 64, 128) SPX_ATTN3_CASE(128, 128, 128)
+#undef SPX_ATTN3_CASE
+    return fail(SPX_E_CONFIG, "the wide-MFMA attention kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
 template <typename T, int BW, int E>
 static int launch_attention_inst(const AttnParams& p, int batch, hipStream_t st) {
     const int waves = p.BH / 16;
@@ -627,7 +867,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
                                      int batch, int Nt, int Ns, int E, int BH, int BW,
                                      int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 2, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
                 "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
     SPX_REQUIRE(q && k && v && out && row_ptr && bcsr_idx, SPX_E_NULL, "a required buffer is NULL");
@@ -645,8 +885,14 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel
+    // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel;
+    // 3: pipelined kernel on 32x32x16 MFMAs (one wavefront per 32 queries; measured within a few
+    // per cent of 2 either way, so 0 keeps 2)
     if (tile_cfg == 0) tile_cfg = attention_v2_supported(BH, BW, E) ? 2 : 1;
+    if (tile_cfg == 3) {
+        if (dtype == SPX_F16) return launch_attention_v3<_Float16>(p, batch, BW, E, st);
+        return launch_attention_v3<bf16_t>(p, batch, BW, E, st);
+    }
     if (tile_cfg == 2) {
         if (dtype == SPX_F16) return launch_attention_v2<_Float16>(p, batch, BW, E, st);
         return launch_attention_v2<bf16_t>(p, batch, BW, E, st);

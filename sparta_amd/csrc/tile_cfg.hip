@@ -35,6 +35,7 @@ static const spx_tile_cfg kAttentionCfgs[] = {
     {0, 0, 0, 0, 1, 16, 6, "auto"},
     {1, 0, 0, 0, 1, 16, 6, "fused-online-softmax"},
     {2, 0, 0, 0, 2, 32, 6, "fused-pipelined"},
+    {3, 0, 0, 0, 2, 32, 6, "fused-pipelined-32x32-mfma"},
 };
 static const spx_tile_cfg kMoeCfgs[] = {
     {0, 0, 0, 4, 0, 0, 7, "auto"},

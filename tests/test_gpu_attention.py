@@ -133,7 +133,7 @@ def test_attention_long_sequence_layout(gpu):
 @pytest.mark.parametrize('BH,BW,E', [(64, 64, 64), (32, 32, 64), (32, 128, 64), (64, 32, 128), (128, 64, 64),
                                      (128, 128, 128), (64, 128, 128), (32, 64, 128), (128, 32, 128)])
 def test_attention_kernel_variants(dtype, element_mask, BH, BW, E, gpu):
-    """Both fused kernels through the C ABI (tile configs 1 and 2) on the same inputs:
+    """The fused kernels through the C ABI (tile configs 1, 2 and 3) on the same inputs:
     each against the oracle, batch sizes that do not fill the eight-way workgroup
     numbering, empty block rows and (element_mask) partly filled blocks."""
     from sparta_amd import _lib
@@ -150,8 +150,10 @@ def test_attention_kernel_variants(dtype, element_mask, BH, BW, E, gpu):
     q, k, v = q.to(gpu), k.to(gpu), v.to(gpu)
     want = ops.attention_reference(q_np, k_np, v_np, mask_np)
     lib = _lib.load()
-    for cfg in (1, 2):
+    for cfg in (1, 2, 3):
         out = torch.full_like(q, float('nan'))
+        if cfg == 3 and not 1 <= (BW * E // 8) // (BH * 2) <= 8:
+            continue  # the wide-MFMA kernel stages one to eight vectors per thread and tile
         rc = lib.spx_attention_forward(
             _lib.dtype_code(dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
             _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf),
