@@ -106,6 +106,16 @@ int spx_bcs_scatter(const void* sparse, void* dense, const void* idx, int idx_ki
  * whose grids follow the natural order (matmul.py:143-149).  ptr int32 [n+1]. */
 int spx_bcs_schedule(const int32_t* ptr, int n, int32_t* order, spx_stream_t stream);
 
+/* spx_bcs_index plus the launch orders of spx_bcs_schedule from the same launch (an index
+ * that is rebuilt for every call has no time for a third kernel): row_order int32 [H/BH]
+ * (needs the BCSR index) and col_order int32 [W/BW] (needs the BCSC index), each optional.
+ * No counterpart in the reference. */
+int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
+                            int32_t* row_ptr, int32_t* bcsr_idx,
+                            int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                            int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
+                            void* workspace, size_t workspace_bytes, spx_stream_t stream);
+
 /* Row / column sums of compressed values (fp32 accumulate), used for the bias
  * gradient of a compressed sparse-output matmul.  Replace
  * BCSFunctionContext.row_sum / col_sum (block_compressed.py:360-403) and

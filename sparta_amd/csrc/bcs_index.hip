@@ -88,7 +88,37 @@ struct EmitParams {
     int32_t* nnz_dev;
     int cap;
     int R, Cn, WPR, WPC;
+    int32_t* row_order;         // optional: block rows / columns by descending number of live blocks
+    int32_t* col_order;
 };
+
+// Launch order: the n segments of ptr sorted by descending length (bucketed at 255), by
+// one workgroup; bins is a 256-entry LDS table.  ptr may have been written by this
+// workgroup just before (the leading barrier orders those stores).
+__device__ void schedule_segments(const int32_t* ptr, int n, int32_t* order, int* bins) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) bins[i] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int c = ptr[i + 1] - ptr[i];
+        atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {  // exclusive scan of the 256 bins by one wavefront
+        int carry = 0;
+        for (int b0 = 0; b0 < 256; b0 += 64) {
+            const int v = bins[b0 + threadIdx.x];
+            const int inc = wave_inclusive_scan(v);
+            bins[b0 + threadIdx.x] = carry + inc - v;
+            carry += __shfl(inc, 63, 64);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int c = ptr[i + 1] - ptr[i];
+        order[atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1)] = i;
+    }
+}
 
 // Exclusive prefix sum of a[0..n) in place by one workgroup; returns the total.
 __device__ int block_scan_inplace(int* a, int n, int* lds) {
@@ -117,6 +147,7 @@ __device__ int block_scan_inplace(int* a, int n, int* lds) {
 
 __global__ __launch_bounds__(1024) void emit_kernel(EmitParams p) {
     __shared__ int lds[32];
+    __shared__ int s_bins[256];
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     const int nwaves = blockDim.x >> 6;
@@ -153,6 +184,7 @@ __global__ __launch_bounds__(1024) void emit_kernel(EmitParams p) {
             }
         }
     }
+    if (p.row_order && p.row_ptr) schedule_segments(p.row_ptr, p.R, p.row_order, s_bins);
     if (!p.col_ptr) return;  // uniform over the workgroup
 
     // ---- column words --------------------------------------------------------
@@ -193,6 +225,7 @@ __global__ __launch_bounds__(1024) void emit_kernel(EmitParams p) {
             }
         }
     }
+    if (p.col_order) schedule_segments(p.col_ptr, p.Cn, p.col_order, s_bins);
 }
 
 // Fast path of the emit step for block grids of at most 2048 row words and 2048
@@ -222,6 +255,7 @@ __global__ __launch_bounds__(1024) void emit_fast_kernel(EmitParams p) {
     __shared__ unsigned long long s_bits[EMIT_FAST_WORDS];
     __shared__ int s_base[EMIT_FAST_WORDS];
     __shared__ int s_scan[16];
+    __shared__ int s_bins[256];
     const int tid = threadIdx.x;
 
     // ---- row words: word g = r * WPR + wi covers columns wi*64 .. wi*64+63 of row r ----
@@ -282,6 +316,7 @@ __global__ __launch_bounds__(1024) void emit_fast_kernel(EmitParams p) {
         p.nnz_dev[0] = nnz;
         if (p.row_ptr) p.row_ptr[p.R] = nnz;
     }
+    if (p.row_order && p.row_ptr) schedule_segments(p.row_ptr, p.R, p.row_order, s_bins);
     if (!p.col_ptr) return;
     __syncthreads();  // s_bits / s_base complete
 
@@ -343,32 +378,12 @@ __global__ __launch_bounds__(1024) void emit_fast_kernel(EmitParams p) {
         }
     }
     if (tid == 0) p.col_ptr[p.Cn] = nnz2;
+    if (p.col_order) schedule_segments(p.col_ptr, p.Cn, p.col_order, s_bins);
 }
 
-// Launch order: segments of ptr sorted by descending length (bucketed at 255).
 __global__ __launch_bounds__(1024) void schedule_kernel(const int32_t* ptr, int n, int32_t* order) {
     __shared__ int bins[256];
-    if (threadIdx.x < 256) bins[threadIdx.x] = 0;
-    __syncthreads();
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const int c = ptr[i + 1] - ptr[i];
-        atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1);
-    }
-    __syncthreads();
-    if (threadIdx.x < 64) {  // exclusive scan of the 256 bins by one wavefront
-        int carry = 0;
-        for (int b0 = 0; b0 < 256; b0 += 64) {
-            const int v = bins[b0 + threadIdx.x];
-            const int inc = wave_inclusive_scan(v);
-            bins[b0 + threadIdx.x] = carry + inc - v;
-            carry += __shfl(inc, 63, 64);
-        }
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const int c = ptr[i + 1] - ptr[i];
-        order[atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1)] = i;
-    }
+    schedule_segments(ptr, n, order, bins);
 }
 
 struct IndexWorkspace {
@@ -408,11 +423,40 @@ extern "C" size_t spx_bcs_index_workspace_bytes(int H, int W, int BH, int BW) {
     return spx::index_workspace(H, W, BH, BW).total;
 }
 
+namespace spx {
+static int bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW,
+                          int32_t* row_ptr, int32_t* bcsr_idx,
+                          int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                          int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
+                          void* workspace, size_t workspace_bytes, spx_stream_t stream);
+}
+
 extern "C" int spx_bcs_index(const uint8_t* mask, int H, int W, int BH, int BW,
                              int32_t* row_ptr, int32_t* bcsr_idx,
                              int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
                              int32_t* nnz_dev, int cap,
                              void* workspace, size_t workspace_bytes, spx_stream_t stream) {
+    return spx::bcs_index_impl(mask, H, W, BH, BW, row_ptr, bcsr_idx, col_ptr, bcsc_idx, bcsc_i64, nnz_dev, cap,
+                               nullptr, nullptr, workspace, workspace_bytes, stream);
+}
+
+extern "C" int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
+                                       int32_t* row_ptr, int32_t* bcsr_idx,
+                                       int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                                       int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
+                                       void* workspace, size_t workspace_bytes, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(!row_order || row_ptr, SPX_E_NULL, "row_order needs the BCSR index");
+    SPX_REQUIRE(!col_order || col_ptr, SPX_E_NULL, "col_order needs the BCSC index");
+    return bcs_index_impl(mask, H, W, BH, BW, row_ptr, bcsr_idx, col_ptr, bcsc_idx, bcsc_i64, nnz_dev, cap,
+                          row_order, col_order, workspace, workspace_bytes, stream);
+}
+
+static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW,
+                               int32_t* row_ptr, int32_t* bcsr_idx,
+                               int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                               int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
+                               void* workspace, size_t workspace_bytes, spx_stream_t stream) {
     using namespace spx;
     int rc = check_index_shape(H, W, BH, BW);
     if (rc) return rc;
@@ -471,6 +515,7 @@ extern "C" int spx_bcs_index(const uint8_t* mask, int H, int W, int BH, int BW,
     ep.col_ptr = col_ptr; ep.bcsc_idx = bcsc_idx; ep.bcsc_i64 = bcsc_i64;
     ep.nnz_dev = nnz_dev; ep.cap = cap;
     ep.R = ws.R; ep.Cn = ws.Cn; ep.WPR = ws.WPR; ep.WPC = ws.WPC;
+    ep.row_order = row_order; ep.col_order = col_order;
     if (ws.R * ws.WPR <= EMIT_FAST_WORDS && ws.Cn * ws.WPC <= EMIT_FAST_WORDS)
         hipLaunchKernelGGL(emit_fast_kernel, dim3(1), dim3(1024), 0, st, ep);
     else

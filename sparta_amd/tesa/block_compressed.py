@@ -234,19 +234,25 @@ class BCSFunctionContext(TeSAFunctionContext):
         if self._BCSC:
             col_ptr = torch.empty((Cn + 1,), **i32)
             bcsc = torch.empty((cap,), dtype=torch.int64 if both else torch.int32, device=dev)
+        # the launch orders of the matmul kernels come out of the same launch
+        row_order = torch.empty((R,), **i32) if self._BCSR else None
+        col_order = torch.empty((Cn,), **i32) if self._BCSC else None
         ws = self._workspace(H, W, dev)
         with torch.cuda.device(dev):
-            rc = _lib.load().spx_bcs_index(
+            rc = _lib.load().spx_bcs_index_scheduled(
                 _lib.dev_ptr(mask), H, W, BH, BW,
                 _lib.dev_ptr(row_ptr), _lib.dev_ptr(bcsr), _lib.dev_ptr(col_ptr), _lib.dev_ptr(bcsc),
-                1 if both else 0, _lib.dev_ptr(nnz_dev), cap, _lib.dev_ptr(ws), ws.numel(),
-                _lib.current_stream(dev))
-        _lib.check(rc, 'spx_bcs_index')
+                1 if both else 0, _lib.dev_ptr(nnz_dev), cap, _lib.dev_ptr(row_order), _lib.dev_ptr(col_order),
+                _lib.dev_ptr(ws), ws.numel(), _lib.current_stream(dev))
+        _lib.check(rc, 'spx_bcs_index_scheduled')
         if both:
-            return BCSRCIndexes(self, mask, row_ptr, col_ptr, bcsr, bcsc, nnz_dev, BH, BW)
-        if self._BCSR:
-            return BCSRIndexes(self, mask, row_ptr, bcsr, nnz_dev, BH, BW)
-        return BCSCIndexes(self, mask, col_ptr, bcsc, nnz_dev, BH, BW)
+            indexes = BCSRCIndexes(self, mask, row_ptr, col_ptr, bcsr, bcsc, nnz_dev, BH, BW)
+        elif self._BCSR:
+            indexes = BCSRIndexes(self, mask, row_ptr, bcsr, nnz_dev, BH, BW)
+        else:
+            indexes = BCSCIndexes(self, mask, col_ptr, bcsc, nnz_dev, BH, BW)
+        indexes.__dict__['_launch_order'] = {k: v for k, v in (('row', row_order), ('col', col_order)) if v is not None}
+        return indexes
 
     # ---- values ------------------------------------------------------------------
     def convert(self, dense: torch.Tensor, index: torch.Tensor, block_nnz: int, H: int, W: int,

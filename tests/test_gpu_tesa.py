@@ -14,6 +14,36 @@ pytestmark = pytest.mark.gpu
 EDGES = [4, 8, 16, 32, 64, 128]
 
 
+def _check_launch_order(order, ptr):
+    """The scheduling hint that comes out of the index launch: a permutation of the
+    segments, longest first (lengths are bucketed at 255)."""
+    order = order.cpu().numpy()
+    n = len(ptr) - 1
+    assert order.dtype == np.int32 and np.array_equal(np.sort(order), np.arange(n))
+    lengths = np.minimum(np.diff(ptr)[order], 255)
+    assert np.all(lengths[:-1] >= lengths[1:])
+
+
+def test_launch_order_matches_standalone_schedule(gpu):
+    """spx_bcs_index_scheduled and spx_bcs_schedule sort the same way (a grid large
+    enough for the general emit kernel and a small one for the fast one)."""
+    from sparta_amd import _lib
+    for shape, blk in (((4096, 8192), (4, 4)), ((512, 768), (32, 32))):
+        mask_np = ops.block_mask(shape, blk, 0.9, seed=5)
+        idx = get_bcs_function(blk[0], blk[1], True, True).build_indexes(torch.from_numpy(mask_np).to(gpu))
+        for by, ptr in (('row', idx.row_ptr), ('col', idx.col_ptr)):
+            n = ptr.numel() - 1
+            alone = torch.empty((n,), dtype=torch.int32, device=gpu)
+            _lib.check(_lib.load().spx_bcs_schedule(_lib.dev_ptr(ptr), n, _lib.dev_ptr(alone), _lib.current_stream(gpu)),
+                       'spx_bcs_schedule')
+            ptr_np = ptr.cpu().numpy()
+            _check_launch_order(idx.launch_order(by), ptr_np)
+            _check_launch_order(alone, ptr_np)
+            fused_len = np.minimum(np.diff(ptr_np)[idx.launch_order(by).cpu().numpy()], 255)
+            alone_len = np.minimum(np.diff(ptr_np)[alone.cpu().numpy()], 255)
+            assert np.array_equal(fused_len, alone_len)
+
+
 def _check_indexes(mask_np, BH, BW, gpu):
     mask = torch.from_numpy(mask_np).to(gpu)
     H, W = mask_np.shape
@@ -32,7 +62,12 @@ def _check_indexes(mask_np, BH, BW, gpu):
     assert np.array_equal(c.BCSC_idx.cpu().numpy(), bcsc32)
     assert c.BCSC_idx.dtype == torch.int32
 
+    _check_launch_order(r.launch_order('row'), row_ptr)
+    _check_launch_order(c.launch_order('col'), col_ptr)
+
     rc = get_bcs_function(BH, BW, True, True).build_indexes(mask)
+    _check_launch_order(rc.launch_order('row'), row_ptr)
+    _check_launch_order(rc.launch_order('col'), col_ptr)
     assert rc.block_nnz == nnz
     assert np.array_equal(rc.row_ptr.cpu().numpy(), row_ptr)
     assert np.array_equal(rc.col_ptr.cpu().numpy(), col_ptr)
