@@ -10,6 +10,7 @@ method and point; the Triton competitors are left out).
     python bench_sweep.py --op attention --quick
     python bench_sweep.py --op matmul --tune 8           # tune every point (8 trials per
                                                          # kernel), write params/<device>.csv
+    python bench_sweep.py --op matmul --tune 1000 --algo grid   # the whole search space
 
 Operator configurations come from the tuned-config tables shipped in
 sparta_amd/params/<op>/ (`<device name>.csv`, else `default.csv`; the format of the
@@ -91,7 +92,7 @@ def sweep_matmul(args, torch, sparta, table_dir, device_name):
             op = sparta.nn.SparseBatchMatMul(B_mask=mask, transpose_A=False, transpose_B=True, compressed=True)
             sample = [data['A'], data['B']]
             if args.tune:
-                best = sparta.nn.tune(op, sample_inputs=sample, sample_grads=[data['grad_C']], algo='rand',
+                best = sparta.nn.tune(op, sample_inputs=sample, sample_grads=[data['grad_C']], algo=args.algo,
                                       max_trials=args.tune, backward_weight=1.0, tile_configs=False)
                 config = best['root']
                 if config is None:
@@ -141,7 +142,7 @@ def sweep_attention(args, torch, sparta, table_dir, device_name):
                 continue
             op = sparta.nn.SparseAttention(mask=mask)
             if args.tune:
-                best = sparta.nn.tune(op, sample_inputs=[q, k, v], sample_grads=[grad], algo='rand',
+                best = sparta.nn.tune(op, sample_inputs=[q, k, v], sample_grads=[grad], algo=args.algo,
                                       max_trials=args.tune, backward_weight=1.0)
                 config = best['root']
                 if config is None:  # every random trial hit an invalid combination: use the fallback
@@ -164,6 +165,7 @@ def main():
     ap.add_argument('--dtype', choices=['fp16', 'bf16', 'fp32'], default='fp16')
     ap.add_argument('--quick', action='store_true', help='4 sparsities per granularity instead of 12')
     ap.add_argument('--tune', type=int, default=0, help='tune every point with this many trials per kernel')
+    ap.add_argument('--algo', choices=['rand', 'grid'], default='rand', help='search algorithm of --tune')
     ap.add_argument('--warmups', type=int, default=20)
     ap.add_argument('--iters', type=int, default=50)
     ap.add_argument('--out', default=os.path.join(ROOT, 'sweep_out'), help='directory for the result CSVs')
