@@ -134,8 +134,7 @@ __global__ __launch_bounds__(512) void attention_kernel(AttnParams p) {
             for (int q = 0; q < 4; ++q)
                 if ((bits >> (8 * q)) & 0xffu) tmax = fmaxf(tmax, s[kt][q]);
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        tmax = xor32_max(xor16_max(tmax));
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = __expf((m_run - m_new) * p.inv_t);
         float psum = 0.f;
@@ -150,8 +149,7 @@ __global__ __launch_bounds__(512) void attention_kernel(AttnParams p) {
             }
             pf[kt] = AttnMma<T>::pack(pv[0], pv[1], pv[2], pv[3]);
         }
-        psum += __shfl_xor(psum, 16, 64);
-        psum += __shfl_xor(psum, 32, 64);
+        psum = xor32_sum(xor16_sum(psum));
         l_run = l_run * alpha + psum;
         m_run = m_new;
         // ---- O^T[e][query] = alpha * O^T + V^T P^T ----------------------------------------
@@ -241,16 +239,29 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
     T* O = reinterpret_cast<T*>(p.out) + b * (int64_t)p.Nt * E;
 
     const int qrow = br * (16 * WAVES) + wave * 16 + r16;
+    // Q is scaled by inv_t * log2(e) once, so that the products come out in log2 units
+    const float c2 = p.inv_t * 1.4426950408889634f;
     Frag qf[EC];
 #pragma unroll
-    for (int c = 0; c < EC; ++c) qf[c] = Mma32<T>::load(Q + (int64_t)qrow * E + c * 32 + g4 * 8);
+    for (int c = 0; c < EC; ++c) {
+        const Frag raw = Mma32<T>::load(Q + (int64_t)qrow * E + c * 32 + g4 * 8);
+        f32x8 scaled;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) scaled[j] = (float)raw[j] * c2;
+        qf[c] = AttnPack<T>::pack(scaled);
+    }
 
     f32x4 oacc[ET];
 #pragma unroll
     for (int t = 0; t < ET; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -1e30f;
+    // The score accumulators start at -m (the reference point of this lane's query, log2
+    // units), so the MFMAs deliver the exponent of exp2 directly.  m starts at 0 and is set
+    // to the row maximum by the first block with a live entry; later it only moves when a
+    // maximum outgrows it by more than 2^RESCALE_LOG2 (numerator and denominator always
+    // share one reference).
+    f32x4 negm = f32x4{0.f, 0.f, 0.f, 0.f};
+    bool fresh = true;   // no live entry seen yet for this lane's query
     f32x4 lacc = f32x4{0.f, 0.f, 0.f, 0.f};
-    const float c2 = p.inv_t * 1.4426950408889634f;
     constexpr float RESCALE_LOG2 = 6.f;
     constexpr short ONE_BITS = sizeof(T) == 2 && Elem<T>::dtype == SPX_F16 ? (short)0x3c00 : (short)0x3f80;
     const Frag ones = __builtin_bit_cast(Frag, s16x8{ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS, ONE_BITS});
@@ -305,7 +316,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
         f32x4 s[KT];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
-            s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            s[kt] = negm;
 #pragma unroll
             for (int c = 0; c < EC; ++c) {
                 const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + (((c * 4 + g4) ^ k_sw) * 16));
@@ -323,20 +334,20 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
                     tmax = fmaxf(tmax, s[kt][q]);
                 }
             }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        // The reference point m_run only has to keep exp2 in range, so it moves (and the
-        // accumulators are rescaled) only when some query's maximum outgrows it by more
-        // than 2^RESCALE_LOG2; numerator and denominator always share one reference.
-        if (__builtin_amdgcn_ballot_w64((tmax - m_run) * c2 > RESCALE_LOG2) != 0) {
-            const float m_new = fmaxf(m_run, tmax);
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2);
-            m_run = m_new;
+        tmax = xor32_max(xor16_max(tmax));
+        const bool any_live = tmax > -1e29f;
+        if (__builtin_amdgcn_ballot_w64(any_live && (fresh || tmax > RESCALE_LOG2)) != 0) {
+            // move the reference by delta (0 for queries that keep theirs)
+            const float delta = any_live ? (fresh ? tmax : fmaxf(tmax, 0.f)) : 0.f;
+            const float alpha = __builtin_amdgcn_exp2f(-delta);
+            negm -= delta;
             lacc *= alpha;
 #pragma unroll
             for (int t = 0; t < ET; ++t) oacc[t] *= alpha;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) s[kt] -= delta;
         }
-        const float mc = m_run * c2;
+        fresh = fresh && !any_live;
         Frag pf[KT / 2];
 #pragma unroll
         for (int kp = 0; kp < KT / 2; ++kp) {
@@ -344,7 +355,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int kt = 2 * kp + (j >> 2), q = j & 3;
-                float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][q], c2, -mc));
+                float x = __builtin_amdgcn_exp2f(s[kt][q]);
                 if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
                 pv[j] = x;
             }
@@ -563,7 +574,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams 
                     tmax = fmaxf(tmax, s[kt][j]);
                 }
             }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        tmax = xor32_max(tmax);
         // m_run only has to keep exp2 in range: it moves (and the accumulators are rescaled)
         // only when some query's maximum outgrows it by more than 2^RESCALE_LOG2
         if (__builtin_amdgcn_ballot_w64((tmax - m_run) * c2 > RESCALE_LOG2) != 0) {
@@ -605,7 +616,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams 
     }
 
     // lane holds O^T[e = t*32 + 8*(j/4) + 4*h2 + j%4][query l32]; rows with no live entry give 0
-    const float l_run = l_part + __shfl_xor(l_part, 32, 64);
+    const float l_run = xor32_sum(l_part);
     const float inv_l = l_run > 0.f ? 1.f / l_run : 0.f;
 #pragma unroll
     for (int t = 0; t < ET; ++t)
@@ -790,8 +801,7 @@ __global__ __launch_bounds__(TB * 4) void attention_seqlen_kernel(SeqlenParams p
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 if (key0 + kt * 16 + g4 * 4 + q < L) tmax = fmaxf(tmax, s[kt][q]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        tmax = xor32_max(xor16_max(tmax));
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = __expf((m_run - m_new) * p.inv_t);
         float psum = 0.f;
@@ -806,8 +816,7 @@ __global__ __launch_bounds__(TB * 4) void attention_seqlen_kernel(SeqlenParams p
             }
             pf[kt] = AttnMma<T>::pack(pv[0], pv[1], pv[2], pv[3]);
         }
-        psum += __shfl_xor(psum, 16, 64);
-        psum += __shfl_xor(psum, 32, 64);
+        psum = xor32_sum(xor16_sum(psum));
         l_run = l_run * alpha + psum;
         m_run = m_new;
 #pragma unroll

@@ -108,6 +108,23 @@ __device__ __forceinline__ float row16_reduce_sum(float v) {
     return v;
 }
 
+// Exchanges between the four 16-lane rows of a wavefront on the VALU (gfx950 lane swaps,
+// no LDS round trip): after the call a holds [row0, row0, row2, row2] and b holds
+// [row1, row1, row3, row3] of the input (16), or [low half, low half] and
+// [high half, high half] (32).  Written as assembly because the compiler folds the
+// corresponding builtin when both operands carry the same value.
+__device__ __forceinline__ void swap_rows16(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_halves32(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+// max / sum over the lanes l, l^16, l^32, l^48 (every lane gets the result)
+__device__ __forceinline__ float xor16_max(float v) { float a = v, b = v; swap_rows16(a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float xor32_max(float v) { float a = v, b = v; swap_halves32(a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float xor16_sum(float v) { float a = v, b = v; swap_rows16(a, b); return a + b; }
+__device__ __forceinline__ float xor32_sum(float v) { float a = v, b = v; swap_halves32(a, b); return a + b; }
+
 __device__ __forceinline__ float wave_reduce_max(float v) {
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) v = fmaxf(v, __shfl_xor(v, d, 64));
