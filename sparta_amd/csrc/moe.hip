@@ -371,431 +371,12 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
     }
 }
 
-// ---- gathered GEMM, 256 x 128 tiles with register prefetch ---------------------------
-// Same tile lookup and LDS layout as moe_gemm_kernel; the workgroup tile is 256 token
-// rows x 128 output columns (wave w owns rows 64w .. 64w+63), and the global loads of
-// K-stage s+1 are in flight (in registers) while stage s feeds the MFMAs, so HBM/L2
-// latency overlaps with the matrix cores.  Two workgroups fit on a CU.
-
-// TM x TN: workgroup tile; WGM: wavefronts along the token dimension (4 / WGM along the
-// output dimension); OCC: workgroups per CU the register budget is sized for.
-template <typename T, int TM, int TN, int WGM, int OCC, int WAVES = 4>
-__global__ __launch_bounds__(64 * WAVES, OCC) void moe_gemm_kernel_v2(MoeParams p) {
-    constexpr int MOE2_TM = TM, MOE2_TN = TN;
-    constexpr int WGN = WAVES / WGM;
-    constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
-    constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
-    constexpr int VE = 16 / (int)sizeof(T);
-    constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
-    constexpr int A_LOADS = MOE2_TM * 8 / (64 * WAVES);
-    constexpr int B_LOADS = MOE2_TN * 8 / (64 * WAVES);
-    constexpr int RSTEP2 = 8 * WAVES;   // tile rows between a thread's vectors
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    __shared__ __align__(16) char As[MOE2_TM * 128];
-    __shared__ __align__(16) char Bs[MOE2_TN * 128];
-    __shared__ int s_expert, s_row0, s_rows;
-
-    if (threadIdx.x < 64) {
-        const int lane = threadIdx.x;
-        const int y = blockIdx.y;
-        int tiles_before = 0;
-        int found_e = -1, found_row0 = 0, found_rows = 0;
-        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
-            const int e = e0 + lane;
-            int cnt = 0, off = 0;
-            if (e < p.n_exp) {
-                off = p.expert_offset[e];
-                cnt = p.expert_offset[e + 1] - off;
-            }
-            const int tiles = (cnt + MOE2_TM - 1) / MOE2_TM;
-            const int inc = wave_inclusive_scan(tiles);
-            const int excl = tiles_before + inc - tiles;
-            const bool mine = y >= excl && y < excl + tiles;
-            const unsigned long long hit = __ballot(mine);
-            if (hit) {
-                const int src = __ffsll((long long)hit) - 1;
-                const int lt = y - __shfl(excl, src, 64);
-                found_e = e0 + src;
-                found_row0 = __shfl(off, src, 64) + lt * MOE2_TM;
-                found_rows = min(MOE2_TM, __shfl(cnt, src, 64) - lt * MOE2_TM);
-            }
-            tiles_before += __shfl(inc, 63, 64);
-        }
-        if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
-    }
-    __syncthreads();
-    const int expert = s_expert;
-    if (expert < 0) return;
-    const int row0 = s_row0, rows = s_rows;
-    const int n0 = blockIdx.x * MOE2_TN;
-
-    const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
-    const int r16 = lane & 15, g4 = lane >> 4;
-    const int wm = wave / WGN, wn = wave % WGN;
-    const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
-
-    const T* X = reinterpret_cast<const T*>(p.tokens);
-    const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
-
-    // staging map: chunk = tid % 8, rows tid / 8 + 32 q
-    const int chunk = threadIdx.x & 7;
-    const int srow = threadIdx.x >> 3;
-    const T* a_src[A_LOADS];
-    int a_dst[A_LOADS];
-#pragma unroll
-    for (int q = 0; q < A_LOADS; ++q) {
-        const int r = srow + RSTEP2 * q;
-        const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
-        a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
-        a_dst[q] = moe_lds_off<T>(r, chunk);
-    }
-    const T* b_src[B_LOADS];
-    int b_dst[B_LOADS];
-#pragma unroll
-    for (int q = 0; q < B_LOADS; ++q) {
-        const int r = srow + RSTEP2 * q;
-        const int n = n0 + r < p.N ? n0 + r : p.N - 1;
-        b_src[q] = W + (int64_t)n * p.K + chunk * VE;
-        b_dst[q] = moe_lds_off<T>(r, chunk);
-    }
-
-    f32x4 acc[MT][NTT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int t = 0; t < NTT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    u32x4 ra[A_LOADS], rb[B_LOADS];
-#pragma unroll
-    for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q]);
-#pragma unroll
-    for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q]);
-
-    for (int k0 = 0; k0 < p.K; k0 += KT) {
-#pragma unroll
-        for (int q = 0; q < A_LOADS; ++q) *reinterpret_cast<u32x4*>(As + a_dst[q]) = ra[q];
-#pragma unroll
-        for (int q = 0; q < B_LOADS; ++q) *reinterpret_cast<u32x4*>(Bs + b_dst[q]) = rb[q];
-        // next stage (the last iteration re-reads the final stage; it is not used)
-        const int kn = k0 + KT < p.K ? k0 + KT : k0;
-#pragma unroll
-        for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + kn);
-#pragma unroll
-        for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + kn);
-        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the MFMAs that hide them
-        __syncthreads();
-        if constexpr (HasMma32<T>::value) {
-#pragma unroll
-            for (int kc = 0; kc < KT; kc += 32) {
-                typename Mma32<T>::frag af[MT], bf[NTT];
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-                    af[i] = *reinterpret_cast<const typename Mma32<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
-#pragma unroll
-                for (int t = 0; t < NTT; ++t)
-                    bf[t] = *reinterpret_cast<const typename Mma32<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma32<T>::mma(bf[t], af[i], acc[i][t]);
-            }
-        } else {
-#pragma unroll
-            for (int kc = 0; kc < KT; kc += 16) {
-                typename Mma16<T>::frag af[MT], bf[NTT];
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
-#pragma unroll
-                for (int t = 0; t < NTT; ++t)
-                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
-            }
-        }
-        __syncthreads();
-    }
-
-    T* out = reinterpret_cast<T*>(p.out);
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int r = wrow + i * 16 + r16;
-        if (r >= rows) continue;
-        const int tok = p.token_perm[row0 + r];
-#pragma unroll
-        for (int t = 0; t < NTT; ++t) {
-            const int n = n0 + wcol + t * 16 + g4 * 4;
-            T vals[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
-            T* dst = out + (int64_t)tok * p.N + n;
-            if (n + 4 <= p.N) {
-                if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
-                else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
-            } else {
-                for (int q = 0; q < 4; ++q)
-                    if (n + q < p.N) dst[q] = vals[q];
-            }
-        }
-    }
-}
-
-// ---- gathered GEMM, 256 x 256 tiles, eight wavefronts, two LDS buffers ------------------
-// On gfx950 a 64 x 64 wavefront tile reads as many LDS bytes per MFMA as the LDS can
-// deliver, and a 128 x 128 workgroup tile pulls twice the operand bytes through L1 that
-// a 256 x 256 one does.  Here each wavefront owns 128 x 64 outputs (12 fragment reads per
-// 32 MFMAs), K-stage s+1 sits in the second LDS buffer and stage s+2 is in flight in
-// registers while stage s feeds the matrix cores; one barrier per stage.
-template <typename T, int TM, int TN, int WAVES, int WGM>
-__global__ __launch_bounds__(64 * WAVES, (TM + TN) > 256 ? 1 : 2) void moe_gemm_kernel_v4(MoeParams p) {
-    constexpr int NTH = 64 * WAVES;
-    constexpr int WGN = WAVES / WGM;
-    constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
-    constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
-    constexpr int VE = 16 / (int)sizeof(T);
-    constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
-    constexpr int A_LOADS = TM * 8 / NTH;
-    constexpr int B_LOADS = TN * 8 / NTH;
-    constexpr int RSTEP = NTH / 8;        // tile rows between a thread's vectors (a multiple of 8)
-    constexpr int A_BYTES = TM * 128;
-    constexpr int BUF = (TM + TN) * 128;
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    extern __shared__ __align__(16) char smem[];
-    __shared__ int s_expert, s_row0, s_rows;
-
-    if (threadIdx.x < 64) {
-        const int lane = threadIdx.x;
-        const int y = blockIdx.y;
-        int tiles_before = 0;
-        int found_e = -1, found_row0 = 0, found_rows = 0;
-        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
-            const int e = e0 + lane;
-            int cnt = 0, off = 0;
-            if (e < p.n_exp) {
-                off = p.expert_offset[e];
-                cnt = p.expert_offset[e + 1] - off;
-            }
-            const int tiles = (cnt + TM - 1) / TM;
-            const int inc = wave_inclusive_scan(tiles);
-            const int excl = tiles_before + inc - tiles;
-            const bool mine = y >= excl && y < excl + tiles;
-            const unsigned long long hit = __ballot(mine);
-            if (hit) {
-                const int src = __ffsll((long long)hit) - 1;
-                const int lt = y - __shfl(excl, src, 64);
-                found_e = e0 + src;
-                found_row0 = __shfl(off, src, 64) + lt * TM;
-                found_rows = min(TM, __shfl(cnt, src, 64) - lt * TM);
-            }
-            tiles_before += __shfl(inc, 63, 64);
-        }
-        if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
-    }
-    __syncthreads();
-    const int expert = s_expert;
-    if (expert < 0) return;
-    const int row0 = s_row0, rows = s_rows;
-    const int n0 = blockIdx.x * TN;
-
-    const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
-    const int r16 = lane & 15, g4 = lane >> 4;
-    const int wm = wave / WGN, wn = wave % WGN;
-    const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
-
-    const T* X = reinterpret_cast<const T*>(p.tokens);
-    const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
-
-    // staging map: chunk = tid % 8, rows tid / 8 + RSTEP q (the swizzle only sees row % 8)
-    const int chunk = threadIdx.x & 7;
-    const int srow = threadIdx.x >> 3;
-    const int st_dst = moe_lds_off<T>(srow, chunk);
-    const T* a_src[A_LOADS];
-#pragma unroll
-    for (int q = 0; q < A_LOADS; ++q) {
-        const int r = srow + RSTEP * q;
-        const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
-        a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
-    }
-    const T* b_src[B_LOADS];
-#pragma unroll
-    for (int q = 0; q < B_LOADS; ++q) {
-        const int r = srow + RSTEP * q;
-        const int n = n0 + r < p.N ? n0 + r : p.N - 1;
-        b_src[q] = W + (int64_t)n * p.K + chunk * VE;
-    }
-
-    // 2-byte types: 32 x 32 x 16 MFMAs (twice the sustained rate of the 16 x 16 x 32 ones)
-    constexpr bool WIDE = HasMma32<T>::value;
-    constexpr int MTW = TM / WGM / 32, NTW = TN / WGN / 32;
-    const int l32 = lane & 31, h2 = lane >> 5;
-    f32x4 acc[WIDE ? 1 : MT][WIDE ? 1 : NTT];
-    f32x16 accw[WIDE ? MTW : 1][WIDE ? NTW : 1];
-#pragma unroll
-    for (int i = 0; i < (WIDE ? 1 : MT); ++i)
-#pragma unroll
-        for (int t = 0; t < (WIDE ? 1 : NTT); ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < (WIDE ? MTW : 1); ++i)
-#pragma unroll
-        for (int t = 0; t < (WIDE ? NTW : 1); ++t)
-#pragma unroll
-            for (int j = 0; j < 16; ++j) accw[i][t][j] = 0.f;
-
-    const int n_st = p.K / KT;
-    u32x4 ra[A_LOADS], rb[B_LOADS];
-#pragma unroll
-    for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q]);
-#pragma unroll
-    for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q]);
-#pragma unroll
-    for (int q = 0; q < A_LOADS; ++q) *reinterpret_cast<u32x4*>(smem + st_dst + q * RSTEP * 128) = ra[q];
-#pragma unroll
-    for (int q = 0; q < B_LOADS; ++q) *reinterpret_cast<u32x4*>(smem + A_BYTES + st_dst + q * RSTEP * 128) = rb[q];
-    {
-        const int k1 = (1 < n_st ? 1 : 0) * KT;
-#pragma unroll
-        for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + k1);
-#pragma unroll
-        for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + k1);
-    }
-    __syncthreads();
-
-    for (int s = 0; s < n_st; ++s) {
-        const char* cur = smem + (s & 1) * BUF;
-        char* nxt = smem + ((s + 1) & 1) * BUF;
-        if (s + 1 < n_st) {
-#pragma unroll
-            for (int q = 0; q < A_LOADS; ++q) *reinterpret_cast<u32x4*>(nxt + st_dst + q * RSTEP * 128) = ra[q];
-#pragma unroll
-            for (int q = 0; q < B_LOADS; ++q) *reinterpret_cast<u32x4*>(nxt + A_BYTES + st_dst + q * RSTEP * 128) = rb[q];
-        }
-        {   // stage s + 2 (clamped: the extra copies are never used)
-            const int k2 = (s + 2 < n_st ? s + 2 : n_st - 1) * KT;
-#pragma unroll
-            for (int q = 0; q < A_LOADS; ++q) ra[q] = *reinterpret_cast<const u32x4*>(a_src[q] + k2);
-#pragma unroll
-            for (int q = 0; q < B_LOADS; ++q) rb[q] = *reinterpret_cast<const u32x4*>(b_src[q] + k2);
-        }
-        // keep the loads ahead of the MFMAs: sunk below them they would be waited for at
-        // the top of the next stage with nothing left to hide their latency
-        __builtin_amdgcn_sched_barrier(0);
-        const char* As = cur;
-        const char* Bs = cur + A_BYTES;
-        if constexpr (WIDE) {
-#pragma unroll
-            for (int kc = 0; kc < KT; kc += 16) {
-                typename MmaW<T>::frag af[MTW], bf[NTW];
-#pragma unroll
-                for (int i = 0; i < MTW; ++i)
-                    af[i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + moe_lds_off<T>(wrow + i * 32 + l32, kc / VE + h2));
-#pragma unroll
-                for (int t = 0; t < NTW; ++t)
-                    bf[t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 32 + l32, kc / VE + h2));
-#pragma unroll
-                for (int i = 0; i < MTW; ++i)
-#pragma unroll
-                    for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[t], af[i], accw[i][t]);
-            }
-        } else {
-#pragma unroll
-            for (int kc = 0; kc < KT; kc += 16) {
-                typename Mma16<T>::frag af[MT], bf[NTT];
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
-#pragma unroll
-                for (int t = 0; t < NTT; ++t)
-                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int t = 0; t < NTT; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
-            }
-        }
-        __syncthreads();
-    }
-
-    T* out = reinterpret_cast<T*>(p.out);
-    if constexpr (WIDE) {
-        // the wavefront's (TM / WGM) x 64 tile leaves through LDS (free after the last
-        // barrier) as rows of 128 bytes, chunks XOR-swizzled by the row; every store
-        // instruction then writes eight complete 128-byte row segments.
-        // lane holds out[m = i*32 + lane%32][n = t*32 + 8*jj + 4*(lane/32) + q] in accw[i][t][4*jj + q]
-        static_assert(!WIDE || TN / WGN == 64, "epilogue assumes 64 output columns per wavefront");
-        constexpr int WR = TM / WGM;
-        char* ep = smem + wave * (WR * 128);
-#pragma unroll
-        for (int i = 0; i < MTW; ++i)
-#pragma unroll
-            for (int t = 0; t < NTW; ++t)
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) {
-                    T vals[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(accw[i][t][4 * jj + q]);
-                    const int row = i * 32 + l32;
-                    const int ch = t * 4 + jj;
-                    *reinterpret_cast<uint64_t*>(ep + row * 128 + ((ch ^ (row & 7)) << 4) + h2 * 8) =
-                        *reinterpret_cast<const uint64_t*>(vals);
-                }
-        const int c = lane & 7;
-        const int n = n0 + wcol + c * 8;
-#pragma unroll
-        for (int pass = 0; pass < WR / 8; ++pass) {
-            const int row = pass * 8 + (lane >> 3);
-            const int r = wrow + row;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * 128 + ((c ^ (row & 7)) << 4));
-            if (r < rows && n < p.N) {
-                const int tok = p.token_perm[row0 + r];
-                *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
-            }
-        }
-    } else {
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        const int r = wrow + i * 16 + r16;
-        if (r >= rows) continue;
-        const int tok = p.token_perm[row0 + r];
-#pragma unroll
-        for (int t = 0; t < NTT; ++t) {
-            const int n = n0 + wcol + t * 16 + g4 * 4;
-            T vals[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[i][t][q]);
-            T* dst = out + (int64_t)tok * p.N + n;
-            if (n + 4 <= p.N) {
-                *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
-            } else {
-                for (int q = 0; q < 4; ++q)
-                    if (n + q < p.N) dst[q] = vals[q];
-            }
-        }
-    }
-    }
-}
-
-template <typename T, int TM, int TN, int WAVES>
-static int launch_moe_v4(const MoeParams& p, hipStream_t st) {
-    const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp;
-    if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
-    const int smem = 2 * (TM + TN) * 128;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel_v4<T, TM, TN, WAVES, 2>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_kernel_v4)");
-    hipLaunchKernelGGL((moe_gemm_kernel_v4<T, TM, TN, WAVES, 2>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
-    SPX_LAUNCH_CHECK("moe_gemm_kernel_v4");
-    return 0;
-}
-
 // ---- gathered GEMM with LDS-direct loads ------------------------------------------------
-// Same tiles as moe_gemm_kernel_v4, but the operands go from global memory straight into
-// LDS (global_load_lds_dwordx4: each wavefront instruction writes 64 x 16 bytes to
-// consecutive LDS addresses starting at M0), so no registers or LDS-store instructions
-// are spent on staging.  NBUF LDS buffers hold stages s .. s + NBUF - 1; one barrier per
+// Same tile lookup and LDS layout as moe_gemm_kernel (k-contiguous weights only); the
+// workgroup tile is TM x TN with WAVES wavefronts (WGM of them along the rows), and the
+// operands go from global memory straight into LDS (global_load_lds_dwordx4: each
+// wavefront instruction writes 64 x 16 bytes to consecutive LDS addresses starting at
+// M0), so no registers or LDS-store instructions are spent on staging.  NBUF LDS buffers hold stages s .. s + NBUF - 1; one barrier per
 // stage.  The loads are issued through inline assembly, which keeps the compiler from
 // serialising them against the fragment reads of the other buffers.
 __device__ __forceinline__ void lds_direct_load16(const void* g, uint32_t lds_wave_base) {
@@ -803,7 +384,7 @@ __device__ __forceinline__ void lds_direct_load16(const void* g, uint32_t lds_wa
 }
 
 template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
-__global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void moe_gemm_kernel_v5(MoeParams p) {
+__global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void moe_gemm_direct_kernel(MoeParams p) {
     constexpr int NTH = 64 * WAVES;
     constexpr int WGN = WAVES / WGM;
     constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
@@ -1024,15 +605,15 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
 }
 
 template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
-static int launch_moe_v5(const MoeParams& p, hipStream_t st) {
+static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
     const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp;
     if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
     const int smem = NBUF * (TM + TN) * 128;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_kernel_v5<T, TM, TN, WAVES, WGM, NBUF>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_kernel_v5)");
-    hipLaunchKernelGGL((moe_gemm_kernel_v5<T, TM, TN, WAVES, WGM, NBUF>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
-    SPX_LAUNCH_CHECK("moe_gemm_kernel_v5");
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_direct_kernel)");
+    hipLaunchKernelGGL((moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
+    SPX_LAUNCH_CHECK("moe_gemm_direct_kernel");
     return 0;
 }
 
@@ -1081,7 +662,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 8, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -1097,59 +678,22 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
     p.w_kcontig = weight_layout == 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    // tile_cfg 0: 7 for k-contiguous weights, else 1; 1: 128x128 tiles, no prefetch (any
-    // weight layout); 2: 256x128 tiles, 3 and 6: 128x128 tiles with the next K stage
-    // prefetched into registers; 4, 5: 256x256 and 128x128 tiles with two LDS buffers;
-    // 7, 8: 128x128 and 256x256 tiles filled by LDS-direct loads (2..8: k-contiguous
-    // weights only).  7 measured best on the benchmark shapes; the others stay selectable.
-    if (tile_cfg == 0) tile_cfg = p.w_kcontig ? 7 : 1;
-    if (tile_cfg >= 7) {
-        SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
-#define SPX_MOE5(T)                                                             \
-        if (tile_cfg == 7) return launch_moe_v5<T, 128, 128, 4, 2, 2>(p, st);   \
-        return launch_moe_v5<T, 256, 256, 8, 2, 2>(p, st);
-        switch (dtype) {
-            case SPX_F32: SPX_MOE5(float)
-            case SPX_F16: SPX_MOE5(_Float16)
-            default: SPX_MOE5(bf16_t)
-        }
-#undef SPX_MOE5
-    }
-    if (tile_cfg == 4 || tile_cfg == 5) {
-        // two LDS buffers, one barrier per stage (k-contiguous weights only):
-        // 4: 256x256 tiles, eight wavefronts; 5: 128x128 tiles, four wavefronts, two workgroups per CU
-        SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
-        if (tile_cfg == 4) {
-            switch (dtype) {
-                case SPX_F32: return launch_moe_v4<float, 256, 256, 8>(p, st);
-                case SPX_F16: return launch_moe_v4<_Float16, 256, 256, 8>(p, st);
-                default: return launch_moe_v4<bf16_t, 256, 256, 8>(p, st);
-            }
-        }
-        switch (dtype) {
-            case SPX_F32: return launch_moe_v4<float, 128, 128, 4>(p, st);
-            case SPX_F16: return launch_moe_v4<_Float16, 128, 128, 4>(p, st);
-            default: return launch_moe_v4<bf16_t, 128, 128, 4>(p, st);
-        }
-    }
+    // tile_cfg 0: 2 for k-contiguous weights, else 1; 1: 128x128 tiles staged through
+    // registers (any weight layout); 2, 3: 128x128 (four wavefronts, two workgroups per
+    // CU) and 256x256 (eight wavefronts) tiles filled by LDS-direct loads (k-contiguous
+    // weights only).  2 measured best on the benchmark shapes.
+    if (tile_cfg == 0) tile_cfg = p.w_kcontig ? 2 : 1;
     if (tile_cfg >= 2) {
         SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
-        const int tm = tile_cfg == 2 ? 256 : 128;
-        const int tiles2 = (n_tok + tm - 1) / tm + n_exp;
-        SPX_REQUIRE(tiles2 <= 65535, SPX_E_SHAPE, "too many row tiles for one launch");
-        dim3 grid2((out_dim + 127) / 128, tiles2, 1);
-#define SPX_MOE2(T)                                                                                   \
-        if (tile_cfg == 2) hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 256, 128, 4, 2>), grid2, dim3(256), 0, st, p); \
-        else if (tile_cfg == 6) hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 128, 128, 2, 2, 8>), grid2, dim3(512), 0, st, p); \
-        else hipLaunchKernelGGL((moe_gemm_kernel_v2<T, 128, 128, 2, 3>), grid2, dim3(256), 0, st, p);
+#define SPX_MOE_DIRECT(T)                                                          \
+        if (tile_cfg == 2) return launch_moe_direct<T, 128, 128, 4, 2, 2>(p, st);  \
+        return launch_moe_direct<T, 256, 256, 8, 2, 2>(p, st);
         switch (dtype) {
-            case SPX_F32: SPX_MOE2(float) break;
-            case SPX_F16: SPX_MOE2(_Float16) break;
-            default: SPX_MOE2(bf16_t) break;
+            case SPX_F32: SPX_MOE_DIRECT(float)
+            case SPX_F16: SPX_MOE_DIRECT(_Float16)
+            default: SPX_MOE_DIRECT(bf16_t)
         }
-#undef SPX_MOE2
-        SPX_LAUNCH_CHECK("moe_gemm_kernel_v2");
-        return 0;
+#undef SPX_MOE_DIRECT
     }
     const int max_tiles = (n_tok + MOE_TM - 1) / MOE_TM + n_exp;
     SPX_REQUIRE(max_tiles <= 65535, SPX_E_SHAPE, "too many row tiles for one launch");

@@ -40,13 +40,8 @@ static const spx_tile_cfg kAttentionCfgs[] = {
 static const spx_tile_cfg kMoeCfgs[] = {
     {0, 0, 0, 4, 0, 0, 7, "auto"},
     {1, 128, 128, 4, 1, 0, 7, "gather-128x128"},
-    {2, 256, 128, 4, 2, 0, 7, "gather-256x128-prefetch"},
-    {3, 128, 128, 4, 2, 0, 7, "gather-128x128-prefetch"},
-    {4, 256, 256, 8, 3, 0, 7, "gather-256x256-two-buffers"},
-    {5, 128, 128, 4, 3, 0, 7, "gather-128x128-two-buffers"},
-    {6, 128, 128, 8, 2, 0, 7, "gather-128x128-prefetch-8-waves"},
-    {7, 128, 128, 4, 2, 0, 7, "gather-128x128-lds-direct"},
-    {8, 256, 256, 8, 2, 0, 7, "gather-256x256-lds-direct"},
+    {2, 128, 128, 4, 2, 0, 7, "gather-128x128-lds-direct"},
+    {3, 256, 256, 8, 2, 0, 7, "gather-256x256-lds-direct"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {

@@ -114,7 +114,7 @@ def test_moe_weight_layouts_agree(gpu):
     assert torch.equal(out, want)
 
 
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3])
 @pytest.mark.parametrize('dtype,n_tok,in_dims,out_dims', [
     (torch.float16, 3000, 256, 520), (torch.bfloat16, 1500, 128, 256), (torch.float32, 700, 96, 136),
     (torch.float16, 5, 64, 64)])
