@@ -542,6 +542,149 @@ static int launch_dds_pipe_t_inst(const DdsParams& p, int nnz_bound, int batch, 
     return 0;
 }
 
+// ---- short-K variant: one workgroup per block row ------------------------------------------
+// When the whole K fits one or two stages (attention scores: K = head dimension) a block
+// is a single load -> MFMA -> store chain and the one-block-per-workgroup kernels are
+// bound by that latency.  Here a workgroup owns a block row: its A panel is staged once,
+// the B panel of the next live block travels in registers while the current one is
+// computed from one of two LDS buffers, and every block leaves through the shared
+// epilogue.  Needs row_ptr, k-contiguous operands and K * sizeof(T) of 128 or 256 bytes.
+template <typename T, int BM, int BN, int KB>
+__global__ __launch_bounds__(256) void dds_row_kernel(DdsParams p) {
+    constexpr int MT = BM / 16, NT = BN / 16;
+    typedef DdsWaveGrid<MT, NT> G;
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int K = KB / (int)sizeof(T);
+    constexpr int LDK = K + VE;
+    constexpr int KW = K / G::KS;
+    constexpr int CH = KB / 16;                     // 16-byte chunks per row
+    constexpr int RP = 256 / CH;                    // panel rows per pass of the workgroup
+    constexpr int NVA = BM / RP, NVB = BN / RP;     // vectors per thread for an A / a B panel
+    static_assert(BM % RP == 0 && BN % RP == 0 && KW % 16 == 0 && G::KS == 1, "panel does not split over the workgroup");
+    constexpr int PANEL_A = BM * LDK * (int)sizeof(T), PANEL_B = BN * LDK * (int)sizeof(T);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) char smem[];
+    T* As = reinterpret_cast<T*>(smem);
+    float* Ef = reinterpret_cast<float*>(smem + PANEL_A + 2 * PANEL_B);
+
+    const int bi = blockIdx.x;
+    const int e_begin = p.row_ptr[bi], e_end = p.row_ptr[bi + 1];
+    if (e_begin >= e_end) return;
+    const int64_t b = blockIdx.y;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15;
+    const int g4 = lane >> 4;
+    const int wt = wave % (G::WGM * G::WGN);
+    const int kpart = wave / (G::WGM * G::WGN);
+    const int wgm = wt / G::WGN;
+    const int wgn = wt % G::WGN;
+
+    const T* A = reinterpret_cast<const T*>(p.A) + b * p.a_batch;
+    const T* B = reinterpret_cast<const T*>(p.B) + b * p.b_batch;
+
+    const int st_row = threadIdx.x / CH, st_chunk = threadIdx.x % CH;
+    const int st_dst = (st_row * LDK + st_chunk * VE) * (int)sizeof(T);
+#pragma unroll
+    for (int u = 0; u < NVA; ++u)
+        *reinterpret_cast<u32x4*>(smem + st_dst + u * RP * LDK * (int)sizeof(T)) =
+            *reinterpret_cast<const u32x4*>(A + ((int64_t)bi * BM + st_row + RP * u) * p.a_ld + st_chunk * VE);
+
+    u32x4 rb[NVB];
+    int bj = p.idx[e_begin] & 0xffff;
+    int bj_next = p.idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
+#pragma unroll
+    for (int u = 0; u < NVB; ++u)
+        rb[u] = *reinterpret_cast<const u32x4*>(B + ((int64_t)bj * BN + st_row + RP * u) * p.b_ld + st_chunk * VE);
+
+    for (int e = e_begin; e < e_end; ++e) {
+        char* bbuf = smem + PANEL_A + ((e - e_begin) & 1) * PANEL_B;
+#pragma unroll
+        for (int u = 0; u < NVB; ++u) *reinterpret_cast<u32x4*>(bbuf + st_dst + u * RP * LDK * (int)sizeof(T)) = rb[u];
+        const int bj_cur = bj;
+        // next live block of the row (the last step re-reads its own panel; the copy is not used)
+        bj = bj_next;
+        bj_next = p.idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
+#pragma unroll
+        for (int u = 0; u < NVB; ++u)
+            rb[u] = *reinterpret_cast<const u32x4*>(B + ((int64_t)bj * BN + st_row + RP * u) * p.b_ld + st_chunk * VE);
+        __syncthreads();   // panels complete; the previous block's epilogue reads are done
+
+        f32x4 acc[G::WTM][G::WTN];
+#pragma unroll
+        for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+            for (int y = 0; y < G::WTN; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const T* a_base = As + (wgm * G::WTM * 16 + r16) * LDK + kpart * KW;
+        const T* b_base = reinterpret_cast<const T*>(bbuf) + (wgn * G::WTN * 16 + r16) * LDK + kpart * KW;
+        if constexpr (HasMma32<T>::value && KW % 32 == 0) {
+#pragma unroll
+            for (int kc = 0; kc < KW; kc += 32) {
+                typename Mma32<T>::frag af[G::WTM], bf[G::WTN];
+#pragma unroll
+                for (int x = 0; x < G::WTM; ++x) af[x] = Mma32<T>::load(a_base + x * 16 * LDK + kc + g4 * 8);
+#pragma unroll
+                for (int y = 0; y < G::WTN; ++y) bf[y] = Mma32<T>::load(b_base + y * 16 * LDK + kc + g4 * 8);
+#pragma unroll
+                for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                    for (int y = 0; y < G::WTN; ++y) acc[x][y] = Mma32<T>::mma(af[x], bf[y], acc[x][y]);
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < KW; kc += 16) {
+                typename Mma16<T>::frag af[G::WTM], bf[G::WTN];
+#pragma unroll
+                for (int x = 0; x < G::WTM; ++x) af[x] = Mma16<T>::load(a_base + x * 16 * LDK + kc + g4 * 4);
+#pragma unroll
+                for (int y = 0; y < G::WTN; ++y) bf[y] = Mma16<T>::load(b_base + y * 16 * LDK + kc + g4 * 4);
+#pragma unroll
+                for (int x = 0; x < G::WTM; ++x)
+#pragma unroll
+                    for (int y = 0; y < G::WTN; ++y) acc[x][y] = Mma16<T>::mma(af[x], bf[y], acc[x][y]);
+            }
+        }
+        // 16-byte stores of complete output rows through the shared epilogue (direct 8-byte
+        // stores from the accumulators were 15 % slower)
+        dds_epilogue<T, BM, BN>(p, acc, Ef, e, bi, bj_cur, b, wgm, wgn, kpart, r16, g4);
+    }
+}
+
+template <typename T, int BM, int BN, int KB>
+static int launch_dds_row_inst(const DdsParams& p, int batch, hipStream_t st) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int K = KB / (int)sizeof(T);
+    typedef DdsWaveGrid<BM / 16, BN / 16> G;
+    const size_t smem = (size_t)(BM + 2 * BN) * (K + VE) * sizeof(T) + (size_t)G::KS * BM * (BN + 4) * sizeof(float);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_row_kernel<T, BM, BN, KB>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(dds_row_kernel)");
+    }
+    hipLaunchKernelGGL((dds_row_kernel<T, BM, BN, KB>), dim3(p.M / BM, batch, 1), dim3(256), smem, st, p);
+    SPX_LAUNCH_CHECK("dds_row_kernel");
+    return 0;
+}
+
+// The block-row kernel covers 32 / 64-wide blocks with K * sizeof(T) of 128 or 256 bytes.
+template <typename T>
+static bool dds_row_ok(const DdsParams& p, int BM, int BN) {
+    const int kb = p.K * (int)sizeof(T);
+    return p.row_ptr && p.a_kcontig && p.b_kcontig && (kb == 128 || kb == 256) && (BM == 32 || BM == 64) &&
+           (BN == 32 || BN == 64) && p.M / BM <= 65535;
+}
+
+template <typename T>
+static int launch_dds_row(const DdsParams& p, int BM, int BN, int batch, hipStream_t st) {
+    const int kb = p.K * (int)sizeof(T);
+#define SPX_DDS_ROW_CASE(bm, bn) \
+    if (BM == bm && BN == bn) return kb == 128 ? launch_dds_row_inst<T, bm, bn, 128>(p, batch, st) \
+                                               : launch_dds_row_inst<T, bm, bn, 256>(p, batch, st);
+    SPX_DDS_ROW_CASE(32, 32) SPX_DDS_ROW_CASE(32, 64) SPX_DDS_ROW_CASE(64, 32) SPX_DDS_ROW_CASE(64, 64)
+#undef SPX_DDS_ROW_CASE
+    return fail(SPX_E_CONFIG, "the block-row kernel takes 32 / 64-wide blocks");
+}
+
 // The pipelined kernels need both operands stored the same way round (both k-contiguous,
 // or A as [K, M] and B as [K, N]) and K a multiple of the stage depth (256 bytes of k per
 // row; 128 bytes for 64 x 64 blocks).  Returns 0 (no), 1 (k-contiguous) or 2.
@@ -571,9 +714,14 @@ static int launch_dds_inst(const DdsParams& p, int nnz_bound, int batch, hipStre
 //           2 = pipelined (register ring + two LDS buffers).
 template <typename T>
 int launch_dds_impl(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, int tile_cfg, hipStream_t st) {
-    if (tile_cfg < 0 || tile_cfg > 2) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    if (tile_cfg < 0 || tile_cfg > 3) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     const int pipe = dds_pipe_ok<T>(p, BM, BN);
-    if (tile_cfg == 0) tile_cfg = pipe ? 2 : 1;
+    const bool row = dds_row_ok<T>(p, BM, BN);
+    if (tile_cfg == 0) tile_cfg = row ? 3 : (pipe ? 2 : 1);
+    if (tile_cfg == 3) {
+        if (!row) return fail(SPX_E_CONFIG, "tile config 3 needs row_ptr, k-contiguous operands, 32/64-wide blocks and K of 128 or 256 bytes");
+        return launch_dds_row<T>(p, BM, BN, batch, st);
+    }
     if (tile_cfg == 2 && !pipe)
         return fail(SPX_E_CONFIG, "tile config 2 needs both operands stored the same way round and K a multiple of the stage depth");
 #define SPX_DDS_CASE(bm, bn) \

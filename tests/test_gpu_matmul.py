@@ -129,6 +129,20 @@ def test_matmul_dds_tile_configs(tile_cfg, K, dtype, blocks, tA, tB, gpu):
              gran=(16, 16), sparsity=0.7, seed=5, tile_cfg=tile_cfg)
 
 
+@pytest.mark.parametrize('tile_cfg', [0, 3])
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('biased', [False, True])
+@pytest.mark.parametrize('dtype,blocks,K', [(torch.float16, (64, 32, 64), 64), (torch.bfloat16, (32, 32, 64), 128),
+                                            (torch.float32, (64, 32, 32), 32), (torch.float16, (32, 32, 32), 128),
+                                            (torch.float32, (32, 32, 64), 64)])
+def test_matmul_dds_block_row_kernel(tile_cfg, compressed, biased, dtype, blocks, K, gpu):
+    """Sparse-output products whose whole K is one or two stages deep (attention scores):
+    one workgroup walks the live blocks of a block row; rows without a live block, one
+    block and many."""
+    run_case(gpu, 'dds', False, True, biased, compressed, dtype, blocks, batch=3, M=448, K=K, N=320,
+             gran=(32, 32), sparsity=0.8, seed=17, tile_cfg=tile_cfg)
+
+
 @pytest.mark.parametrize('tile_cfg', [0, 7])
 @pytest.mark.parametrize('compressed', [False, True])
 @pytest.mark.parametrize('mode,tA,tB', [('dsd', False, False), ('sdd', True, True), ('dsd', True, True), ('dsd', True, False),
