@@ -210,6 +210,10 @@ template <typename T>
 int launch_spmm_panel(const SpmmParams& p, int BN, int batch, int nst, hipStream_t st);
 template <typename T>
 int launch_spmm_ksplit(const SpmmParams& p, int BN, int batch, hipStream_t st);
+template <typename T>
+bool spmm_thin_supported(const SpmmParams& p, int BN);
+template <typename T>
+int launch_spmm_thin(const SpmmParams& p, int batch, hipStream_t st);
 
 // tile_cfg: 0 = pick by layout and size;
 //   1 / 2  LDS-staged kernel, 64 / 128-row workgroup tiles (any layout);
@@ -220,6 +224,8 @@ int launch_spmm_ksplit(const SpmmParams& p, int BN, int batch, hipStream_t st);
 //          live blocks of a block-column (k-contiguous operands, BN <= 32): few rows.
 //   7      panel kernel whose four wavefronts share the sparse block through LDS (the
 //          sparse operand may be stored with n contiguous: it is transposed on the way).
+//   9      thin dense operand (64 or 128 values of m, stored with m contiguous; 16-bit
+//          types, 64-wide k-contiguous sparse blocks): one workgroup per block-column.
 template <typename T>
 int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipStream_t st) {
     const bool kcontig = p.d_kcontig && p.s_kcontig;
@@ -228,8 +234,14 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
     // ... and reads a dense operand stored with m contiguous through LDS transpose reads
     const bool panel7_ok = (p.BK * (int)sizeof(T)) % 64 == 0 &&
                            (p.d_kcontig || (p.Mc % (16 / (int)sizeof(T)) == 0 && p.d_ld % (16 / (int)sizeof(T)) == 0));
-    if (tile_cfg < 0 || tile_cfg > 8) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    if (tile_cfg < 0 || tile_cfg > 9) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     const bool ksplit_ok = panel_ok && BN <= 32;
+    const bool thin_ok = spmm_thin_supported<T>(p, BN);
+    if (tile_cfg == 0 && thin_ok) tile_cfg = 9;
+    if (tile_cfg == 9) {
+        if (!thin_ok) return fail(SPX_E_CONFIG, "tile config 9 needs a 16-bit dense operand with 64 or 128 contiguous m and 64-wide k-contiguous blocks of depth 32 / 64");
+        return launch_spmm_thin<T>(p, batch, st);
+    }
     if (tile_cfg == 0) {
         // 256-row tiles only when they still give every CU a few workgroups; small
         // problems are latency-bound and want more, shorter workgroups.

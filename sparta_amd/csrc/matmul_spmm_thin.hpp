@@ -1,0 +1,185 @@
+// Sparse-operand matmul, variant for a thin dense operand stored with m contiguous:
+// out[m, n] = sum_k D[m, k] S[k, n] with only 64 or 128 values of m, D given as
+// D[k * d_ld + m], S blocks stored with k contiguous and out as out[n * o_ld + m].
+// This is probabilities x values of an attention layer run as separate operators
+// ('sdd' with a [K, head_dim] second operand): m is the head dimension, n the queries,
+// k the keys.
+//
+// A workgroup owns one block-column (64 values of n) of one batch entry; wavefront w takes
+// its 16 n (w = 0..3) and all of m.  Per live block the S block (k-contiguous rows of the
+// 64 n, XOR-swizzled 16-byte chunks) and the D tile (BK k-rows of m, padded pitch) travel
+// global -> registers -> one of two LDS buffers, one barrier per block; S fragments are
+// plain 16-byte reads, D fragments come from the LDS transpose read of gfx950 (in a 16-lane
+// group lane i addresses 4 consecutive m of k-row i / 4, lane j receives column j of the
+// four rows).  The products are taken as  out^T-tile[m][n] += D-frag x S-frag, so a lane ends
+// up with four consecutive m of one n and stores them as 8 bytes.  Workgroups are numbered so
+// that all block-columns of one batch entry run on one XCD and find its D there.
+#pragma once
+#include "matmul_spmm.hpp"
+
+namespace spx {
+
+template <typename T, int MC, int BK>
+__global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, int batch) {
+    static_assert(sizeof(T) == 2, "16-bit element types only");
+    constexpr int BN = 64;
+    constexpr int MT = MC / 16;                 // 16-wide tiles of m
+    constexpr int KS = BK / 32;                 // 32-deep MFMA steps per block
+    constexpr int SP = BK * 2;                  // S row pitch in bytes
+    constexpr int CPR = SP / 16;                // 16-byte chunks per S row (4 or 8)
+    constexpr int VP = MC * 2 + 32;             // D row pitch in bytes
+    constexpr int S_BYTES = BN * SP;
+    constexpr int TILE = S_BYTES + BK * VP;
+    constexpr int NVS = BN * CPR / 256;         // vectors per thread: S block
+    constexpr int DPR = MC / 8;                 // 16-byte chunks per D row
+    constexpr int NVD = BK * DPR / 256;         // vectors per thread: D tile
+    static_assert(NVS >= 1 && NVD >= 1, "tile does not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    __shared__ __align__(16) char smem[2 * TILE];
+
+    // workgroup L runs on XCD L % 8: give each XCD whole batch entries
+    const int L = blockIdx.x;
+    const int slot_l = L >> 3;
+    const int64_t b = (slot_l / nb) * 8 + (L & 7);
+    const int j = slot_l % nb;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* D = reinterpret_cast<const T*>(p.D) + b * p.d_batch;
+    const T* S = reinterpret_cast<const T*>(p.S) + b * p.s_batch;
+
+    // staging maps
+    int s_row[NVS], s_chunk[NVS], s_dst[NVS];
+#pragma unroll
+    for (int i = 0; i < NVS; ++i) {
+        const int v = threadIdx.x + i * 256;
+        s_row[i] = v / CPR;
+        s_chunk[i] = v % CPR;
+        const int swz = CPR == 8 ? (s_row[i] & 7) : ((s_row[i] >> 2) & 3);
+        s_dst[i] = s_row[i] * SP + ((s_chunk[i] ^ swz) << 4);
+    }
+    int d_row[NVD], d_chunk[NVD];
+#pragma unroll
+    for (int i = 0; i < NVD; ++i) {
+        const int v = threadIdx.x + i * 256;
+        d_row[i] = v / DPR;
+        d_chunk[i] = v % DPR;
+    }
+    const int64_t sld = p.compressed ? BK : p.s_ld;
+
+    // fragment bases
+    const int f_row = wave * 16 + r16;
+    const int f_swz = CPR == 8 ? (f_row & 7) : ((f_row >> 2) & 3);
+    const int v_src = S_BYTES + (g4 * 8 + (r16 >> 2)) * VP + (r16 & 3) * 8;
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int e_begin = p.ptr[j];
+    const int e_end = p.ptr[j + 1];
+    auto entry = [&](int e, int& kb, int64_t& slot) {
+        if (p.idx_kind == SPX_IDX_BCSC_I64) {
+            const long long v = reinterpret_cast<const long long*>(p.idx)[e];
+            kb = (int)(v & 0xffff);
+            slot = v >> 32;
+        } else {
+            kb = reinterpret_cast<const int32_t*>(p.idx)[e] & 0xffff;
+            slot = e;
+        }
+    };
+    u32x4 sr[NVS], dr[NVD];
+    auto issue = [&](int kb, int64_t slot) {
+        const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN) : S + (int64_t)j * BN * p.s_ld + (int64_t)kb * BK;
+#pragma unroll
+        for (int i = 0; i < NVS; ++i) sr[i] = *reinterpret_cast<const u32x4*>(sblk + s_row[i] * sld + s_chunk[i] * 8);
+#pragma unroll
+        for (int i = 0; i < NVD; ++i)
+            dr[i] = *reinterpret_cast<const u32x4*>(D + ((int64_t)kb * BK + d_row[i]) * p.d_ld + d_chunk[i] * 8);
+    };
+    // (kb, slot) of the block in the staging registers and of the one after it, fetched a
+    // whole step before its address is needed
+    int kb = 0, kb_next = 0;
+    int64_t slot = 0, slot_next = 0;
+    if (e_begin < e_end) {
+        entry(e_begin, kb, slot);
+        entry(e_begin + 1 < e_end ? e_begin + 1 : e_begin, kb_next, slot_next);
+        issue(kb, slot);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        char* buf = smem + ((e - e_begin) & 1) * TILE;
+#pragma unroll
+        for (int i = 0; i < NVS; ++i) *reinterpret_cast<u32x4*>(buf + s_dst[i]) = sr[i];
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) *reinterpret_cast<u32x4*>(buf + S_BYTES + d_row[i] * VP + d_chunk[i] * 16) = dr[i];
+        // next live block (the last step re-reads its own block; the copy is not used)
+        kb = kb_next; slot = slot_next;
+        entry(e + 2 < e_end ? e + 2 : e_end - 1, kb_next, slot_next);
+        issue(kb, slot);
+        __syncthreads();   // the tile is complete; everyone is done with the buffer written next
+
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
+            const Frag sf = *reinterpret_cast<const Frag*>(buf + f_row * SP + ((((c * 4 + g4) ^ f_swz) & (CPR - 1)) << 4));
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + v_src + (c * 32) * VP + t * 32));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + v_src + (c * 32 + 4) * VP + t * 32));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                acc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), sf, acc[t]);
+            }
+        }
+    }
+
+    // lane holds out[m = t*16 + g4*4 + q][n = j*BN + wave*16 + r16]
+    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
+    T* out = reinterpret_cast<T*>(p.out) + b * p.o_batch;
+    const int n = j * BN + f_row;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        T vals[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float v = acc[t][q];
+            if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? t * 16 + g4 * 4 + q : n]);
+            vals[q] = Elem<T>::from_float(v);
+        }
+        *reinterpret_cast<uint64_t*>(out + (int64_t)n * p.o_ld + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+    }
+}
+
+// 16-bit types, 64 or 128 values of m stored contiguously (D[k * d_ld + m], out[n * o_ld + m]),
+// k-contiguous 64-wide sparse blocks of depth 32 or 64.
+template <typename T>
+bool spmm_thin_ok(const SpmmParams& p, int BN) {
+    if (sizeof(T) != 2) return false;
+    return !p.d_kcontig && p.s_kcontig && !p.out_ncontig && (p.Mc == 64 || p.Mc == 128) && BN == 64 &&
+           (p.BK == 32 || p.BK == 64) && p.d_ld % 8 == 0 && p.o_ld % 4 == 0 && (p.compressed || p.s_ld % 8 == 0) &&
+           p.d_batch % 8 == 0 && p.s_batch % 8 == 0 && p.o_batch % 4 == 0;
+}
+
+template <typename T>
+int launch_spmm_thin_impl(const SpmmParams& p, int batch, hipStream_t st) {
+    if constexpr (sizeof(T) == 2) {
+        const int nb = p.Nc / 64;
+        const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nb;
+        if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+#define SPX_THIN_CASE(mc, bk)                                                                                     \
+        if (p.Mc == mc && p.BK == bk) {                                                                           \
+            hipLaunchKernelGGL((spmm_thin_kernel<T, mc, bk>), dim3((unsigned)groups), dim3(256), 0, st, p, nb, batch); \
+            SPX_LAUNCH_CHECK("spmm_thin_kernel");                                                                 \
+            return 0;                                                                                             \
+        }
+        SPX_THIN_CASE(64, 32) SPX_THIN_CASE(64, 64) SPX_THIN_CASE(128, 32) SPX_THIN_CASE(128, 64)
+#undef SPX_THIN_CASE
+    }
+    return fail(SPX_E_CONFIG, "the thin-operand kernel takes 16-bit types, 64 or 128 contiguous m and 64-wide blocks of depth 32 / 64");
+}
+
+}  // namespace spx

@@ -19,6 +19,7 @@ static const spx_tile_cfg kSpmmCfgs[] = {
     {6, 256, 0, 4, 3, 16, 7, "panel-256x3"},
     {7, 256, 0, 4, 2, 16, 7, "panel-256-sharedS"},
     {8, 64, 0, 4, 2, 16, 7, "panel-64-ksplit"},
+    {9, 64, 0, 4, 2, 64, 6, "thin-dense-operand"},
 };
 static const spx_tile_cfg kDdsCfgs[] = {
     {0, 0, 0, 4, 1, 16, 7, "auto"},
