@@ -1,9 +1,9 @@
 // Sparse-operand matmul, variant for a thin dense operand stored with m contiguous:
 // out[m, n] = sum_k D[m, k] S[k, n] with only 64 or 128 values of m, D given as
-// D[k * d_ld + m], S blocks stored with k contiguous and out as out[n * o_ld + m].
+// D[k * d_ld + m], out as out[n * o_ld + m], S blocks in either storage order.
 // This is probabilities x values of an attention layer run as separate operators
-// ('sdd' with a [K, head_dim] second operand): m is the head dimension, n the queries,
-// k the keys.
+// ('sdd' with a [K, head_dim] second operand: m is the head dimension, n the queries,
+// k the keys) and, with the sparse operand transposed, the gradient of the values.
 //
 // A workgroup owns one block-column (64 values of n) of one batch entry; wavefront w takes
 // its 16 n (w = 0..3) and all of m.  Per live block the S block (k-contiguous rows of the
@@ -19,18 +19,20 @@
 
 namespace spx {
 
-template <typename T, int MC, int BK>
+// ST: the sparse blocks are stored with n contiguous ([k][n], the layout a transposed sparse
+// operand has); their fragments then come from transpose reads as well.
+template <typename T, int MC, int BK, bool ST>
 __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, int batch) {
     static_assert(sizeof(T) == 2, "16-bit element types only");
     constexpr int BN = 64;
     constexpr int MT = MC / 16;                 // 16-wide tiles of m
     constexpr int KS = BK / 32;                 // 32-deep MFMA steps per block
-    constexpr int SP = BK * 2;                  // S row pitch in bytes
-    constexpr int CPR = SP / 16;                // 16-byte chunks per S row (4 or 8)
+    constexpr int SP = ST ? BN * 2 + 32 : BK * 2;   // S row pitch in bytes ([k][n] rows are padded)
+    constexpr int CPR = (ST ? BN : BK) * 2 / 16;    // 16-byte chunks per stored S row (4 or 8)
     constexpr int VP = MC * 2 + 32;             // D row pitch in bytes
-    constexpr int S_BYTES = BN * SP;
+    constexpr int S_BYTES = (ST ? BK : BN) * SP;
     constexpr int TILE = S_BYTES + BK * VP;
-    constexpr int NVS = BN * CPR / 256;         // vectors per thread: S block
+    constexpr int NVS = BN * BK / 8 / 256;      // vectors per thread: S block
     constexpr int DPR = MC / 8;                 // 16-byte chunks per D row
     constexpr int NVD = BK * DPR / 256;         // vectors per thread: D tile
     static_assert(NVS >= 1 && NVD >= 1, "tile does not split over the workgroup");
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
         const int v = threadIdx.x + i * 256;
         s_row[i] = v / CPR;
         s_chunk[i] = v % CPR;
-        const int swz = CPR == 8 ? (s_row[i] & 7) : ((s_row[i] >> 2) & 3);
+        const int swz = ST ? 0 : (CPR == 8 ? (s_row[i] & 7) : ((s_row[i] >> 2) & 3));
         s_dst[i] = s_row[i] * SP + ((s_chunk[i] ^ swz) << 4);
     }
     int d_row[NVD], d_chunk[NVD];
@@ -71,12 +73,13 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
         d_row[i] = v / DPR;
         d_chunk[i] = v % DPR;
     }
-    const int64_t sld = p.compressed ? BK : p.s_ld;
+    const int64_t sld = p.compressed ? (ST ? BN : BK) : p.s_ld;
 
     // fragment bases
     const int f_row = wave * 16 + r16;
     const int f_swz = CPR == 8 ? (f_row & 7) : ((f_row >> 2) & 3);
     const int v_src = S_BYTES + (g4 * 8 + (r16 >> 2)) * VP + (r16 & 3) * 8;
+    const int st_src = (g4 * 8 + (r16 >> 2)) * SP + (wave * 16 + (r16 & 3) * 4) * 2;   // ST: transpose read of the S tile
 
     f32x4 acc[MT];
 #pragma unroll
@@ -96,7 +99,9 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
     };
     u32x4 sr[NVS], dr[NVD];
     auto issue = [&](int kb, int64_t slot) {
-        const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN) : S + (int64_t)j * BN * p.s_ld + (int64_t)kb * BK;
+        const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN)
+                      : ST           ? S + (int64_t)kb * BK * p.s_ld + (int64_t)j * BN
+                                     : S + (int64_t)j * BN * p.s_ld + (int64_t)kb * BK;
 #pragma unroll
         for (int i = 0; i < NVS; ++i) sr[i] = *reinterpret_cast<const u32x4*>(sblk + s_row[i] * sld + s_chunk[i] * 8);
 #pragma unroll
@@ -126,7 +131,14 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
 
 #pragma unroll
         for (int c = 0; c < KS; ++c) {
-            const Frag sf = *reinterpret_cast<const Frag*>(buf + f_row * SP + ((((c * 4 + g4) ^ f_swz) & (CPR - 1)) << 4));
+            Frag sf;
+            if constexpr (ST) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + st_src + (c * 32) * SP));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + st_src + (c * 32 + 4) * SP));
+                sf = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            } else {
+                sf = *reinterpret_cast<const Frag*>(buf + f_row * SP + ((((c * 4 + g4) ^ f_swz) & (CPR - 1)) << 4));
+            }
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + v_src + (c * 32) * VP + t * 32));
@@ -155,11 +167,11 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
 }
 
 // 16-bit types, 64 or 128 values of m stored contiguously (D[k * d_ld + m], out[n * o_ld + m]),
-// k-contiguous 64-wide sparse blocks of depth 32 or 64.
+// 64-wide sparse blocks of depth 32 or 64 in either storage order.
 template <typename T>
 bool spmm_thin_ok(const SpmmParams& p, int BN) {
     if (sizeof(T) != 2) return false;
-    return !p.d_kcontig && p.s_kcontig && !p.out_ncontig && (p.Mc == 64 || p.Mc == 128) && BN == 64 &&
+    return !p.d_kcontig && !p.out_ncontig && (p.Mc == 64 || p.Mc == 128) && BN == 64 &&
            (p.BK == 32 || p.BK == 64) && p.d_ld % 8 == 0 && p.o_ld % 4 == 0 && (p.compressed || p.s_ld % 8 == 0) &&
            p.d_batch % 8 == 0 && p.s_batch % 8 == 0 && p.o_batch % 4 == 0;
 }
@@ -172,7 +184,10 @@ int launch_spmm_thin_impl(const SpmmParams& p, int batch, hipStream_t st) {
         if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
 #define SPX_THIN_CASE(mc, bk)                                                                                     \
         if (p.Mc == mc && p.BK == bk) {                                                                           \
-            hipLaunchKernelGGL((spmm_thin_kernel<T, mc, bk>), dim3((unsigned)groups), dim3(256), 0, st, p, nb, batch); \
+            if (p.s_kcontig)                                                                                      \
+                hipLaunchKernelGGL((spmm_thin_kernel<T, mc, bk, false>), dim3((unsigned)groups), dim3(256), 0, st, p, nb, batch); \
+            else                                                                                                  \
+                hipLaunchKernelGGL((spmm_thin_kernel<T, mc, bk, true>), dim3((unsigned)groups), dim3(256), 0, st, p, nb, batch); \
             SPX_LAUNCH_CHECK("spmm_thin_kernel");                                                                 \
             return 0;                                                                                             \
         }

@@ -148,12 +148,14 @@ def test_matmul_dds_block_row_kernel(tile_cfg, compressed, biased, dtype, blocks
 @pytest.mark.parametrize('biased', [False, True])
 @pytest.mark.parametrize('dtype,BK,N', [(torch.float16, 64, 64), (torch.bfloat16, 32, 64), (torch.float16, 32, 128),
                                         (torch.bfloat16, 64, 128)])
-def test_matmul_thin_dense_operand(tile_cfg, compressed, biased, dtype, BK, N, gpu):
-    """Sparse first operand times a [K, 64] / [K, 128] matrix (probabilities x values of an
-    attention layer): the kernel with one workgroup per block row of the sparse operand;
-    block rows without a live block, with one and with many; batch sizes that do not fill
-    the eight-way workgroup numbering."""
-    run_case(gpu, 'sdd', False, False, biased, compressed, dtype, (64, BK, 32), batch=5, M=448, K=320, N=N,
+@pytest.mark.parametrize('tA', [False, True])
+def test_matmul_thin_dense_operand(tile_cfg, compressed, biased, dtype, BK, N, tA, gpu):
+    """Sparse first operand (as stored, or transposed as in the gradient of the second
+    operand) times a [K, 64] / [K, 128] matrix - probabilities x values of an attention
+    layer: the kernel with one workgroup per block row of the sparse operand; block rows
+    without a live block, with one and with many; batch sizes that do not fill the
+    eight-way workgroup numbering."""
+    run_case(gpu, 'sdd', tA, False, biased, compressed, dtype, (64, BK, 32), batch=5, M=448, K=320, N=N,
              gran=(32, 32), sparsity=0.8, seed=19, tile_cfg=tile_cfg)
 
 
