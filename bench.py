@@ -129,13 +129,15 @@ def main():
     ap.add_argument('--config', default='headline',
                     help="'headline' (default, the one JSON line the harness reads) or one of c1..c5 / all: "
                          "secondary measurements of the other benchmark configurations")
+    ap.add_argument('--attention-tile-cfg', type=int, default=0,
+                    help='tile configuration of the fused attention kernel in --config c3 (0 = the library\'s choice)')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).', file=sys.stderr)
         sys.exit(2)
     if args.config != 'headline':
         import bench_configs
-        bench_configs.run(args.config, args.steps, args.warmup, time_graph, time_eager)
+        bench_configs.run(args.config, args.steps, args.warmup, time_graph, time_eager, args.attention_tile_cfg)
         return
 
     import torch

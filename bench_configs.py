@@ -28,7 +28,7 @@ def _emit(name, sec, flops=None, bytes_alg=None, extra=None):
     print(json.dumps(out), flush=True)
 
 
-def run(which, steps, warmup, time_graph, time_eager):
+def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
     import torch
     import sparta_amd as sparta
     from oracle import ops
@@ -98,7 +98,7 @@ def run(which, steps, warmup, time_graph, time_eager):
             mask = torch.from_numpy(np.kron(grid, np.ones((blk, blk), dtype=np.uint8))).to(dev)
             g = torch.Generator().manual_seed(2022)
             q, k_, v = (torch.randn((BH, N, E), generator=g).half().to(dev) for _ in range(3))
-            att = sparta.nn.SparseAttention(mask=mask)
+            att = sparta.nn.SparseAttention(mask=mask, fused_tile_cfg=attention_tile_cfg)
             mm = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 64, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 64}
             att.build({'qk/forward:C': dict(mm),
                        'sm/forward:y': {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': 64, 'BLOCK_SIZE_W_VALUE': 64, 'ROW_TILE_VALUE': 4},
@@ -108,7 +108,7 @@ def run(which, steps, warmup, time_graph, time_eager):
             flops = 2 * nnz * 2.0 * blk * blk * E * BH
             sec = timed(lambda: att(q, k_, v))
             _emit('c3 fused sparse attention 96x4096x64 fp16, 64x64 blocks', sec, flops=flops,
-                  bytes_alg=4 * BH * N * E * 2, extra={'nnz_blocks': nnz})
+                  bytes_alg=4 * BH * N * E * 2, extra={'nnz_blocks': nnz, 'tile_cfg': attention_tile_cfg})
             att._fused = False
             sec = timed(lambda: att(q, k_, v))
             _emit('c3 three-operator pipeline (dds, softmax, sdd)', sec, flops=flops)

@@ -29,11 +29,13 @@ class SparseAttention(OperatorBase):
         fused: run the single fused forward kernel when autograd is not recording
             (default True).  The three-operator pipeline is always built as well and
             is used whenever gradients are needed.
+        fused_tile_cfg: tile configuration of the fused kernel (0 = the library's choice;
+            see spx_tile_cfg_info for the others).
 
     Shape: query (B*H, N_target, E), key / value (B*H, N_source, E) -> (B*H, N_target, E).
     """
 
-    def __init__(self, mask: torch.Tensor, fused: bool = True):
+    def __init__(self, mask: torch.Tensor, fused: bool = True, fused_tile_cfg: int = 0):
         super().__init__()
         self.mask = mask
         self._Nt, self._Ns = mask.shape
@@ -42,6 +44,7 @@ class SparseAttention(OperatorBase):
         self._matmul_out = SparseBatchMatMul(A_mask=mask, transpose_A=False, transpose_B=False, compressed=True)
         self._sparse_port: Optional[PortConfig] = None
         self._fused = fused
+        self._fused_tile_cfg = int(fused_tile_cfg)
         self._fused_mask_key = None   # index object the cached element mask belongs to
         self._fused_mask = None
         self._inv_temperature = 1.0
@@ -83,7 +86,7 @@ class SparseAttention(OperatorBase):
             _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
             _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(self._fused_mask),
             float(self._inv_temperature), batch, self._Nt, self._Ns, E,
-            indexes.block_H, indexes.block_W, 0, _lib.current_stream(q.device))
+            indexes.block_H, indexes.block_W, self._fused_tile_cfg, _lib.current_stream(q.device))
         _lib.check(rc, 'spx_attention_forward')
         return out
 
