@@ -453,7 +453,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams 
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 32, EC = E / 16, ET = E / 32, KS = BW / 16;
     constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
-    constexpr int VP = E * 2 + 32;            // V row pitch in bytes
+    constexpr int VP = E * 2 + 64;            // V row pitch in bytes: a transpose read covers 4 rows x 64 bytes per 32 lanes
     constexpr int TILE = BW * (KP + VP);
     constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
     constexpr int VPR = E / 8;                // 16-byte vectors per tile row
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams 
 
 template <typename T, int BW, int E, int WAVES>
 static int launch_attention_v3_inst(const AttnParams& p, int batch, hipStream_t st) {
-    constexpr int TILE = BW * (E * 4 + 32);
+    constexpr int TILE = BW * (E * 4 + 64);
     constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
     const int nbr = p.Nt / p.BH;
     const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
