@@ -237,3 +237,31 @@ def test_matmul_headline_shape_fp16(mode, gpu):
     if mode == 'dds':
         want = want * mask
     torch.testing.assert_close(C.float(), want, rtol=1e-2, atol=1e-2)
+
+
+def _random_cases(n, seed):
+    """Seeded draws over modes, layouts, dtypes, block shapes and ragged sizes: whatever
+    kernel the dispatcher picks for each of them has to agree with the oracle."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        mode = ['sdd', 'dsd', 'dds'][rng.integers(3)]
+        dtype = [torch.float16, torch.bfloat16, torch.float32][rng.integers(3)]
+        blocks = tuple(int(x) for x in rng.choice([16, 32, 64], size=3))
+        BM, BK, BN = blocks
+        M = BM * int(rng.integers(1, 9)) * (4 if rng.random() < 0.3 else 1)
+        K = BK * int(rng.integers(1, 7))
+        N = BN * int(rng.integers(1, 9)) * (4 if rng.random() < 0.3 else 1)
+        cases.append((mode, bool(rng.integers(2)), bool(rng.integers(2)), bool(rng.integers(2)), bool(rng.integers(2)),
+                      dtype, blocks, int(rng.integers(1, 4)), M, K, N, float(rng.choice([0.0, 0.5, 0.8, 0.95])),
+                      int(rng.integers(1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize('case', _random_cases(72, 2024), ids=lambda c: f'{c[0]}-{int(c[1])}{int(c[2])}{int(c[3])}{int(c[4])}-'
+                         f'{str(c[5]).split(".")[-1]}-{c[6][0]}x{c[6][1]}x{c[6][2]}-{c[8]}x{c[9]}x{c[10]}')
+def test_matmul_random_configurations(case, gpu):
+    mode, tA, tB, biased, compressed, dtype, blocks, batch, M, K, N, sparsity, seed = case
+    gran = tuple(int(g) for g in np.random.default_rng(seed).choice([4, 8, 16], size=2))
+    run_case(gpu, mode, tA, tB, biased, compressed, dtype, blocks, batch=batch, M=M, K=K, N=N, gran=gran,
+             sparsity=sparsity, seed=seed % 1000, tile_cfg=0)
