@@ -200,6 +200,19 @@ int spx_attention_forward(int dtype, const void* q, const void* k, const void* v
                           int batch, int Nt, int Ns, int E, int BH, int BW,
                           int tile_cfg, spx_stream_t stream);
 
+/* Forward pass for training: like spx_attention_forward, and also writes the normalised
+ * probabilities in the compressed layout of the softmax operator (block e of the BCSR
+ * order at e * BH * BW, row-major inside the block; probs_batch_stride elements between
+ * batch entries), which the backward kernels read.  Replaces the three launches of
+ * SparseAttention.forward when gradients are recorded (sparse_attention.py:76-80).
+ * Query blocks 32 / 64 / 128, key blocks 32 / 64 / 128, head dims 64 / 128. */
+int spx_attention_forward_train(int dtype, const void* q, const void* k, const void* v, void* out,
+                                void* probs, int64_t probs_batch_stride,
+                                const int32_t* row_ptr, const int32_t* bcsr_idx,
+                                const uint8_t* mask, float inv_temperature,
+                                int batch, int Nt, int Ns, int E, int BH, int BW,
+                                spx_stream_t stream);
+
 /* ------------------------------------------------------------------------ *
  * Sequence-length attention: q, k, v, out are [batch, heads, N, E]; batch b
  * attends over its first seqlens[b] positions only (int32 [batch], on the

@@ -31,6 +31,8 @@ struct AttnParams {
     const uint8_t* mask;  // [Nt, Ns] or NULL
     float inv_t;
     int Nt, Ns, BH;
+    void* probs;          // training kernel: compressed probabilities, block e at e * BH * BW
+    int64_t probs_batch;  // elements between batch entries of probs
 };
 
 template <typename T> struct AttnMma;
@@ -435,6 +437,279 @@ static int launch_attention_v2(const AttnParams& p, int batch, int BW, int E, hi
     SPX_ATTN2_CASE(128, 32, 128) SPX_ATTN2_CASE(128, 64, 128) SPX_ATTN2_CASE(128, 128, 128)
 #undef SPX_ATTN2_CASE
     return fail(SPX_E_CONFIG, "the pipelined attention kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
+// ---- forward pass for training: output and probabilities in one launch --------------------
+// Gradients need the normalised probabilities P in memory (compressed like the output of
+// the softmax operator).  The kernel walks the live blocks of its block row twice with the
+// register layout of attention_kernel_v2: pass 1 computes the row maximum and the row sum
+// (scores and exp2 only: K tiles, no V); pass 2 recomputes the scores against the final
+// maximum, scales by 1 / sum, writes the rounded probabilities (8-byte pieces: a lane holds
+// 4 consecutive keys of each 16-key tile for its query) and feeds the same values to the
+// P.V MFMAs, so the output needs no final division.  One launch replaces the scores,
+// softmax and P.V operators of the forward pipeline.
+template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(AttnParams p, int nbr, int batch) {
+    constexpr int NT = 64 * WAVES;
+    constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
+    constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
+    constexpr int VP = E * 2 + 32;            // V row pitch in bytes
+    constexpr int TILE = BW * (KP + VP);
+    constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
+    constexpr int VPR = E / 8;                // 16-byte vectors per tile row
+    constexpr int NV = BW * VPR / NT;         // vectors per thread and tile
+    constexpr int RSTEP = NT / VPR;           // tile rows between a thread's vectors
+    static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    const int L = blockIdx.x;
+    const int slot = L >> 3;
+    const int64_t b = (slot / nbr) * 8 + (L & 7);
+    const int br = slot % nbr;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.Nt * E;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    const T* Vg = reinterpret_cast<const T*>(p.v) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    T* O = reinterpret_cast<T*>(p.out) + b * (int64_t)p.Nt * E;
+    T* P = reinterpret_cast<T*>(p.probs) + b * p.probs_batch;
+
+    const int qrow = br * (16 * WAVES) + wave * 16 + r16;
+    const float c2 = p.inv_t * 1.4426950408889634f;
+    Frag qf[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        const Frag raw = Mma32<T>::load(Q + (int64_t)qrow * E + c * 32 + g4 * 8);
+        f32x8 scaled;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) scaled[j] = (float)raw[j] * c2;
+        qf[c] = AttnPack<T>::pack(scaled);
+    }
+
+    const int st_row = threadIdx.x / VPR, st_chunk = threadIdx.x % VPR;
+    const int k_dst = st_row * KP + (st_chunk ^ (st_row & 7)) * 16;
+    const int v_dst = BW * KP + st_row * VP + st_chunk * 16;
+    const int k_src = r16 * KP;
+    const int k_sw = r16 & 7;
+    const int v_src = BW * KP + (g4 * 4 + (r16 >> 2)) * VP + (r16 & 3) * 8;
+
+    const int e_begin = p.row_ptr[br];
+    const int e_end = p.row_ptr[br + 1];
+    if (e_begin >= e_end) {
+        // no live block: zero output rows (uniform over the workgroup)
+#pragma unroll
+        for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = 0ull;
+        return;
+    }
+    u32x4 kr[NV], vr[NV];
+    constexpr float RESCALE_LOG2 = 6.f;
+
+    // ---- pass 1: row maximum (as -m in log2 units) and row sum ------------------------------
+    f32x4 negm = f32x4{0.f, 0.f, 0.f, 0.f};
+    bool fresh = true;
+    float l_part = 0.f;
+    {
+        int bc = p.bcsr_idx[e_begin] & 0xffff;
+        {
+            const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+        }
+        for (int e = e_begin; e < e_end; ++e) {
+            char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
+            if constexpr (NBUF == 1) __syncthreads();
+#pragma unroll
+            for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + k_dst + i * RSTEP * KP) = kr[i];
+            const int key0 = bc * BW;
+            bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+            {
+                const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+                for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+            }
+            unsigned live[KT];
+            if constexpr (HAS_MASK) {
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+                    live[kt] = *reinterpret_cast<const uint32_t*>(p.mask + (int64_t)qrow * p.Ns + key0 + kt * 16 + g4 * 4);
+            }
+            __syncthreads();
+            f32x4 s[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                s[kt] = negm;
+#pragma unroll
+                for (int c = 0; c < EC; ++c) {
+                    const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + (((c * 4 + g4) ^ k_sw) * 16));
+                    s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
+                }
+            }
+            float tmax = -1e30f;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (HAS_MASK) {
+                        if ((live[kt] >> (8 * q)) & 0xffu) tmax = fmaxf(tmax, s[kt][q]);
+                    } else {
+                        tmax = fmaxf(tmax, s[kt][q]);
+                    }
+                }
+            tmax = xor32_max(xor16_max(tmax));
+            const bool any_live = tmax > -1e29f;
+            if (__builtin_amdgcn_ballot_w64(any_live && (fresh || tmax > RESCALE_LOG2)) != 0) {
+                const float delta = any_live ? (fresh ? tmax : fmaxf(tmax, 0.f)) : 0.f;
+                negm -= delta;
+                l_part *= __builtin_amdgcn_exp2f(-delta);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) s[kt] -= delta;
+            }
+            fresh = fresh && !any_live;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float x = __builtin_amdgcn_exp2f(s[kt][q]);
+                    if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
+                    l_part += x;
+                }
+        }
+    }
+    const float l_run = xor32_sum(xor16_sum(l_part));
+    const float inv_l = l_run > 0.f ? 1.f / l_run : 0.f;
+    __syncthreads();   // everyone is done with the K tiles of pass 1
+
+    // ---- pass 2: probabilities and output ----------------------------------------------------
+    f32x4 oacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    int bc = p.bcsr_idx[e_begin] & 0xffff;
+    {
+        const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + k_dst + i * RSTEP * KP) = kr[i];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
+        const int key0 = bc * BW;
+        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        {
+            const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+        }
+        unsigned live[KT];
+        if constexpr (HAS_MASK) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+                live[kt] = *reinterpret_cast<const uint32_t*>(p.mask + (int64_t)qrow * p.Ns + key0 + kt * 16 + g4 * 4);
+        }
+        __syncthreads();
+        f32x4 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            s[kt] = negm;
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + (((c * 4 + g4) ^ k_sw) * 16));
+                s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
+            }
+        }
+        T* pblk = P + (int64_t)e * (16 * WAVES * BW) + (wave * 16 + r16) * BW + g4 * 4;
+        Frag pf[KT / 2];
+#pragma unroll
+        for (int kp = 0; kp < KT / 2; ++kp) {
+            f32x8 pv;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int kt = 2 * kp + (j >> 2), q = j & 3;
+                float x = __builtin_amdgcn_exp2f(s[kt][q]) * inv_l;
+                if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
+                pv[j] = x;
+            }
+            pf[kp] = AttnPack<T>::pack(pv);
+            const s16x8 bits = __builtin_bit_cast(s16x8, pf[kp]);
+            *reinterpret_cast<s16x4*>(pblk + (2 * kp) * 16) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
+            *reinterpret_cast<s16x4*>(pblk + (2 * kp + 1) * 16) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int kp = 0; kp < KT / 2; ++kp) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + v_src + (kp * 32) * VP + t * 32));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + v_src + (kp * 32 + 16) * VP + t * 32));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                oacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), pf[kp], oacc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T vals[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][q]);
+        *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+    }
+}
+
+template <typename T, int BW, int E, int WAVES>
+static int launch_attention_train_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr int TILE = BW * (E * 4 + 32);
+    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    const int nbr = p.Nt / p.BH;
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (p.mask) {
+        if (smem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_train_kernel<T, BW, E, WAVES, true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_train_kernel)");
+        }
+        hipLaunchKernelGGL((attention_train_kernel<T, BW, E, WAVES, true>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    } else {
+        if (smem > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_train_kernel<T, BW, E, WAVES, false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_train_kernel)");
+        }
+        hipLaunchKernelGGL((attention_train_kernel<T, BW, E, WAVES, false>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    }
+    SPX_LAUNCH_CHECK("attention_train_kernel");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_train(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTNT_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_train_inst<T, bw, e, bh / 16>(p, batch, st);
+    SPX_ATTNT_CASE(32, 32, 64) SPX_ATTNT_CASE(32, 64, 64) SPX_ATTNT_CASE(32, 128, 64)
+    SPX_ATTNT_CASE(32, 32, 128) SPX_ATTNT_CASE(32, 64, 128) SPX_ATTNT_CASE(32, 128, 128)
+    SPX_ATTNT_CASE(64, 32, 64) SPX_ATTNT_CASE(64, 64, 64) SPX_ATTNT_CASE(64, 128, 64)
+    SPX_ATTNT_CASE(64, 32, 128) SPX_ATTNT_CASE(64, 64, 128) SPX_ATTNT_CASE(64, 128, 128)
+    SPX_ATTNT_CASE(128, 64, 64) SPX_ATTNT_CASE(128, 128, 64)
+    SPX_ATTNT_CASE(128, 32, 128) SPX_ATTNT_CASE(128, 64, 128) SPX_ATTNT_CASE(128, 128, 128)
+#undef SPX_ATTNT_CASE
+    return fail(SPX_E_CONFIG, "the training forward kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
 }
 
 // ---- pipelined variant on 32 x 32 x 16 MFMAs ---------------------------------------------
@@ -893,6 +1168,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx; p.mask = mask;
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
+    p.probs = nullptr; p.probs_batch = 0;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel;
     // 3: pipelined kernel on 32x32x16 MFMAs (one wavefront per 32 queries; measured within a few
@@ -908,6 +1184,37 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     }
     if (dtype == SPX_F16) return launch_attention<_Float16>(p, batch, BW, E, st);
     return launch_attention<bf16_t>(p, batch, BW, E, st);
+}
+
+extern "C" int spx_attention_forward_train(int dtype, const void* q, const void* k, const void* v, void* out,
+                                           void* probs, int64_t probs_batch_stride,
+                                           const int32_t* row_ptr, const int32_t* bcsr_idx,
+                                           const uint8_t* mask, float inv_temperature,
+                                           int batch, int Nt, int Ns, int E, int BH, int BW,
+                                           spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
+                "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
+    SPX_REQUIRE(q && k && v && out && probs && row_ptr && bcsr_idx, SPX_E_NULL, "a required buffer is NULL");
+    SPX_REQUIRE(Nt > 0 && Ns > 0 && BH > 0 && BW > 0 && Nt % BH == 0 && Ns % BW == 0, SPX_E_SHAPE,
+                "mask shape (%d,%d) is not a multiple of the block (%d,%d)", Nt, Ns, BH, BW);
+    SPX_REQUIRE(attention_v2_supported(BH, BW, E), SPX_E_CONFIG,
+                "the training forward kernel covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 (got %d, %d, %d)", BH, BW, E);
+    SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
+    SPX_REQUIRE(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 16) && aligned(probs, 16), SPX_E_ALIGN,
+                "q, k, v, out, probs must be 16-byte aligned");
+    SPX_REQUIRE(probs_batch_stride % 8 == 0, SPX_E_ALIGN, "probs_batch_stride must be a multiple of 8 elements");
+    SPX_REQUIRE(!mask || (Ns % 4 == 0 && aligned(mask, 4)), SPX_E_ALIGN, "mask rows must be 4-byte aligned");
+    if (batch == 0) return 0;
+    AttnParams p;
+    p.q = q; p.k = k; p.v = v; p.out = out;
+    p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx; p.mask = mask;
+    p.inv_t = inv_temperature;
+    p.Nt = Nt; p.Ns = Ns; p.BH = BH;
+    p.probs = probs; p.probs_batch = probs_batch_stride;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (dtype == SPX_F16) return launch_attention_train<_Float16>(p, batch, BW, E, st);
+    return launch_attention_train<bf16_t>(p, batch, BW, E, st);
 }
 
 extern "C" int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const void* v, void* out,

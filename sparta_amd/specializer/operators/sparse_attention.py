@@ -23,6 +23,37 @@ from sparta_amd.specializer.kernels import KernelBase, PortConfig
 _PARTS = (('qk', '_matmul_qk', 'C'), ('sm', '_softmax', 'y'), ('out', '_matmul_out', 'A'))
 
 
+class _FusedAttentionFunc(torch.autograd.Function):
+    """Forward: one launch gives the output and the probabilities.  Backward: the five
+    backward kernels of the three operators, fed with the saved probabilities."""
+
+    @staticmethod
+    def forward(ctx, op: 'SparseAttention', query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
+        q, k, v = query.detach(), key.detach(), value.detach()
+        out, probs = op._fused_forward_train(q, k, v)
+        ctx.save_for_backward(q, k, v, probs)
+        ctx.op = op
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        q, k, v, probs = ctx.saved_tensors
+        op = ctx.op
+        out_ctx, qk_ctx, sm_ctx = op._matmul_out._sparse_ctx, op._matmul_qk._sparse_ctx, op._softmax._sparse_ctx
+        grad_out = grad_out.detach().contiguous()
+        grad_q = grad_k = grad_v = None
+        if ctx.needs_input_grad[3]:
+            grad_v = out_ctx.backward_B(grad_out, probs)
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            grad_probs = out_ctx.backward_A(grad_out, v)
+            grad_scores = sm_ctx.backward(grad_probs, probs)
+            if ctx.needs_input_grad[1]:
+                grad_q = qk_ctx.backward_A(grad_scores, k)
+            if ctx.needs_input_grad[2]:
+                grad_k = qk_ctx.backward_B(grad_scores, q)
+        return None, grad_q, grad_k, grad_v
+
+
 class SparseAttention(OperatorBase):
     r"""Args:
         mask: (N_target, N_source) mask of the score entries that take part.
@@ -55,12 +86,52 @@ class SparseAttention(OperatorBase):
 
     # ---- forward ---------------------------------------------------------------------
     def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
-        if self.ready and self._fused and self._fused_supported(query) and not (
-                torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)):
-            return self._fused_forward(query, key, value)
+        if self.ready and self._fused and self._fused_supported(query):
+            recording = torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)
+            if not recording:
+                return self._fused_forward(query, key, value)
+            if self._fused_train_supported(query):
+                return _FusedAttentionFunc.apply(self, query, key, value)
         scores = self._matmul_qk.forward(query, key)
         probs = self._softmax.forward(scores)
         return self._matmul_out.forward(probs, value)
+
+    def _fused_train_supported(self, query: torch.Tensor) -> bool:
+        """The training forward kernel (output and probabilities in one launch) needs the
+        block shapes it covers, 3-D inputs and the five backward kernels built."""
+        indexes = self._sparse_port.indexes
+        BH, BW, E = indexes.block_H, indexes.block_W, query.shape[-1]
+        if not (query.dim() == 3 and BH in (32, 64, 128) and BW in (32, 64, 128) and E in (64, 128) and BW * E // 8 >= BH * 4):
+            return False
+        ctxs = (self._matmul_qk._sparse_ctx, self._matmul_out._sparse_ctx)
+        return (all(hasattr(c, 'backward_A') and hasattr(c, 'backward_B') for c in ctxs)
+                and hasattr(self._softmax._sparse_ctx, 'backward'))
+
+    def _element_mask(self):
+        indexes = self._sparse_port.indexes
+        if self._fused_mask_key is not indexes:
+            # A mask that is uniform inside its blocks needs no per-element test in the
+            # kernel; decided once per index build (one synchronising comparison).
+            block_level = indexes.is_block_uniform()
+            self._fused_mask = None if block_level else indexes.raw_mask
+            self._fused_mask_key = indexes
+        return self._fused_mask
+
+    def _fused_forward_train(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
+        """(output, compressed probabilities) from spx_attention_forward_train."""
+        indexes = self._sparse_port.indexes
+        mask = self._element_mask()
+        batch, _, E = query.shape
+        q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
+        out = torch.empty_like(q)
+        probs = torch.empty((batch, indexes.block_nnz * indexes.block_H * indexes.block_W), dtype=q.dtype, device=q.device)
+        rc = _lib.load().spx_attention_forward_train(
+            _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
+            _lib.dev_ptr(probs), probs.shape[1], _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf),
+            _lib.dev_ptr(mask), float(self._inv_temperature), batch, self._Nt, self._Ns, E,
+            indexes.block_H, indexes.block_W, _lib.current_stream(q.device))
+        _lib.check(rc, 'spx_attention_forward_train')
+        return out, probs
 
     def _fused_supported(self, query: torch.Tensor) -> bool:
         """The fused kernel covers 16-bit inputs, head dims 32 / 64 / 128 and score
@@ -71,12 +142,7 @@ class SparseAttention(OperatorBase):
 
     def _fused_forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
         indexes = self._sparse_port.indexes
-        if self._fused_mask_key is not indexes:
-            # A mask that is uniform inside its blocks needs no per-element test in the
-            # kernel; decided once per index build (one synchronising comparison).
-            block_level = indexes.is_block_uniform()
-            self._fused_mask = None if block_level else indexes.raw_mask
-            self._fused_mask_key = indexes
+        self._element_mask()
         lead = query.shape[:-2]
         E = query.shape[-1]
         batch = int(np.prod(lead)) if len(lead) else 1

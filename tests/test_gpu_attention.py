@@ -162,3 +162,61 @@ def test_attention_kernel_variants(dtype, element_mask, BH, BW, E, gpu):
         _lib.check(rc, 'spx_attention_forward')
         assert_close(out, want, dtype, f'attention tile config {cfg} {dtype} {(BH, BW, E)} mask={element_mask}')
         assert float(out[:, :BH].abs().max()) == 0.0
+
+
+def train_config(bh, bw):
+    mm = lambda m, k, n: {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': m, 'BLOCK_SIZE_K_VALUE': k, 'BLOCK_SIZE_N_VALUE': n}
+    sm = {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': bh, 'BLOCK_SIZE_W_VALUE': bw, 'ROW_TILE_VALUE': 4}
+    # the score tile (bh, bw) is (BM, BN) of qk, (BM, BK) of out and of their backward kernels' sparse operands
+    return {'qk/forward:C': mm(bh, 32, bw), 'qk/backward:A': mm(bh, bw, 32), 'qk/backward:B': mm(bw, bh, 32),
+            'sm/forward:y': dict(sm), 'sm/backward:x': dict(sm),
+            'out/forward:C': mm(bh, bw, 32), 'out/backward:A': mm(bh, 32, bw), 'out/backward:B': mm(bw, bh, 32)}
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('bh,bw,E', [(64, 64, 64), (32, 64, 64), (64, 32, 128), (64, 64, 128)])
+@pytest.mark.parametrize('gran', [(1, 1), None])
+def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, gpu, H=3, Nt=256, Ns=384):
+    """With gradients recorded and the backward kernels built, the forward pass is one
+    launch that also writes the probabilities: output and the three gradients agree with
+    the three-operator pipeline and with dense fp32 autograd; empty block rows and (with an
+    element-granular mask) partly masked blocks and fully masked queries included."""
+    _, q = randn((H, Nt, E), 31, dtype)
+    _, k = randn((H, Ns, E), 32, dtype)
+    _, v = randn((H, Ns, E), 33, dtype)
+    _, g = randn((H, Nt, E), 34, dtype)
+    mask_np = ops.block_mask((Nt, Ns), gran or (bh, bw), 0.8 if gran else 0.6, seed=35)
+    mask_np[:bh] = 0            # an empty block row
+    mask_np[bh + 3] = 0         # a fully masked query inside a live block row
+    mask = torch.from_numpy(mask_np).to(gpu)
+    att = SparseAttention(mask=mask)
+    leaves = [t.to(gpu).requires_grad_(True) for t in (q, k, v)]
+    att.build(train_config(bh, bw), sample_inputs=[t.detach() for t in leaves])
+    calls = []
+    inner = att._fused_forward_train
+    att._fused_forward_train = lambda *a: (calls.append(1), inner(*a))[1]
+
+    def run(fused):
+        att._fused = fused
+        for t in leaves:
+            t.grad = None
+        out = att(*leaves)
+        out.backward(g.to(gpu))
+        return [out.detach().float()] + [t.grad.detach().float() for t in leaves]
+
+    got = run(True)
+    assert calls, 'the training forward kernel was not used'
+    piped = run(False)
+    assert len(calls) == 1
+    # dense fp32 autograd on the same (rounded) inputs
+    ref_leaves = [t.detach().float().requires_grad_(True) for t in leaves]
+    scores = ref_leaves[0] @ ref_leaves[1].transpose(1, 2) / float(np.sqrt(E))
+    scores = scores.masked_fill(mask == 0, float('-inf'))
+    probs = torch.softmax(scores, -1).nan_to_num(0.0)
+    ref_out = probs @ ref_leaves[2]
+    ref_out.backward(g.to(gpu).float())
+    want = [ref_out.detach()] + [t.grad for t in ref_leaves]
+    for name, a, b, c in zip(('out', 'grad_q', 'grad_k', 'grad_v'), got, piped, want):
+        torch.testing.assert_close(a, c, rtol=2e-2, atol=2e-2, msg=lambda m: f'{name} vs dense autograd: {m}')
+        torch.testing.assert_close(a, b, rtol=2e-2, atol=2e-2, msg=lambda m: f'{name} vs pipeline: {m}')
+    assert float(got[0][:, :bh].abs().max()) == 0.0 and float(got[0][:, bh + 3].abs().max()) == 0.0
