@@ -213,6 +213,22 @@ int spx_attention_forward_train(int dtype, const void* q, const void* k, const v
                                 int batch, int Nt, int Ns, int E, int BH, int BW,
                                 spx_stream_t stream);
 
+/* Row side of the backward pass, from the probabilities spx_attention_forward_train saved:
+ *   grad_scores = probs o (grad_out v^T - D) * inv_temperature,  D[i] = sum_e grad_out[i,e] out[i,e]
+ *   grad_q      = grad_scores k
+ * grad_scores has the compressed layout and batch stride of probs; it is the operand of the
+ * remaining product grad_k = grad_scores^T q (spx_matmul with the sparse operand transposed),
+ * as probs is of grad_v = probs^T grad_out.  Masked entries carry probs = 0 and get
+ * grad_scores = 0.  Replaces three launches of the reference's backward chain: the
+ * dense x dense -> sparse product of SparseBatchMatMul's backward, SparseSoftmax's backward
+ * and the sparse x dense product for the query gradient (sparse_attention.py:76-80 run in
+ * reverse by autograd).  Same block shapes as spx_attention_forward_train. */
+int spx_attention_backward_scores(int dtype, const void* grad_out, const void* out, const void* probs,
+                                  const void* k, const void* v, void* grad_scores, void* grad_q,
+                                  int64_t probs_batch_stride,
+                                  const int32_t* row_ptr, const int32_t* bcsr_idx, float inv_temperature,
+                                  int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
+
 /* ------------------------------------------------------------------------ *
  * Sequence-length attention: q, k, v, out are [batch, heads, N, E]; batch b
  * attends over its first seqlens[b] positions only (int32 [batch], on the

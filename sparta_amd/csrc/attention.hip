@@ -31,8 +31,11 @@ struct AttnParams {
     const uint8_t* mask;  // [Nt, Ns] or NULL
     float inv_t;
     int Nt, Ns, BH;
-    void* probs;          // training kernel: compressed probabilities, block e at e * BH * BW
-    int64_t probs_batch;  // elements between batch entries of probs
+    void* probs;          // training kernels: compressed probabilities, block e at e * BH * BW
+    int64_t probs_batch;  // elements between batch entries of probs (and of grad_scores)
+    const void* grad_out; // backward kernel: gradient of the output
+    void* grad_scores;    // backward kernel: compressed gradient of the scores (layout of probs)
+    void* grad_q;         // backward kernel: gradient of the queries
 };
 
 template <typename T> struct AttnMma;
@@ -712,6 +715,199 @@ static int launch_attention_train(const AttnParams& p, int batch, int BW, int E,
     return fail(SPX_E_CONFIG, "the training forward kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
 }
 
+// ---- backward pass, row side: gradient of the scores and of the queries ---------------------
+// With P saved by the training forward kernel, the gradient of the scores is
+//   dS = P o (dP - D) / T,   dP = dO V^T,   D[q] = sum_e dO[q, e] O[q, e],
+// and dQ = dS K.  One workgroup per block row walks its live blocks like the forward
+// kernels do, with the roles of K and V exchanged (V rows feed the first product, K is read
+// through transpose reads for the second): dP^T tiles come out of the MFMAs already reduced
+// by D (the accumulators start at -D / T, dO is scaled by 1 / T once), are multiplied by the
+// probabilities (8-byte loads of the 4 keys a lane holds per tile), written as dS in the
+// layout of P and fed to the dQ MFMAs.  Masked entries have P = 0 and so dS = 0: no mask is
+// needed.  dK and dV stay with the sparse-operand matmul kernels (dK = dS^T Q, dV = P^T dO).
+// Replaces three launches of the operator pipeline's backward (dP, softmax backward, dQ).
+template <typename T, int BW, int E, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kernel(AttnParams p, int nbr, int batch) {
+    constexpr int NT = 64 * WAVES;
+    constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
+    constexpr int RP = E * 2;                 // pitch of the row-read tile (V): 16-byte chunks XOR-swizzled by row % 8
+    constexpr int TP = E * 2 + 32;            // pitch of the transpose-read tile (K)
+    constexpr int TILE = BW * (RP + TP);
+    constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
+    constexpr int VPR = E / 8;
+    constexpr int NV = BW * VPR / NT;
+    constexpr int RSTEP = NT / VPR;
+    static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    const int L = blockIdx.x;
+    const int slot = L >> 3;
+    const int64_t b = (slot / nbr) * 8 + (L & 7);
+    const int br = slot % nbr;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* dO = reinterpret_cast<const T*>(p.grad_out) + b * (int64_t)p.Nt * E;
+    const T* O = reinterpret_cast<const T*>(p.out) + b * (int64_t)p.Nt * E;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    const T* Vg = reinterpret_cast<const T*>(p.v) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    const T* P = reinterpret_cast<const T*>(p.probs) + b * p.probs_batch;
+    T* dS = reinterpret_cast<T*>(p.grad_scores) + b * p.probs_batch;
+    T* dQ = reinterpret_cast<T*>(p.grad_q) + b * (int64_t)p.Nt * E;
+
+    const int qrow = br * (16 * WAVES) + wave * 16 + r16;
+    // dO fragments scaled by 1 / T, and D / T = sum_e dO O / T for this lane's query
+    Frag gf[EC];
+    float d_part = 0.f;
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        const Frag g_raw = Mma32<T>::load(dO + (int64_t)qrow * E + c * 32 + g4 * 8);
+        const Frag o_raw = Mma32<T>::load(O + (int64_t)qrow * E + c * 32 + g4 * 8);
+        f32x8 scaled;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            scaled[j] = (float)g_raw[j] * p.inv_t;
+            d_part += scaled[j] * (float)o_raw[j];
+        }
+        gf[c] = AttnPack<T>::pack(scaled);
+    }
+    const float d_row = xor32_sum(xor16_sum(d_part));
+    const f32x4 negd = f32x4{-d_row, -d_row, -d_row, -d_row};
+
+    f32x4 qacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) qacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int st_row = threadIdx.x / VPR, st_chunk = threadIdx.x % VPR;
+    const int r_dst = st_row * RP + (st_chunk ^ (st_row & 7)) * 16;     // V tile
+    const int t_dst = BW * RP + st_row * TP + st_chunk * 16;            // K tile
+    const int r_src = r16 * RP;
+    const int r_sw = r16 & 7;
+    const int t_src = BW * RP + (g4 * 4 + (r16 >> 2)) * TP + (r16 & 3) * 8;
+
+    const int e_begin = p.row_ptr[br];
+    const int e_end = p.row_ptr[br + 1];
+    u32x4 kr[NV], vr[NV];
+    int bc = 0;
+    if (e_begin < e_end) {
+        bc = p.bcsr_idx[e_begin] & 0xffff;
+        const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + r_dst + i * RSTEP * RP) = vr[i];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + t_dst + i * RSTEP * TP) = kr[i];
+        // this lane's probabilities of the block: 4 consecutive keys of every 16-key tile
+        const int64_t blk = (int64_t)e * (16 * WAVES * BW) + (wave * 16 + r16) * BW + g4 * 4;
+        uint2 pb[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) pb[kt] = *reinterpret_cast<const uint2*>(P + blk + kt * 16);
+        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        {
+            const int64_t off = (int64_t)bc * BW * E;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+        }
+        __syncthreads();
+
+        // ---- (dP - D)^T / T tiles: keys x this wave's 16 queries -----------------------------
+        f32x4 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            s[kt] = negd;
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag vf = *reinterpret_cast<const Frag*>(buf + r_src + kt * 16 * RP + (((c * 4 + g4) ^ r_sw) * 16));
+                s[kt] = Mma32<T>::mma(vf, gf[c], s[kt]);
+            }
+        }
+        Frag sf[KT / 2];
+#pragma unroll
+        for (int kp = 0; kp < KT / 2; ++kp) {
+            f32x8 ds;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int kt = 2 * kp + (j >> 2), q = j & 3;
+                const uint32_t word = (q & 2) ? pb[kt].y : pb[kt].x;
+                const unsigned short half = (unsigned short)((q & 1) ? word >> 16 : word & 0xffffu);
+                ds[j] = Elem<T>::to_float(__builtin_bit_cast(T, half)) * s[kt][q];
+            }
+            sf[kp] = AttnPack<T>::pack(ds);
+            const s16x8 bits = __builtin_bit_cast(s16x8, sf[kp]);
+            *reinterpret_cast<s16x4*>(dS + blk + (2 * kp) * 16) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
+            *reinterpret_cast<s16x4*>(dS + blk + (2 * kp + 1) * 16) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
+        }
+        // ---- dQ^T[e][query] += K^T dS^T ------------------------------------------------------
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int kp = 0; kp < KT / 2; ++kp) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + t_src + (kp * 32) * TP + t * 32));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + t_src + (kp * 32 + 16) * TP + t * 32));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                qacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), sf[kp], qacc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T vals[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(qacc[t][q]);
+        *reinterpret_cast<uint64_t*>(dQ + (int64_t)qrow * E + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+    }
+}
+
+template <typename T, int BW, int E, int WAVES>
+static int launch_attention_bwd_row_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr int TILE = BW * (E * 4 + 32);
+    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    const int nbr = p.Nt / p.BH;
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_row_kernel<T, BW, E, WAVES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_bwd_row_kernel)");
+    }
+    hipLaunchKernelGGL((attention_bwd_row_kernel<T, BW, E, WAVES>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    SPX_LAUNCH_CHECK("attention_bwd_row_kernel");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_bwd_row(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTNB_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_bwd_row_inst<T, bw, e, bh / 16>(p, batch, st);
+    SPX_ATTNB_CASE(32, 32, 64) SPX_ATTNB_CASE(32, 64, 64) SPX_ATTNB_CASE(32, 128, 64)
+    SPX_ATTNB_CASE(32, 32, 128) SPX_ATTNB_CASE(32, 64, 128) SPX_ATTNB_CASE(32, 128, 128)
+    SPX_ATTNB_CASE(64, 32, 64) SPX_ATTNB_CASE(64, 64, 64) SPX_ATTNB_CASE(64, 128, 64)
+    SPX_ATTNB_CASE(64, 32, 128) SPX_ATTNB_CASE(64, 64, 128) SPX_ATTNB_CASE(64, 128, 128)
+    SPX_ATTNB_CASE(128, 64, 64) SPX_ATTNB_CASE(128, 128, 64)
+    SPX_ATTNB_CASE(128, 32, 128) SPX_ATTNB_CASE(128, 64, 128) SPX_ATTNB_CASE(128, 128, 128)
+#undef SPX_ATTNB_CASE
+    return fail(SPX_E_CONFIG, "the attention backward kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
 // ---- pipelined variant on 32 x 32 x 16 MFMAs ---------------------------------------------
 // The 32 x 32 x 16 MFMA sustains about twice the rate of the 16 x 16 x 32 one on gfx950,
 // so here a wavefront owns 32 queries and every product runs on the wide shape:
@@ -1169,6 +1365,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     p.probs = nullptr; p.probs_batch = 0;
+    p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel;
     // 3: pipelined kernel on 32x32x16 MFMAs (one wavefront per 32 queries; measured within a few
@@ -1212,9 +1409,41 @@ extern "C" int spx_attention_forward_train(int dtype, const void* q, const void*
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     p.probs = probs; p.probs_batch = probs_batch_stride;
+    p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (dtype == SPX_F16) return launch_attention_train<_Float16>(p, batch, BW, E, st);
     return launch_attention_train<bf16_t>(p, batch, BW, E, st);
+}
+
+extern "C" int spx_attention_backward_scores(int dtype, const void* grad_out, const void* out, const void* probs,
+                                             const void* k, const void* v, void* grad_scores, void* grad_q,
+                                             int64_t probs_batch_stride,
+                                             const int32_t* row_ptr, const int32_t* bcsr_idx, float inv_temperature,
+                                             int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
+                "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
+    SPX_REQUIRE(grad_out && out && probs && k && v && grad_scores && grad_q && row_ptr && bcsr_idx, SPX_E_NULL,
+                "a required buffer is NULL");
+    SPX_REQUIRE(Nt > 0 && Ns > 0 && BH > 0 && BW > 0 && Nt % BH == 0 && Ns % BW == 0, SPX_E_SHAPE,
+                "mask shape (%d,%d) is not a multiple of the block (%d,%d)", Nt, Ns, BH, BW);
+    SPX_REQUIRE(attention_v2_supported(BH, BW, E), SPX_E_CONFIG,
+                "the attention backward kernel covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 (got %d, %d, %d)", BH, BW, E);
+    SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
+    SPX_REQUIRE(aligned(grad_out, 16) && aligned(out, 16) && aligned(probs, 16) && aligned(k, 16) && aligned(v, 16) &&
+                aligned(grad_scores, 16) && aligned(grad_q, 16), SPX_E_ALIGN, "buffers must be 16-byte aligned");
+    SPX_REQUIRE(probs_batch_stride % 8 == 0, SPX_E_ALIGN, "probs_batch_stride must be a multiple of 8 elements");
+    if (batch == 0) return 0;
+    AttnParams p;
+    p.q = nullptr; p.k = k; p.v = v; p.out = const_cast<void*>(out);
+    p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx; p.mask = nullptr;
+    p.inv_t = inv_temperature;
+    p.Nt = Nt; p.Ns = Ns; p.BH = BH;
+    p.probs = const_cast<void*>(probs); p.probs_batch = probs_batch_stride;
+    p.grad_out = grad_out; p.grad_scores = grad_scores; p.grad_q = grad_q;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (dtype == SPX_F16) return launch_attention_bwd_row<_Float16>(p, batch, BW, E, st);
+    return launch_attention_bwd_row<bf16_t>(p, batch, BW, E, st);
 }
 
 extern "C" int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const void* v, void* out,

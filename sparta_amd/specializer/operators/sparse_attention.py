@@ -24,33 +24,33 @@ _PARTS = (('qk', '_matmul_qk', 'C'), ('sm', '_softmax', 'y'), ('out', '_matmul_o
 
 
 class _FusedAttentionFunc(torch.autograd.Function):
-    """Forward: one launch gives the output and the probabilities.  Backward: the five
-    backward kernels of the three operators, fed with the saved probabilities."""
+    """Forward: one launch gives the output and the probabilities.  Backward: one launch
+    gives the gradients of the scores and of the queries; the key and value gradients are
+    the two transposed sparse x dense products of the matmul operators."""
 
     @staticmethod
     def forward(ctx, op: 'SparseAttention', query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
         q, k, v = query.detach(), key.detach(), value.detach()
         out, probs = op._fused_forward_train(q, k, v)
-        ctx.save_for_backward(q, k, v, probs)
+        ctx.save_for_backward(q, k, v, out, probs)
         ctx.op = op
         return out
 
     @staticmethod
     def backward(ctx, grad_out: torch.Tensor):
-        q, k, v, probs = ctx.saved_tensors
+        q, k, v, out, probs = ctx.saved_tensors
         op = ctx.op
-        out_ctx, qk_ctx, sm_ctx = op._matmul_out._sparse_ctx, op._matmul_qk._sparse_ctx, op._softmax._sparse_ctx
+        out_ctx, qk_ctx = op._matmul_out._sparse_ctx, op._matmul_qk._sparse_ctx
         grad_out = grad_out.detach().contiguous()
         grad_q = grad_k = grad_v = None
         if ctx.needs_input_grad[3]:
             grad_v = out_ctx.backward_B(grad_out, probs)
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            grad_probs = out_ctx.backward_A(grad_out, v)
-            grad_scores = sm_ctx.backward(grad_probs, probs)
-            if ctx.needs_input_grad[1]:
-                grad_q = qk_ctx.backward_A(grad_scores, k)
+            grad_scores, grad_q = op._fused_backward_scores(grad_out, out, probs, k, v)
             if ctx.needs_input_grad[2]:
                 grad_k = qk_ctx.backward_B(grad_scores, q)
+            if not ctx.needs_input_grad[1]:
+                grad_q = None
         return None, grad_q, grad_k, grad_v
 
 
@@ -98,14 +98,13 @@ class SparseAttention(OperatorBase):
 
     def _fused_train_supported(self, query: torch.Tensor) -> bool:
         """The training forward kernel (output and probabilities in one launch) needs the
-        block shapes it covers, 3-D inputs and the five backward kernels built."""
+        block shapes it covers, 3-D inputs and the matmul operators' backward kernels built."""
         indexes = self._sparse_port.indexes
         BH, BW, E = indexes.block_H, indexes.block_W, query.shape[-1]
         if not (query.dim() == 3 and BH in (32, 64, 128) and BW in (32, 64, 128) and E in (64, 128) and BW * E // 8 >= BH * 4):
             return False
         ctxs = (self._matmul_qk._sparse_ctx, self._matmul_out._sparse_ctx)
-        return (all(hasattr(c, 'backward_A') and hasattr(c, 'backward_B') for c in ctxs)
-                and hasattr(self._softmax._sparse_ctx, 'backward'))
+        return all(hasattr(c, 'backward_B') for c in ctxs)
 
     def _element_mask(self):
         indexes = self._sparse_port.indexes
@@ -132,6 +131,21 @@ class SparseAttention(OperatorBase):
             indexes.block_H, indexes.block_W, _lib.current_stream(q.device))
         _lib.check(rc, 'spx_attention_forward_train')
         return out, probs
+
+    def _fused_backward_scores(self, grad_out, out, probs, key, value):
+        """(compressed score gradient, query gradient) from spx_attention_backward_scores."""
+        indexes = self._sparse_port.indexes
+        batch, _, E = grad_out.shape
+        k, v = key.contiguous(), value.contiguous()
+        grad_scores = torch.empty_like(probs)
+        grad_q = torch.empty_like(grad_out)
+        rc = _lib.load().spx_attention_backward_scores(
+            _lib.dtype_code(grad_out.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(out), _lib.dev_ptr(probs),
+            _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(grad_scores), _lib.dev_ptr(grad_q), probs.shape[1],
+            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), float(self._inv_temperature),
+            batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W, _lib.current_stream(grad_out.device))
+        _lib.check(rc, 'spx_attention_backward_scores')
+        return grad_scores, grad_q
 
     def _fused_supported(self, query: torch.Tensor) -> bool:
         """The fused kernel covers 16-bit inputs, head dims 32 / 64 / 128 and score
