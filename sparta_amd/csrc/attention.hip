@@ -180,6 +180,27 @@ __global__ __launch_bounds__(512) void attention_kernel(AttnParams p) {
     }
 }
 
+// Store a wave's 16 x W output tile (W 2-byte elements per row, rows contiguous in memory)
+// from the MFMA layout, where lane (r16, g4) holds the four elements 16 t + 4 g4 .. + 3 of
+// row r16 as pieces[t]: the pieces pass through a wave-private LDS tile and reach memory as
+// whole 16-byte vectors.  8-byte pieces stored directly arrive as partial cache lines and
+// cost about twice the time.
+template <int W>
+__device__ __forceinline__ void wave_rows_store(char* tile, void* dst, const uint64_t* pieces) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int PP = W * 2 + 16;
+    const int lane = lane_id();
+    const int r16 = lane & 15, g4 = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < W / 16; ++t) *reinterpret_cast<uint64_t*>(tile + r16 * PP + t * 32 + g4 * 8) = pieces[t];
+#pragma unroll
+    for (int i = 0; i < W / 32; ++i) {
+        const int c = i * 64 + lane;
+        *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst) + c * 16) =
+            *reinterpret_cast<const u32x4*>(tile + (c / (W / 8)) * PP + (c % (W / 8)) * 16);
+    }
+}
+
 // ---- pipelined variant ------------------------------------------------------------------
 // Same mathematics and register layout as attention_kernel, rebuilt around the
 // instruction budget of a block step:
@@ -386,12 +407,20 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
     // every accumulator row of lacc holds the row sum of query r16
     const float l_run = lacc[0];
     const float inv_l = l_run > 0.f ? 1.f / l_run : 0.f;
+    uint64_t pieces[ET];
 #pragma unroll
     for (int t = 0; t < ET; ++t) {
         T vals[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][q] * inv_l);
-        *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+        pieces[t] = *reinterpret_cast<const uint64_t*>(vals);
+    }
+    if constexpr (WAVES * 16 * (E * 2 + 16) <= NBUF * TILE) {
+        __syncthreads();   // the K / V tiles are dead: their space carries the output tiles
+        wave_rows_store<E>(smem + wave * (16 * (E * 2 + 16)), O + (int64_t)(qrow - r16) * E, pieces);
+    } else {
+#pragma unroll
+        for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = pieces[t];
     }
 }
 
@@ -462,6 +491,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
     constexpr int VPR = E / 8;                // 16-byte vectors per tile row
     constexpr int NV = BW * VPR / NT;         // vectors per thread and tile
     constexpr int RSTEP = NT / VPR;           // tile rows between a thread's vectors
+    constexpr int PP = BW * 2 + 16;           // row pitch of a wave's private 16 x BW probability tile
+    constexpr int PN = BW / 32;               // 16-byte vectors of that tile per lane
     static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
     typedef typename Mma32<T>::frag Frag;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -504,6 +535,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
     const int k_src = r16 * KP;
     const int k_sw = r16 & 7;
     const int v_src = BW * KP + (g4 * 4 + (r16 >> 2)) * VP + (r16 & 3) * 8;
+    char* ptile = smem + NBUF * TILE + wave * (16 * PP);
+    const int pt_piece = r16 * PP + g4 * 8;
 
     const int e_begin = p.row_ptr[br];
     const int e_end = p.row_ptr[br + 1];
@@ -636,7 +669,6 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
                 s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
             }
         }
-        T* pblk = P + (int64_t)e * (16 * WAVES * BW) + (wave * 16 + r16) * BW + g4 * 4;
         Frag pf[KT / 2];
 #pragma unroll
         for (int kp = 0; kp < KT / 2; ++kp) {
@@ -650,8 +682,17 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
             }
             pf[kp] = AttnPack<T>::pack(pv);
             const s16x8 bits = __builtin_bit_cast(s16x8, pf[kp]);
-            *reinterpret_cast<s16x4*>(pblk + (2 * kp) * 16) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
-            *reinterpret_cast<s16x4*>(pblk + (2 * kp + 1) * 16) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
+            *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp) * 32) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
+            *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp + 1) * 32) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
+        }
+        // The wave's 16 rows of the block are 32 * BW contiguous bytes of P: written as whole
+        // 16-byte vectors out of the wave's private tile (8-byte pieces straight from the
+        // MFMA layout reach memory as partial lines, at half the rate).
+#pragma unroll
+        for (int i = 0; i < PN; ++i) {
+            const int c = i * 64 + lane;
+            *reinterpret_cast<u32x4*>(P + (int64_t)e * (16 * WAVES * BW) + wave * (16 * BW) + c * 8) =
+                *reinterpret_cast<const u32x4*>(ptile + (c / (BW / 8)) * PP + (c % (BW / 8)) * 16);
         }
 #pragma unroll
         for (int t = 0; t < ET; ++t) {
@@ -666,19 +707,27 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
             }
         }
     }
+    uint64_t pieces[ET];
 #pragma unroll
     for (int t = 0; t < ET; ++t) {
         T vals[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][q]);
-        *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+        pieces[t] = *reinterpret_cast<const uint64_t*>(vals);
+    }
+    if constexpr (WAVES * 16 * (E * 2 + 16) <= NBUF * TILE) {
+        __syncthreads();   // the K / V tiles are dead: their space carries the output tiles
+        wave_rows_store<E>(smem + wave * (16 * (E * 2 + 16)), O + (int64_t)(qrow - r16) * E, pieces);
+    } else {
+#pragma unroll
+        for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = pieces[t];
     }
 }
 
 template <typename T, int BW, int E, int WAVES>
 static int launch_attention_train_inst(const AttnParams& p, int batch, hipStream_t st) {
     constexpr int TILE = BW * (E * 4 + 32);
-    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    constexpr size_t smem = (2 * TILE <= 64 * 1024 ? 2 * TILE : TILE) + WAVES * 16 * (BW * 2 + 16);
     const int nbr = p.Nt / p.BH;
     const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
     if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
@@ -737,6 +786,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
     constexpr int VPR = E / 8;
     constexpr int NV = BW * VPR / NT;
     constexpr int RSTEP = NT / VPR;
+    constexpr int PP = BW * 2 + 16;           // row pitch of a wave's private 16 x BW probability tile
+    constexpr int PN = BW / 32;               // 16-byte vectors of that tile per lane
     static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
     typedef typename Mma32<T>::frag Frag;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -793,11 +844,27 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
     const int r_sw = r16 & 7;
     const int t_src = BW * RP + (g4 * 4 + (r16 >> 2)) * TP + (r16 & 3) * 8;
 
+    // A wave's 16 rows of a block are 32 * BW contiguous bytes of P (and of dS): they move
+    // between memory and the wave's private tile in LDS as whole 16-byte vectors, and
+    // between the tile and the MFMA layout (4 keys of one query per lane) as 8-byte pieces.
+    char* ptile = smem + NBUF * TILE + wave * (16 * PP);
+    int pt_vec[PN];
+#pragma unroll
+    for (int i = 0; i < PN; ++i) {
+        const int c = i * 64 + lane;
+        pt_vec[i] = (c / (BW / 8)) * PP + (c % (BW / 8)) * 16;
+    }
+    const int pt_piece = r16 * PP + g4 * 8;
+    const int64_t wave_off = (int64_t)wave * (16 * BW) + lane * 8;   // elements, inside a block
+
     const int e_begin = p.row_ptr[br];
     const int e_end = p.row_ptr[br + 1];
-    u32x4 kr[NV], vr[NV];
+    u32x4 kr[NV], vr[NV], pr[PN];
     int bc = 0;
     if (e_begin < e_end) {
+#pragma unroll
+        for (int i = 0; i < PN; ++i)
+            pr[i] = *reinterpret_cast<const u32x4*>(P + (int64_t)e_begin * (16 * WAVES * BW) + wave_off + i * 512);
         bc = p.bcsr_idx[e_begin] & 0xffff;
         const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -812,13 +879,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
         for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + r_dst + i * RSTEP * RP) = vr[i];
 #pragma unroll
         for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + t_dst + i * RSTEP * TP) = kr[i];
-        // this lane's probabilities of the block: 4 consecutive keys of every 16-key tile
-        const int64_t blk = (int64_t)e * (16 * WAVES * BW) + (wave * 16 + r16) * BW + g4 * 4;
-        uint2 pb[KT];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) pb[kt] = *reinterpret_cast<const uint2*>(P + blk + kt * 16);
-        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        for (int i = 0; i < PN; ++i) *reinterpret_cast<u32x4*>(ptile + pt_vec[i]) = pr[i];
+        const int e_next = e + 1 < e_end ? e + 1 : e;
+        bc = p.bcsr_idx[e_next] & 0xffff;
         {
+#pragma unroll
+            for (int i = 0; i < PN; ++i)
+                pr[i] = *reinterpret_cast<const u32x4*>(P + (int64_t)e_next * (16 * WAVES * BW) + wave_off + i * 512);
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
             for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
@@ -838,6 +906,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
                 s[kt] = Mma32<T>::mma(vf, gf[c], s[kt]);
             }
         }
+        // this lane's probabilities of the block: 4 consecutive keys of every 16-key tile
+        uint2 pb[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) pb[kt] = *reinterpret_cast<const uint2*>(ptile + pt_piece + kt * 32);
         Frag sf[KT / 2];
 #pragma unroll
         for (int kp = 0; kp < KT / 2; ++kp) {
@@ -851,9 +923,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
             }
             sf[kp] = AttnPack<T>::pack(ds);
             const s16x8 bits = __builtin_bit_cast(s16x8, sf[kp]);
-            *reinterpret_cast<s16x4*>(dS + blk + (2 * kp) * 16) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
-            *reinterpret_cast<s16x4*>(dS + blk + (2 * kp + 1) * 16) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
+            *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp) * 32) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
+            *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp + 1) * 32) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
         }
+#pragma unroll
+        for (int i = 0; i < PN; ++i)
+            *reinterpret_cast<u32x4*>(dS + (int64_t)e * (16 * WAVES * BW) + wave_off + i * 512) =
+                *reinterpret_cast<const u32x4*>(ptile + pt_vec[i]);
         // ---- dQ^T[e][query] += K^T dS^T ------------------------------------------------------
 #pragma unroll
         for (int t = 0; t < ET; ++t) {
@@ -868,19 +944,27 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
             }
         }
     }
+    uint64_t pieces[ET];
 #pragma unroll
     for (int t = 0; t < ET; ++t) {
         T vals[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(qacc[t][q]);
-        *reinterpret_cast<uint64_t*>(dQ + (int64_t)qrow * E + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
+        pieces[t] = *reinterpret_cast<const uint64_t*>(vals);
+    }
+    if constexpr (WAVES * 16 * (E * 2 + 16) <= NBUF * TILE) {
+        __syncthreads();   // the K / V tiles are dead: their space carries the output tiles
+        wave_rows_store<E>(smem + wave * (16 * (E * 2 + 16)), dQ + (int64_t)(qrow - r16) * E, pieces);
+    } else {
+#pragma unroll
+        for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(dQ + (int64_t)qrow * E + t * 16 + g4 * 4) = pieces[t];
     }
 }
 
 template <typename T, int BW, int E, int WAVES>
 static int launch_attention_bwd_row_inst(const AttnParams& p, int batch, hipStream_t st) {
     constexpr int TILE = BW * (E * 4 + 32);
-    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    constexpr size_t smem = (2 * TILE <= 64 * 1024 ? 2 * TILE : TILE) + WAVES * 16 * (BW * 2 + 16);
     const int nbr = p.Nt / p.BH;
     const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
     if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
