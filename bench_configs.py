@@ -115,6 +115,31 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
             qq, kk, vv = (t.view(8, 12, N, E) for t in (q, k_, v))
             sec = timed(lambda: torch.nn.functional.scaled_dot_product_attention(qq, kk, vv))
             _emit('c3 dense torch SDPA (no mask)', sec, flops=4.0 * BH * N * N * E)
+            # one training step (forward + backward, gradients of q, k, v) on the same problem
+            with torch.enable_grad():
+                sq = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 64, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 64}
+                sm = {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': 64, 'BLOCK_SIZE_W_VALUE': 64, 'ROW_TILE_VALUE': 4}
+                leaves = [t.clone().requires_grad_(True) for t in (q, k_, v)]
+                grad = torch.randn((BH, N, E), generator=g).half().to(dev)
+                att_t = sparta.nn.SparseAttention(mask=mask)
+                att_t.build({f'{part}/{pas}': dict(sq) for part in ('qk', 'out') for pas in ('forward:C', 'backward:A', 'backward:B')}
+                            | {'sm/forward:y': dict(sm), 'sm/backward:x': dict(sm)}, sample_inputs=leaves)
+
+                def step(fn):
+                    for t in leaves:
+                        t.grad = None
+                    fn(*leaves).backward(grad)
+
+                n_step = min(steps, 20)
+                for fused, name in ((True, 'c3 training step, fused forward and score-gradient kernels'),
+                                    (False, 'c3 training step, three operators forward and six kernels backward')):
+                    att_t._fused = fused
+                    sec = time_eager(torch, lambda: step(att_t), n_step, 3) / n_step
+                    _emit(name, sec, flops=3 * flops)
+                dense = lambda a, b, c: torch.nn.functional.scaled_dot_product_attention(
+                    a.view(8, 12, N, E), b.view(8, 12, N, E), c.view(8, 12, N, E)).view(BH, N, E)
+                sec = time_eager(torch, lambda: step(dense), n_step, 3) / n_step
+                _emit('c3 training step, dense torch SDPA (no mask)', sec, flops=3 * 4.0 * BH * N * N * E)
 
         if 'c4' in todo:
             T, D, F = 8192, 768, 3072
