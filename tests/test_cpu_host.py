@@ -58,6 +58,26 @@ def test_host_validation_without_gpu():
     assert rc == _lib.E_CONFIG  # BCSC index handed to a BCSR-mode kernel
     rc = lib.spx_softmax_forward(1, 0, one, one, one, one, one, 1.0, 1, 64, 64, 5, 32, 0, 0, None)
     assert rc == _lib.E_CONFIG
+    # attention entry points: dtype, null pointers, shapes and block shapes are checked before any launch
+    f16 = _lib.F16
+    rc = lib.spx_attention_forward(0, one, one, one, one, one, one, None, 0.125, 1, 256, 256, 64, 64, 64, 0, None)
+    assert rc == _lib.E_DTYPE
+    rc = lib.spx_attention_forward(f16, one, one, one, one, one, one, None, 0.125, 1, 250, 256, 64, 64, 64, 0, None)
+    assert rc == _lib.E_SHAPE
+    rc = lib.spx_attention_forward(f16, one, one, None, one, one, one, None, 0.125, 1, 256, 256, 64, 64, 64, 0, None)
+    assert rc == _lib.E_NULL
+    rc = lib.spx_attention_forward(f16, one, one, one, one, one, one, None, 0.125, 1, 256, 256, 64, 64, 64, 99, None)
+    assert rc == _lib.E_CONFIG
+    rc = lib.spx_attention_forward_train(f16, one, one, one, one, one, 4096, one, one, None, 0.125, 1, 256, 256, 48, 64, 64, None)
+    assert rc == _lib.E_CONFIG and 'head dim' in _lib.last_error()
+    rc = lib.spx_attention_forward_train(f16, one, one, one, one, None, 4096, one, one, None, 0.125, 1, 256, 256, 64, 64, 64, None)
+    assert rc == _lib.E_NULL
+    rc = lib.spx_attention_backward_scores(f16, one, one, one, one, one, one, one, 4096, one, one, 0.125, 1, 256, 256, 64, 16, 64, None)
+    assert rc == _lib.E_CONFIG
+    rc = lib.spx_attention_backward_scores(f16, one, one, one, one, one, one, one, 4100, one, one, 0.125, 1, 256, 256, 64, 64, 64, None)
+    assert rc == _lib.E_ALIGN
+    rc = lib.spx_attention_backward_scores(0, one, one, one, one, one, one, one, 4096, one, one, 0.125, 1, 256, 256, 64, 64, 64, None)
+    assert rc == _lib.E_DTYPE
     with pytest.raises(AssertionError):
         _lib.check(_lib.E_SHAPE, 'x')
     with pytest.raises(ValueError):
