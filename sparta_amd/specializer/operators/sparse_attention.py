@@ -201,11 +201,10 @@ class SparseAttention(OperatorBase):
     def build(self, config: Dict[str, Any], sample_inputs: List[torch.Tensor]):
         query, key, value = sample_inputs
         self._set_temperature(self._check_qkv(query, key, value))
-        with warnings.catch_warnings():
-            warnings.simplefilter('ignore')
-            scores = self._matmul_qk.forward(query, key)
-            probs = self._softmax.forward(scores)
-        part_inputs = {'qk': [query, key], 'sm': [scores], 'out': [probs, value]}
+        # The parts only read the shapes of their sample inputs: the dense score tensor
+        # (batch x N_target x N_source) is never materialised.
+        scores = torch.empty(tuple(query.shape[:-1]) + (self._Ns,), dtype=query.dtype, device='meta')
+        part_inputs = {'qk': [query, key], 'sm': [scores], 'out': [scores, value]}
 
         # One port (hence one index and one compressed layout) for every selected kernel.
         shared: Optional[PortConfig] = None

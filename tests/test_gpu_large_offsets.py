@@ -1,0 +1,163 @@
+"""Tensors of more than 2**31 elements: every kernel family has to form its addresses in
+64 bits.  Inputs are generated on the GPU (the CPU oracle would take minutes at these
+sizes); the check is dense fp32 torch on the batch entries / rows whose element offsets
+lie beyond 2**31, and on the first entry for contrast."""
+import numpy as np
+import pytest
+import torch
+
+from sparta_amd.nn import DynamicSparseMoE, SparseAttention
+from sparta_amd.specializer.kernels import SparTASparseMatMulKernel, SparTASparseSoftmaxForwardKernel
+from sparta_amd.tesa import get_bcs_function
+
+pytestmark = pytest.mark.gpu
+LIMIT = 2 ** 31
+
+
+def _randn(shape, seed, gpu, dtype=torch.float16):
+    g = torch.Generator(device=gpu).manual_seed(seed)
+    return torch.randn(shape, generator=g, device=gpu, dtype=torch.float32).to(dtype)
+
+
+def _block_mask(shape, block, density, seed, gpu):
+    g = torch.Generator(device=gpu).manual_seed(seed)
+    grid = torch.rand((shape[0] // block[0], shape[1] // block[1]), generator=g, device=gpu) < density
+    return grid.repeat_interleave(block[0], 0).repeat_interleave(block[1], 1).to(torch.uint8)
+
+
+def _kernel(mode, mask, batch, M, K, N, tB=True):
+    k = SparTASparseMatMulKernel(mode=mode, biased=False, transpose_A=False, transpose_B=tB, compressed=True)
+    port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
+    k.ports[port].set_mask(mask)
+    k.set_shape(batch, M, K, N)
+    k.compile({'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32})
+    return k, k.ports[port].indexes
+
+
+def test_dense_output_beyond_2g_elements(gpu, batch=4, M=16384, K=64, N=49152):
+    """dsd: the dense output [4, 16384, 49152] holds 3.2 G elements."""
+    assert (batch - 1) * M * N > LIMIT
+    x = _randn((batch, M, K), 1, gpu)
+    w = _randn((batch, N, K), 2, gpu)
+    mask = _block_mask((N, K), (32, 32), 0.5, 3, gpu)
+    kernel, indexes = _kernel('dsd', mask, batch, M, K, N)
+    out = kernel(x, indexes.convert(w * mask.half()))
+    assert out.numel() > LIMIT
+    for b in (0, batch - 1):
+        wm = (w[b] * mask.half()).float()
+        for r0 in (0, M - 2048):
+            want = x[b, r0:r0 + 2048].float() @ wm.t()
+            torch.testing.assert_close(out[b, r0:r0 + 2048].float(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize('mode', ['dds', 'sdd'])
+def test_compressed_values_beyond_2g_elements(mode, gpu, batch=3, M=32768, K=64, N=32768):
+    """A compressed operand / result of 3 x 1 M live 32 x 32 blocks (3.2 G elements): the
+    sparse-output product writes it, convert / inverse move it, the sparse-operand product
+    reads it."""
+    if mode == 'dds':
+        mask = torch.ones((M, N), dtype=torch.uint8, device=gpu)
+        mask[:64, 32:96] = 0
+        a = _randn((batch, M, K), 4, gpu)
+        b = _randn((batch, N, K), 5, gpu)
+        kernel, indexes = _kernel('dds', mask, batch, M, K, N)
+        c = kernel(a, b)
+        assert c.numel() > LIMIT and (batch - 1) * c.shape[1] > LIMIT // 2
+        for e in (0, batch - 1):
+            dense = indexes.inverse(c[e:e + 1])[0]
+            for r0 in (0, M - 1024):
+                want = (a[e, r0:r0 + 1024].float() @ b[e].float().t()) * mask[r0:r0 + 1024].float()
+                torch.testing.assert_close(dense[r0:r0 + 1024].float(), want, rtol=1e-2, atol=1e-2)
+            del dense
+    else:
+        # sdd with a [32768, 32768] sparse A (all blocks live) and a thin dense B
+        mask = torch.ones((M, N), dtype=torch.uint8, device=gpu)
+        kernel, indexes = _kernel('sdd', mask, batch, M, N, K)     # contraction over N here
+        a_vals = _randn((batch, indexes.block_nnz * 1024), 6, gpu) * 0.05
+        assert a_vals.numel() > LIMIT
+        b = _randn((batch, K, N), 7, gpu)                          # transpose_B: [n, k] with n = 64 rows
+        out = kernel(a_vals, b)
+        for e in (0, batch - 1):
+            a_dense = indexes.inverse(a_vals[e:e + 1])[0]
+            for r0 in (0, M - 1024):
+                want = a_dense[r0:r0 + 1024].float() @ b[e].float().t()
+                torch.testing.assert_close(out[e, r0:r0 + 1024].float(), want, rtol=2e-2, atol=2e-2)
+            del a_dense
+
+
+def test_softmax_beyond_2g_elements(gpu, batch=3, H=32768, W=32768):
+    mask = _block_mask((H, W), (32, 32), 0.999, 8, gpu)      # every block live with near certainty
+    kernel = SparTASparseSoftmaxForwardKernel(compressed=True)
+    kernel.ports['y'].set_mask(mask)
+    kernel.set_shape(batch, H, W)
+    kernel.compile({'BLOCK_SIZE_H_VALUE': 32, 'BLOCK_SIZE_W_VALUE': 32, 'ROW_TILE_VALUE': 4})
+    indexes = kernel.ports['y'].indexes
+    x = _randn((batch, indexes.block_nnz * 1024), 9, gpu)
+    assert x.numel() > LIMIT
+    y = kernel(x, np.float32(0.5))
+    for e in (0, batch - 1):
+        xd = indexes.inverse(x[e:e + 1])[0]
+        yd = indexes.inverse(y[e:e + 1])[0]
+        for r0 in (0, H - 512):
+            rows = xd[r0:r0 + 512].float() / 2.0
+            rows = rows.masked_fill(mask[r0:r0 + 512] == 0, float('-inf'))
+            torch.testing.assert_close(yd[r0:r0 + 512].float(), torch.softmax(rows, -1), rtol=1e-2, atol=1e-3)
+        del xd, yd
+
+
+def test_attention_beyond_2g_elements(gpu, batch=8256, N=4096, E=64):
+    """q, k, v, out of 8256 x 4096 x 64 = 2.16 G elements each; the training path also
+    writes 8256 x 72 blocks of probabilities (2.4 G elements)."""
+    grid = np.zeros((64, 64), dtype=np.uint8)
+    i = np.arange(64)
+    grid[i, i] = 1
+    grid[i[8:], i[8:] - 8] |= (i[8:] % 8 == 0).astype(np.uint8)
+    grid[0] = 0
+    grid[0, 0] = 1
+    mask = torch.from_numpy(np.kron(grid, np.ones((64, 64), dtype=np.uint8))).to(gpu)
+    q, k, v = (_randn((batch, N, E), 10 + s, gpu) for s in range(3))
+    assert q.numel() > LIMIT
+    att = SparseAttention(mask=mask)
+    mm = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 64, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 64}
+    sm = {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': 64, 'BLOCK_SIZE_W_VALUE': 64, 'ROW_TILE_VALUE': 4}
+    att.build({f'{part}/{pas}': dict(mm) for part in ('qk', 'out') for pas in ('forward:C', 'backward:A', 'backward:B')}
+              | {'sm/forward:y': dict(sm), 'sm/backward:x': dict(sm)}, sample_inputs=[q, k, v])
+
+    def dense(b, leaves=None):
+        qq, kk, vv = leaves if leaves is not None else (q[b].float(), k[b].float(), v[b].float())
+        s = (qq @ kk.t()) / 8.0
+        s = s.masked_fill(mask == 0, float('-inf'))
+        return torch.softmax(s, -1) @ vv
+
+    with torch.no_grad():
+        out = att(q, k, v)
+    for b in (0, batch - 1):
+        torch.testing.assert_close(out[b].float(), dense(b), rtol=1e-2, atol=1e-2)
+    del out
+    # training path: forward with probabilities, score-gradient kernel, the two thin products
+    leaves = [t.requires_grad_(True) for t in (q, k, v)]
+    grad = _randn((batch, N, E), 14, gpu)
+    out = att(*leaves)
+    out.backward(grad)
+    for b in (0, batch - 1):
+        ref_leaves = [t[b].detach().float().requires_grad_(True) for t in leaves]
+        dense(b, ref_leaves).backward(grad[b].float())
+        for t, r in zip(leaves, ref_leaves):
+            torch.testing.assert_close(t.grad[b].float(), r.grad, rtol=2e-2, atol=2e-2)
+
+
+def test_moe_beyond_2g_elements(gpu, n_tok=589824, K=128, N=4096, n_exp=4):
+    mods = [torch.nn.Linear(K, N, bias=False, dtype=torch.float16, device=gpu) for _ in range(n_exp)]
+    moe = DynamicSparseMoE(mods)
+    x = _randn((n_tok, K), 15, gpu)
+    g = torch.Generator(device=gpu).manual_seed(16)
+    ids = torch.randint(0, n_exp, (n_tok,), generator=g, device=gpu, dtype=torch.int32)
+    out = moe(x, ids)
+    assert out.numel() > LIMIT
+    for r0 in (0, n_tok - 4096):
+        rows = slice(r0, r0 + 4096)
+        want = torch.zeros((4096, N), device=gpu)
+        for e in range(n_exp):
+            sel = ids[rows] == e
+            want[sel] = x[rows][sel].float() @ mods[e].weight.float().t()
+        torch.testing.assert_close(out[rows].float(), want, rtol=1e-2, atol=1e-2)
