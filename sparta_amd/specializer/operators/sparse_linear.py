@@ -16,10 +16,11 @@ class SparseLinear(OperatorBase):
             after `build` the `weight` parameter holds the BCSR-compressed values.
         output_mask: mask of the output [batch, out_features] -> 'dds' kernel, dense storage.
         Exactly one of the three masks must be given.
-        dynamic: the mask changes every few steps.  Compressed weights are then kept
-            at full capacity and `update_mask` enqueues the index rebuild and the
-            re-compression without ever waiting for the host (the reference
-            synchronises once per rebuild).
+        dynamic: the mask changes every few steps.  `update_mask` then enqueues the
+            index rebuild without ever waiting for the host (the reference synchronises
+            once per rebuild); with a weight mask the weight stays dense and the kernels
+            read its live blocks through the index (no re-compression), with an input
+            mask the compressed operand is kept at full capacity.
 
     Shape: input (B, in_features) -> output (B, out_features).
 
@@ -50,7 +51,9 @@ class SparseLinear(OperatorBase):
             self._sparse_ctx = SparseBatchMatMulCtx('sdd', False, True, biased, False)
             M = input_mask.shape[0]
         elif weight_mask is not None:
-            self._sparse_ctx = SparseBatchMatMulCtx('dsd', False, True, biased, True)
+            # dynamic: the kernels read the live blocks out of the dense weight through the
+            # index, so a new mask costs an index rebuild and nothing else
+            self._sparse_ctx = SparseBatchMatMulCtx('dsd', False, True, biased, not dynamic)
         elif output_mask is not None:
             self._sparse_ctx = SparseBatchMatMulCtx('dds', False, True, biased, False)
             M = output_mask.shape[0]
@@ -93,8 +96,12 @@ class SparseLinear(OperatorBase):
         it is: values inside live blocks are not multiplied by the element mask."""
         weight = self._raw_weight
         indexes = self.get_sparse_indexes('B')
+        if indexes is not None and self._dynamic:
+            if self.weight is None:
+                self.weight = torch.nn.Parameter(weight, requires_grad=True)
+            return
         if indexes is not None:
-            weight = indexes.convert(weight.detach(), at_capacity=self._dynamic)
+            weight = indexes.convert(weight.detach())
         self.weight = torch.nn.Parameter(weight, requires_grad=True)
 
     def _compile(self, config: Optional[Dict[str, Dict[str, Any]]] = None):
