@@ -216,18 +216,34 @@ int spx_attention_forward_train(int dtype, const void* q, const void* k, const v
 /* Row side of the backward pass, from the probabilities spx_attention_forward_train saved:
  *   grad_scores = probs o (grad_out v^T - D) * inv_temperature,  D[i] = sum_e grad_out[i,e] out[i,e]
  *   grad_q      = grad_scores k
- * grad_scores has the compressed layout and batch stride of probs; it is the operand of the
- * remaining product grad_k = grad_scores^T q (spx_matmul with the sparse operand transposed),
- * as probs is of grad_v = probs^T grad_out.  Masked entries carry probs = 0 and get
- * grad_scores = 0.  Replaces three launches of the reference's backward chain: the
- * dense x dense -> sparse product of SparseBatchMatMul's backward, SparseSoftmax's backward
- * and the sparse x dense product for the query gradient (sparse_attention.py:76-80 run in
- * reverse by autograd).  Same block shapes as spx_attention_forward_train. */
+ * grad_scores (may be NULL: not stored) has the compressed layout and batch stride of probs; it
+ * is the operand of grad_k = grad_scores^T q through spx_matmul with the sparse operand
+ * transposed, as probs is of grad_v = probs^T grad_out.  row_dot (may be NULL) receives
+ * D[b, i] * inv_temperature as float [batch, Nt], which spx_attention_backward_kv reads.
+ * Masked entries carry probs = 0 and get grad_scores = 0.  Replaces three launches of the
+ * reference's backward chain: the dense x dense -> sparse product of SparseBatchMatMul's
+ * backward, SparseSoftmax's backward and the sparse x dense product for the query gradient
+ * (sparse_attention.py:76-80 run in reverse by autograd).  Same block shapes as
+ * spx_attention_forward_train. */
 int spx_attention_backward_scores(int dtype, const void* grad_out, const void* out, const void* probs,
                                   const void* k, const void* v, void* grad_scores, void* grad_q,
-                                  int64_t probs_batch_stride,
+                                  float* row_dot, int64_t probs_batch_stride,
                                   const int32_t* row_ptr, const int32_t* bcsr_idx, float inv_temperature,
                                   int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
+
+/* Column side of the backward pass: grad_v = probs^T grad_out and grad_k = grad_scores^T q
+ * with grad_scores recomputed from probs, grad_out, v and row_dot (written by
+ * spx_attention_backward_scores), walking the BCSC index (idx_kind SPX_IDX_BCSC_I64 when the
+ * values are in BCSR order, as spx_attention_forward_train writes them; SPX_IDX_BCSC_I32 for
+ * values in BCSC order).  Replaces the two transposed sparse x dense products of the
+ * reference's backward chain (batch_matmul.py:47-71, backward:B of both matmuls) and the
+ * write and two reads of the score gradient between them.  Query blocks 32 / 64 / 128, key
+ * blocks 32 / 64 / 128, head dims 64 / 128, BH * E >= 32 * BW. */
+int spx_attention_backward_kv(int dtype, const void* grad_out, const void* q, const void* v,
+                              const void* probs, const float* row_dot, void* grad_k, void* grad_v,
+                              int64_t probs_batch_stride,
+                              const int32_t* col_ptr, const void* bcsc_idx, int idx_kind, float inv_temperature,
+                              int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
 
 /* ------------------------------------------------------------------------ *
  * Sequence-length attention: q, k, v, out are [batch, heads, N, E]; batch b

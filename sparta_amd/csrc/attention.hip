@@ -36,6 +36,12 @@ struct AttnParams {
     const void* grad_out; // backward kernel: gradient of the output
     void* grad_scores;    // backward kernel: compressed gradient of the scores (layout of probs)
     void* grad_q;         // backward kernel: gradient of the queries
+    float* row_dot;       // backward kernels: D[b, i] / T = sum_e grad_out o out / T per query
+    const int32_t* col_ptr;   // column-side backward kernel: BCSC index
+    const void* bcsc_idx;
+    int bcsc_wide;        // 1: int64 entries (bcsr_pos << 32 | col << 16 | row), 0: int32 (col << 16 | row)
+    void* grad_k;
+    void* grad_v;
 };
 
 template <typename T> struct AttnMma;
@@ -831,6 +837,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
         gf[c] = AttnPack<T>::pack(scaled);
     }
     const float d_row = xor32_sum(xor16_sum(d_part));
+    if (p.row_dot && g4 == 0) p.row_dot[b * p.Nt + qrow] = d_row;
+    const bool store_ds = p.grad_scores != nullptr;   // the column-side kernel recomputes dS from P
     const f32x4 negd = f32x4{-d_row, -d_row, -d_row, -d_row};
 
     f32x4 qacc[ET];
@@ -926,10 +934,12 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
             *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp) * 32) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
             *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp + 1) * 32) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
         }
+        if (store_ds) {
 #pragma unroll
-        for (int i = 0; i < PN; ++i)
-            *reinterpret_cast<u32x4*>(dS + (int64_t)e * (16 * WAVES * BW) + wave_off + i * 512) =
-                *reinterpret_cast<const u32x4*>(ptile + pt_vec[i]);
+            for (int i = 0; i < PN; ++i)
+                *reinterpret_cast<u32x4*>(dS + (int64_t)e * (16 * WAVES * BW) + wave_off + i * 512) =
+                    *reinterpret_cast<const u32x4*>(ptile + pt_vec[i]);
+        }
         // ---- dQ^T[e][query] += K^T dS^T ------------------------------------------------------
 #pragma unroll
         for (int t = 0; t < ET; ++t) {
@@ -990,6 +1000,234 @@ static int launch_attention_bwd_row(const AttnParams& p, int batch, int BW, int 
     SPX_ATTNB_CASE(128, 32, 128) SPX_ATTNB_CASE(128, 64, 128) SPX_ATTNB_CASE(128, 128, 128)
 #undef SPX_ATTNB_CASE
     return fail(SPX_E_CONFIG, "the attention backward kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
+// ---- backward pass, column side: gradients of the keys and of the values -------------------
+//   dV = P^T dO,   dK = dS^T Q,   dS = P o (dO V^T - D) / T  (recomputed here from P)
+// One workgroup per block column (BW keys) and batch entry, one wavefront per 16 keys, walking
+// the live blocks of the column through the BCSC index.  Per block the dO and Q tiles of the
+// query block and the P block (at its BCSR position) are staged in LDS, rows padded for
+// transpose reads:
+//   (dP - D)^T/T tiles: 16 queries x 16 keys = dO rows x V rows (V of the column, scaled by
+//     1/T, lives in registers; accumulators start at -D/T read from row_dot), a lane gets
+//     4 consecutive queries of one key;
+//   P in that same layout by one transpose read per tile; dS = P o (dP - D)/T;
+//   two tiles side by side are the B operand (32 queries deep) of
+//     dK^T[e][key] += Q^T dS   and, for P itself,   dV^T[e][key] += dO^T P,
+//   whose A operands are transpose reads of the Q and dO tiles.
+// The score gradient never goes to memory: P is read once here and once by the row-side
+// kernel, instead of P and dS being read by two separate products after dS was written.
+template <typename T, int BH, int E, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attention_bwd_col_kernel(AttnParams p, int nbc, int batch) {
+    constexpr int BW = 16 * WAVES;
+    constexpr int NT = 64 * WAVES;
+    constexpr int QT = BH / 16, ET = E / 16, EC = E / 32;
+    constexpr int DP = E * 2 + 32;            // row pitch of the dO and Q tiles
+    constexpr int PP = BW * 2 + 32;           // row pitch of the P block
+    constexpr int Q_OFF = BH * DP, P_OFF = 2 * BH * DP;
+    constexpr int TILE = 2 * BH * DP + BH * PP;
+    constexpr int VPR = E / 8, PPR = BW / 8;  // 16-byte vectors per row
+    constexpr int NVD = BH * VPR / NT;        // vectors per thread: dO / Q tile
+    constexpr int NVP = BH * PPR / NT;        // vectors per thread: P block
+    static_assert(BH * VPR % NT == 0 && BH * PPR % NT == 0 && QT % 2 == 0, "tiles do not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    const int L = blockIdx.x;
+    const int slot_l = L >> 3;
+    const int64_t b = (slot_l / nbc) * 8 + (L & 7);
+    const int j = slot_l % nbc;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* dO = reinterpret_cast<const T*>(p.grad_out) + b * (int64_t)p.Nt * E + threadIdx.x * 8;
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.Nt * E + threadIdx.x * 8;
+    const T* P = reinterpret_cast<const T*>(p.probs) + b * p.probs_batch + threadIdx.x * 8;
+    const float* Dv = p.row_dot + b * (int64_t)p.Nt + g4 * 4;
+    T* dK = reinterpret_cast<T*>(p.grad_k) + b * (int64_t)p.Ns * E;
+    T* dV = reinterpret_cast<T*>(p.grad_v) + b * (int64_t)p.Ns * E;
+
+    const int krow = j * BW + wave * 16 + r16;
+    Frag vf[EC];     // V of this lane's key, scaled by 1 / T
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        const Frag raw = Mma32<T>::load(reinterpret_cast<const T*>(p.v) + (b * (int64_t)p.Ns + krow) * E + c * 32 + g4 * 8);
+        f32x8 scaled;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) scaled[x] = (float)raw[x] * p.inv_t;
+        vf[c] = AttnPack<T>::pack(scaled);
+    }
+
+    f32x4 kacc[ET], vacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) kacc[t] = vacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // staging maps (a tile is contiguous in memory: vector v = tid + i * NT is row v / VPR)
+    const int d_dst = (threadIdx.x / VPR) * DP + (threadIdx.x % VPR) * 16;
+    const int p_dst = P_OFF + (threadIdx.x / PPR) * PP + (threadIdx.x % PPR) * 16;
+    constexpr int D_RSTEP = NT / VPR, P_RSTEP = NT / PPR;
+    static_assert(NT % VPR == 0 && NT % PPR == 0, "rows per pass");
+    const int a_src = r16 * DP + g4 * 16;                                    // dO rows as A operand of dP
+    const int t_src = (g4 * 4 + (r16 >> 2)) * DP + (r16 & 3) * 8;            // transpose reads of dO / Q
+    const int pt_src = P_OFF + (g4 * 4 + (r16 >> 2)) * PP + (wave * 16 + (r16 & 3) * 4) * 2;
+
+    const int e_begin = p.col_ptr[j];
+    const int e_end = p.col_ptr[j + 1];
+    auto entry = [&](int e, int& qb, int64_t& pos) {
+        if (p.bcsc_wide) {
+            const long long v = reinterpret_cast<const long long*>(p.bcsc_idx)[e];
+            qb = (int)(v & 0xffff);
+            pos = v >> 32;
+        } else {
+            qb = reinterpret_cast<const int32_t*>(p.bcsc_idx)[e] & 0xffff;
+            pos = e;
+        }
+    };
+    u32x4 do_r[NVD], q_r[NVD], p_r[NVP];
+    f32x4 d_r[QT];
+    auto issue = [&](int qb, int64_t pos) {
+        const int64_t off = (int64_t)qb * BH * E;
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) do_r[i] = *reinterpret_cast<const u32x4*>(dO + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) q_r[i] = *reinterpret_cast<const u32x4*>(Q + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NVP; ++i) p_r[i] = *reinterpret_cast<const u32x4*>(P + pos * (int64_t)(BH * BW) + i * NT * 8);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) d_r[t] = *reinterpret_cast<const f32x4*>(Dv + qb * BH + t * 16);
+    };
+    int qb = 0, qb_next = 0;
+    int64_t pos = 0, pos_next = 0;
+    if (e_begin < e_end) {
+        entry(e_begin, qb, pos);
+        entry(e_begin + 1 < e_end ? e_begin + 1 : e_begin, qb_next, pos_next);
+        issue(qb, pos);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        __syncthreads();   // everyone is done with the previous tiles
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) *reinterpret_cast<u32x4*>(smem + d_dst + i * D_RSTEP * DP) = do_r[i];
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) *reinterpret_cast<u32x4*>(smem + Q_OFF + d_dst + i * D_RSTEP * DP) = q_r[i];
+#pragma unroll
+        for (int i = 0; i < NVP; ++i) *reinterpret_cast<u32x4*>(smem + p_dst + i * P_RSTEP * PP) = p_r[i];
+        f32x4 s[QT];
+#pragma unroll
+        for (int t = 0; t < QT; ++t) s[t] = -d_r[t];
+        // next live block of the column (the last step re-reads its own block; the copy is not used)
+        qb = qb_next; pos = pos_next;
+        entry(e + 2 < e_end ? e + 2 : e_end - 1, qb_next, pos_next);
+        issue(qb, pos);
+        __syncthreads();
+
+        // ---- (dP - D) / T: 16 queries x this wave's 16 keys per tile -------------------------
+#pragma unroll
+        for (int t = 0; t < QT; ++t) {
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag af = *reinterpret_cast<const Frag*>(smem + a_src + t * 16 * DP + c * 64);
+                s[t] = Mma32<T>::mma(af, vf[c], s[t]);
+            }
+        }
+        // ---- P in the same layout; dS = P o (dP - D) / T; both as B operands ------------------
+        Frag pf[QT / 2], sf[QT / 2];
+#pragma unroll
+        for (int kp = 0; kp < QT / 2; ++kp) {
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + pt_src + (kp * 32) * PP));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + pt_src + (kp * 32 + 16) * PP));
+            pf[kp] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            f32x8 ds;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) ds[x] = (float)pf[kp][x] * s[2 * kp + (x >> 2)][x & 3];
+            sf[kp] = AttnPack<T>::pack(ds);
+        }
+        // ---- dK^T[e][key] += Q^T dS,  dV^T[e][key] += dO^T P ----------------------------------
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int kp = 0; kp < QT / 2; ++kp) {
+                const s16x4 qlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + Q_OFF + t_src + (kp * 32) * DP + t * 32));
+                const s16x4 qhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + Q_OFF + t_src + (kp * 32 + 16) * DP + t * 32));
+                const s16x8 qa = __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7);
+                kacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, qa), sf[kp], kacc[t]);
+                const s16x4 glo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + t_src + (kp * 32) * DP + t * 32));
+                const s16x4 ghi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + t_src + (kp * 32 + 16) * DP + t * 32));
+                const s16x8 ga = __builtin_shufflevector(glo, ghi, 0, 1, 2, 3, 4, 5, 6, 7);
+                vacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, ga), pf[kp], vacc[t]);
+            }
+        }
+    }
+
+    // lane holds dK^T[e = 16 t + 4 g4 + q][key r16] (and dV^T): rows of 16 keys per wave
+    uint64_t kp_[ET], vp_[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T kv[4], vv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            kv[q] = Elem<T>::from_float(kacc[t][q]);
+            vv[q] = Elem<T>::from_float(vacc[t][q]);
+        }
+        kp_[t] = *reinterpret_cast<const uint64_t*>(kv);
+        vp_[t] = *reinterpret_cast<const uint64_t*>(vv);
+    }
+    const int64_t row0 = (int64_t)(krow - r16) * E;
+    if constexpr (WAVES * 16 * (E * 2 + 16) <= TILE) {
+        __syncthreads();   // the tiles are dead: their space carries the output tiles
+        char* tile = smem + wave * (16 * (E * 2 + 16));
+        wave_rows_store<E>(tile, dK + row0, kp_);
+        wave_rows_store<E>(tile, dV + row0, vp_);
+    } else {
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+            *reinterpret_cast<uint64_t*>(dK + row0 + (int64_t)r16 * E + t * 16 + g4 * 4) = kp_[t];
+            *reinterpret_cast<uint64_t*>(dV + row0 + (int64_t)r16 * E + t * 16 + g4 * 4) = vp_[t];
+        }
+    }
+}
+
+// Query blocks of 32 / 64 / 128, key blocks of 32 / 64 / 128, head dims 64 / 128, with at
+// least one vector of the dO tile per thread.
+static bool attention_bwd_col_supported(int BH, int BW, int E) {
+    return (BH == 32 || BH == 64 || BH == 128) && (BW == 32 || BW == 64 || BW == 128) && (E == 64 || E == 128) &&
+           BH * E >= 32 * BW;
+}
+
+template <typename T, int BH, int E, int WAVES>
+static int launch_attention_bwd_col_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr size_t smem = 2 * BH * (E * 2 + 32) + BH * (WAVES * 32 + 32);
+    const int nbc = p.Ns / (16 * WAVES);
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbc;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_col_kernel<T, BH, E, WAVES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_bwd_col_kernel)");
+    }
+    hipLaunchKernelGGL((attention_bwd_col_kernel<T, BH, E, WAVES>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbc, batch);
+    SPX_LAUNCH_CHECK("attention_bwd_col_kernel");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_bwd_col(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTNC_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_bwd_col_inst<T, bh, e, bw / 16>(p, batch, st);
+    SPX_ATTNC_CASE(32, 32, 64) SPX_ATTNC_CASE(32, 64, 64)
+    SPX_ATTNC_CASE(32, 32, 128) SPX_ATTNC_CASE(32, 64, 128) SPX_ATTNC_CASE(32, 128, 128)
+    SPX_ATTNC_CASE(64, 32, 64) SPX_ATTNC_CASE(64, 64, 64) SPX_ATTNC_CASE(64, 128, 64)
+    SPX_ATTNC_CASE(64, 32, 128) SPX_ATTNC_CASE(64, 64, 128) SPX_ATTNC_CASE(64, 128, 128)
+    SPX_ATTNC_CASE(128, 32, 64) SPX_ATTNC_CASE(128, 64, 64) SPX_ATTNC_CASE(128, 128, 64)
+    SPX_ATTNC_CASE(128, 32, 128) SPX_ATTNC_CASE(128, 64, 128) SPX_ATTNC_CASE(128, 128, 128)
+#undef SPX_ATTNC_CASE
+    return fail(SPX_E_CONFIG, "the key / value gradient kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
 }
 
 // ---- pipelined variant on 32 x 32 x 16 MFMAs ---------------------------------------------
@@ -1449,7 +1687,8 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     p.probs = nullptr; p.probs_batch = 0;
-    p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr;
+    p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr; p.row_dot = nullptr;
+    p.col_ptr = nullptr; p.bcsc_idx = nullptr; p.bcsc_wide = 0; p.grad_k = nullptr; p.grad_v = nullptr;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel;
     // 3: pipelined kernel on 32x32x16 MFMAs (one wavefront per 32 queries; measured within a few
@@ -1493,7 +1732,8 @@ extern "C" int spx_attention_forward_train(int dtype, const void* q, const void*
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     p.probs = probs; p.probs_batch = probs_batch_stride;
-    p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr;
+    p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr; p.row_dot = nullptr;
+    p.col_ptr = nullptr; p.bcsc_idx = nullptr; p.bcsc_wide = 0; p.grad_k = nullptr; p.grad_v = nullptr;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (dtype == SPX_F16) return launch_attention_train<_Float16>(p, batch, BW, E, st);
     return launch_attention_train<bf16_t>(p, batch, BW, E, st);
@@ -1501,13 +1741,13 @@ extern "C" int spx_attention_forward_train(int dtype, const void* q, const void*
 
 extern "C" int spx_attention_backward_scores(int dtype, const void* grad_out, const void* out, const void* probs,
                                              const void* k, const void* v, void* grad_scores, void* grad_q,
-                                             int64_t probs_batch_stride,
+                                             float* row_dot, int64_t probs_batch_stride,
                                              const int32_t* row_ptr, const int32_t* bcsr_idx, float inv_temperature,
                                              int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream) {
     using namespace spx;
     SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
                 "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
-    SPX_REQUIRE(grad_out && out && probs && k && v && grad_scores && grad_q && row_ptr && bcsr_idx, SPX_E_NULL,
+    SPX_REQUIRE(grad_out && out && probs && k && v && grad_q && row_ptr && bcsr_idx, SPX_E_NULL,
                 "a required buffer is NULL");
     SPX_REQUIRE(Nt > 0 && Ns > 0 && BH > 0 && BW > 0 && Nt % BH == 0 && Ns % BW == 0, SPX_E_SHAPE,
                 "mask shape (%d,%d) is not a multiple of the block (%d,%d)", Nt, Ns, BH, BW);
@@ -1515,19 +1755,54 @@ extern "C" int spx_attention_backward_scores(int dtype, const void* grad_out, co
                 "the attention backward kernel covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 (got %d, %d, %d)", BH, BW, E);
     SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
     SPX_REQUIRE(aligned(grad_out, 16) && aligned(out, 16) && aligned(probs, 16) && aligned(k, 16) && aligned(v, 16) &&
-                aligned(grad_scores, 16) && aligned(grad_q, 16), SPX_E_ALIGN, "buffers must be 16-byte aligned");
+                aligned(grad_scores, 16) && aligned(grad_q, 16) && aligned(row_dot, 16), SPX_E_ALIGN,
+                "buffers must be 16-byte aligned");
     SPX_REQUIRE(probs_batch_stride % 8 == 0, SPX_E_ALIGN, "probs_batch_stride must be a multiple of 8 elements");
     if (batch == 0) return 0;
-    AttnParams p;
-    p.q = nullptr; p.k = k; p.v = v; p.out = const_cast<void*>(out);
-    p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx; p.mask = nullptr;
+    AttnParams p = {};
+    p.k = k; p.v = v; p.out = const_cast<void*>(out);
+    p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx;
     p.inv_t = inv_temperature;
     p.Nt = Nt; p.Ns = Ns; p.BH = BH;
     p.probs = const_cast<void*>(probs); p.probs_batch = probs_batch_stride;
-    p.grad_out = grad_out; p.grad_scores = grad_scores; p.grad_q = grad_q;
+    p.grad_out = grad_out; p.grad_scores = grad_scores; p.grad_q = grad_q; p.row_dot = row_dot;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (dtype == SPX_F16) return launch_attention_bwd_row<_Float16>(p, batch, BW, E, st);
     return launch_attention_bwd_row<bf16_t>(p, batch, BW, E, st);
+}
+
+extern "C" int spx_attention_backward_kv(int dtype, const void* grad_out, const void* q, const void* v,
+                                         const void* probs, const float* row_dot, void* grad_k, void* grad_v,
+                                         int64_t probs_batch_stride,
+                                         const int32_t* col_ptr, const void* bcsc_idx, int idx_kind, float inv_temperature,
+                                         int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
+                "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
+    SPX_REQUIRE(grad_out && q && v && probs && row_dot && grad_k && grad_v && col_ptr && bcsc_idx, SPX_E_NULL,
+                "a required buffer is NULL");
+    SPX_REQUIRE(idx_kind == SPX_IDX_BCSC_I32 || idx_kind == SPX_IDX_BCSC_I64, SPX_E_CONFIG,
+                "the key / value gradient kernel walks a BCSC index (got index kind %d)", idx_kind);
+    SPX_REQUIRE(Nt > 0 && Ns > 0 && BH > 0 && BW > 0 && Nt % BH == 0 && Ns % BW == 0, SPX_E_SHAPE,
+                "mask shape (%d,%d) is not a multiple of the block (%d,%d)", Nt, Ns, BH, BW);
+    SPX_REQUIRE(attention_bwd_col_supported(BH, BW, E), SPX_E_CONFIG,
+                "the key / value gradient kernel covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 with BH * E >= 32 * BW (got %d, %d, %d)", BH, BW, E);
+    SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
+    SPX_REQUIRE(aligned(grad_out, 16) && aligned(q, 16) && aligned(v, 16) && aligned(probs, 16) && aligned(row_dot, 16) &&
+                aligned(grad_k, 16) && aligned(grad_v, 16), SPX_E_ALIGN, "buffers must be 16-byte aligned");
+    SPX_REQUIRE(probs_batch_stride % 8 == 0, SPX_E_ALIGN, "probs_batch_stride must be a multiple of 8 elements");
+    if (batch == 0) return 0;
+    AttnParams p = {};
+    p.q = q; p.v = v;
+    p.inv_t = inv_temperature;
+    p.Nt = Nt; p.Ns = Ns; p.BH = BH;
+    p.probs = const_cast<void*>(probs); p.probs_batch = probs_batch_stride;
+    p.grad_out = grad_out; p.row_dot = const_cast<float*>(row_dot);
+    p.col_ptr = col_ptr; p.bcsc_idx = bcsc_idx; p.bcsc_wide = idx_kind == SPX_IDX_BCSC_I64;
+    p.grad_k = grad_k; p.grad_v = grad_v;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (dtype == SPX_F16) return launch_attention_bwd_col<_Float16>(p, batch, BW, E, st);
+    return launch_attention_bwd_col<bf16_t>(p, batch, BW, E, st);
 }
 
 extern "C" int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const void* v, void* out,

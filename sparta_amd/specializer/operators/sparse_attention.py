@@ -24,9 +24,10 @@ _PARTS = (('qk', '_matmul_qk', 'C'), ('sm', '_softmax', 'y'), ('out', '_matmul_o
 
 
 class _FusedAttentionFunc(torch.autograd.Function):
-    """Forward: one launch gives the output and the probabilities.  Backward: one launch
-    gives the gradients of the scores and of the queries; the key and value gradients are
-    the two transposed sparse x dense products of the matmul operators."""
+    """Forward: one launch gives the output and the probabilities.  Backward: a row-side
+    launch for the query gradient and a column-side launch for the key and value gradients,
+    both reading the saved probabilities (block shapes the column-side kernel does not
+    cover take the two transposed sparse x dense products of the matmul operators)."""
 
     @staticmethod
     def forward(ctx, op: 'SparseAttention', query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
@@ -42,16 +43,21 @@ class _FusedAttentionFunc(torch.autograd.Function):
         op = ctx.op
         out_ctx, qk_ctx = op._matmul_out._sparse_ctx, op._matmul_qk._sparse_ctx
         grad_out = grad_out.detach().contiguous()
+        need_q, need_k, need_v = ctx.needs_input_grad[1:4]
         grad_q = grad_k = grad_v = None
-        if ctx.needs_input_grad[3]:
-            grad_v = out_ctx.backward_B(grad_out, probs)
-        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            grad_scores, grad_q = op._fused_backward_scores(grad_out, out, probs, k, v)
-            if ctx.needs_input_grad[2]:
-                grad_k = qk_ctx.backward_B(grad_scores, q)
-            if not ctx.needs_input_grad[1]:
-                grad_q = None
-        return None, grad_q, grad_k, grad_v
+        if (need_k or need_v) and op._fused_backward_kv_supported(grad_out):
+            # two launches: the row side gives grad_q and the row constants, the column side
+            # recomputes the score gradient from the probabilities for grad_k and grad_v
+            _, grad_q, row_dot = op._fused_backward_scores(grad_out, out, probs, k, v, store_scores=False)
+            grad_k, grad_v = op._fused_backward_kv(grad_out, q, v, probs, row_dot)
+        else:
+            if need_v:
+                grad_v = out_ctx.backward_B(grad_out, probs)
+            if need_q or need_k:
+                grad_scores, grad_q, _ = op._fused_backward_scores(grad_out, out, probs, k, v, store_scores=need_k)
+                if need_k:
+                    grad_k = qk_ctx.backward_B(grad_scores, q)
+        return None, grad_q if need_q else None, grad_k if need_k else None, grad_v if need_v else None
 
 
 class SparseAttention(OperatorBase):
@@ -132,20 +138,48 @@ class SparseAttention(OperatorBase):
         _lib.check(rc, 'spx_attention_forward_train')
         return out, probs
 
-    def _fused_backward_scores(self, grad_out, out, probs, key, value):
-        """(compressed score gradient, query gradient) from spx_attention_backward_scores."""
+    def _fused_backward_scores(self, grad_out, out, probs, key, value, store_scores=True):
+        """(compressed score gradient or None, query gradient, row constants) from
+        spx_attention_backward_scores."""
         indexes = self._sparse_port.indexes
         batch, _, E = grad_out.shape
         k, v = key.contiguous(), value.contiguous()
-        grad_scores = torch.empty_like(probs)
+        grad_scores = torch.empty_like(probs) if store_scores else None
         grad_q = torch.empty_like(grad_out)
+        row_dot = torch.empty((batch, self._Nt), dtype=torch.float32, device=grad_out.device)
         rc = _lib.load().spx_attention_backward_scores(
             _lib.dtype_code(grad_out.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(out), _lib.dev_ptr(probs),
-            _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(grad_scores), _lib.dev_ptr(grad_q), probs.shape[1],
-            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), float(self._inv_temperature),
-            batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W, _lib.current_stream(grad_out.device))
+            _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(grad_scores), _lib.dev_ptr(grad_q), _lib.dev_ptr(row_dot),
+            probs.shape[1], _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf),
+            float(self._inv_temperature), batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W,
+            _lib.current_stream(grad_out.device))
         _lib.check(rc, 'spx_attention_backward_scores')
-        return grad_scores, grad_q
+        return grad_scores, grad_q, row_dot
+
+    def _fused_backward_kv_supported(self, grad_out: torch.Tensor) -> bool:
+        """The column-side kernel needs the BCSC index next to the BCSR one (the probabilities
+        are stored in BCSR order) and the block shapes it covers."""
+        indexes = self._sparse_port.indexes
+        BH, BW, E = indexes.block_H, indexes.block_W, grad_out.shape[-1]
+        return (getattr(indexes, 'col_ptr', None) is not None and getattr(indexes, 'row_ptr', None) is not None
+                and BH in (32, 64, 128) and BW in (32, 64, 128) and E in (64, 128) and BH * E >= 32 * BW)
+
+    def _fused_backward_kv(self, grad_out, query, value, probs, row_dot):
+        """(key gradient, value gradient) from spx_attention_backward_kv."""
+        indexes = self._sparse_port.indexes
+        batch, _, E = grad_out.shape
+        q, v = query.contiguous(), value.contiguous()
+        grad_k = torch.empty_like(v)
+        grad_v = torch.empty_like(v)
+        idx = indexes._bcsc_buf
+        kind = _lib.IDX_BCSC_I64 if idx.dtype == torch.int64 else _lib.IDX_BCSC_I32
+        rc = _lib.load().spx_attention_backward_kv(
+            _lib.dtype_code(grad_out.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(q), _lib.dev_ptr(v),
+            _lib.dev_ptr(probs), _lib.dev_ptr(row_dot), _lib.dev_ptr(grad_k), _lib.dev_ptr(grad_v), probs.shape[1],
+            _lib.dev_ptr(indexes.col_ptr), _lib.dev_ptr(idx), kind, float(self._inv_temperature),
+            batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W, _lib.current_stream(grad_out.device))
+        _lib.check(rc, 'spx_attention_backward_kv')
+        return grad_k, grad_v
 
     def _fused_supported(self, query: torch.Tensor) -> bool:
         """The fused kernel covers 16-bit inputs, head dims 32 / 64 / 128 and score

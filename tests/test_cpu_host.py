@@ -72,12 +72,19 @@ def test_host_validation_without_gpu():
     assert rc == _lib.E_CONFIG and 'head dim' in _lib.last_error()
     rc = lib.spx_attention_forward_train(f16, one, one, one, one, None, 4096, one, one, None, 0.125, 1, 256, 256, 64, 64, 64, None)
     assert rc == _lib.E_NULL
-    rc = lib.spx_attention_backward_scores(f16, one, one, one, one, one, one, one, 4096, one, one, 0.125, 1, 256, 256, 64, 16, 64, None)
+    rc = lib.spx_attention_backward_scores(f16, one, one, one, one, one, None, one, None, 4096, one, one, 0.125, 1, 256, 256, 64, 16, 64, None)
     assert rc == _lib.E_CONFIG
-    rc = lib.spx_attention_backward_scores(f16, one, one, one, one, one, one, one, 4100, one, one, 0.125, 1, 256, 256, 64, 64, 64, None)
+    rc = lib.spx_attention_backward_scores(f16, one, one, one, one, one, one, one, one, 4100, one, one, 0.125, 1, 256, 256, 64, 64, 64, None)
     assert rc == _lib.E_ALIGN
-    rc = lib.spx_attention_backward_scores(0, one, one, one, one, one, one, one, 4096, one, one, 0.125, 1, 256, 256, 64, 64, 64, None)
+    rc = lib.spx_attention_backward_scores(0, one, one, one, one, one, one, one, one, 4096, one, one, 0.125, 1, 256, 256, 64, 64, 64, None)
     assert rc == _lib.E_DTYPE
+    kv = lambda **kw: lib.spx_attention_backward_kv(
+        kw.get('dtype', f16), one, one, one, one, kw.get('row_dot', one), one, one, 4096, one, one, kw.get('kind', _lib.IDX_BCSC_I64),
+        0.125, 1, 256, 256, kw.get('E', 64), kw.get('BH', 64), kw.get('BW', 64), None)
+    assert kv(dtype=0) == _lib.E_DTYPE
+    assert kv(row_dot=None) == _lib.E_NULL
+    assert kv(kind=_lib.IDX_BCSR_I32) == _lib.E_CONFIG and 'BCSC' in _lib.last_error()
+    assert kv(BH=32, BW=128) == _lib.E_CONFIG
     with pytest.raises(AssertionError):
         _lib.check(_lib.E_SHAPE, 'x')
     with pytest.raises(ValueError):

@@ -197,7 +197,9 @@ def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, gpu, H=3, Nt=
     att._fused_forward_train = lambda *a: (calls.append(1), inner(*a))[1]
     bwd_calls = []
     inner_bwd = att._fused_backward_scores
-    att._fused_backward_scores = lambda *a: (bwd_calls.append(1), inner_bwd(*a))[1]
+    att._fused_backward_scores = lambda *a, **kw: (bwd_calls.append(1), inner_bwd(*a, **kw))[1]
+    inner_kv = att._fused_backward_kv
+    att._fused_backward_kv = lambda *a: (bwd_calls.append(2), inner_kv(*a))[1]
 
     def run(fused):
         att._fused = fused
@@ -210,7 +212,7 @@ def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, gpu, H=3, Nt=
     got = run(True)
     assert calls, 'the training forward kernel was not used'
     piped = run(False)
-    assert len(calls) == 1 and len(bwd_calls) == 1
+    assert len(calls) == 1 and bwd_calls == [1, 2]
     # dense fp32 autograd on the same (rounded) inputs
     ref_leaves = [t.detach().float().requires_grad_(True) for t in leaves]
     scores = ref_leaves[0] @ ref_leaves[1].transpose(1, 2) / float(np.sqrt(E))
@@ -227,7 +229,8 @@ def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, gpu, H=3, Nt=
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('BH,BW,E', [(32, 32, 64), (32, 128, 64), (64, 64, 64), (64, 128, 128), (128, 64, 64),
-                                     (128, 128, 128), (128, 32, 128), (32, 64, 128)])
+                                     (128, 128, 128), (128, 32, 128), (32, 64, 128), (64, 128, 64), (32, 128, 128),
+                                     (64, 32, 64), (128, 128, 64)])
 @pytest.mark.parametrize('element_mask', [False, True])
 def test_attention_backward_scores_kernel(dtype, BH, BW, E, element_mask, gpu, batch=3, Nt=256, Ns=384):
     """spx_attention_forward_train followed by spx_attention_backward_scores through the
@@ -243,7 +246,7 @@ def test_attention_backward_scores_kernel(dtype, BH, BW, E, element_mask, gpu, b
     mask_np = ops.block_mask((Nt, Ns), (1, 1) if element_mask else (BH, BW), 0.8 if element_mask else 0.6, seed=45)
     mask_np[:BH] = 0
     mask = torch.from_numpy(mask_np).to(gpu)
-    indexes = get_bcs_function(BH, BW, True, False).build_indexes(mask)
+    indexes = get_bcs_function(BH, BW, True, True).build_indexes(mask)
     q, k, v, g = q.to(gpu), k.to(gpu), v.to(gpu), g.to(gpu)
     inv_t = 1.0 / float(np.sqrt(E))
     lib = _lib.load()
@@ -258,19 +261,39 @@ def test_attention_backward_scores_kernel(dtype, BH, BW, E, element_mask, gpu, b
     _lib.check(rc, 'spx_attention_forward_train')
     grad_scores = torch.full_like(probs, float('nan'))
     grad_q = torch.full_like(q, float('nan'))
+    row_dot = torch.full((batch, Nt), float('nan'), dtype=torch.float32, device=gpu)
     rc = lib.spx_attention_backward_scores(
         _lib.dtype_code(dtype), _lib.dev_ptr(g), _lib.dev_ptr(out), _lib.dev_ptr(probs), _lib.dev_ptr(k), _lib.dev_ptr(v),
-        _lib.dev_ptr(grad_scores), _lib.dev_ptr(grad_q), n_val, _lib.dev_ptr(indexes.row_ptr),
+        _lib.dev_ptr(grad_scores), _lib.dev_ptr(grad_q), _lib.dev_ptr(row_dot), n_val, _lib.dev_ptr(indexes.row_ptr),
         _lib.dev_ptr(indexes._bcsr_buf), inv_t, batch, Nt, Ns, E, BH, BW, _lib.current_stream(gpu))
     _lib.check(rc, 'spx_attention_backward_scores')
+    # without the score gradient: same grad_q
+    grad_q2 = torch.full_like(q, float('nan'))
+    rc = lib.spx_attention_backward_scores(
+        _lib.dtype_code(dtype), _lib.dev_ptr(g), _lib.dev_ptr(out), _lib.dev_ptr(probs), _lib.dev_ptr(k), _lib.dev_ptr(v),
+        None, _lib.dev_ptr(grad_q2), None, n_val, _lib.dev_ptr(indexes.row_ptr),
+        _lib.dev_ptr(indexes._bcsr_buf), inv_t, batch, Nt, Ns, E, BH, BW, _lib.current_stream(gpu))
+    _lib.check(rc, 'spx_attention_backward_scores')
+    assert torch.equal(grad_q, grad_q2)
 
-    qf = q.float().requires_grad_(True)
-    scores = (qf @ k.float().transpose(1, 2)).requires_grad_(True)
+    qf, kf, vf = (t.float().requires_grad_(True) for t in (q, k, v))
+    scores = (qf @ kf.transpose(1, 2)).requires_grad_(True)
     scores.retain_grad()
     masked = (scores * inv_t).masked_fill(mask == 0, float('-inf'))
     p_ref = torch.softmax(masked, -1).nan_to_num(0.0)
-    (p_ref @ v.float()).backward(g.float())
+    (p_ref @ vf).backward(g.float())
     tol = dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(row_dot, (g.float() * out.float()).sum(-1) * inv_t, rtol=1e-3, atol=1e-3)
+    if BH * E >= 32 * BW:
+        grad_k = torch.full_like(k, float('nan'))
+        grad_v = torch.full_like(v, float('nan'))
+        rc = lib.spx_attention_backward_kv(
+            _lib.dtype_code(dtype), _lib.dev_ptr(g), _lib.dev_ptr(q), _lib.dev_ptr(v), _lib.dev_ptr(probs),
+            _lib.dev_ptr(row_dot), _lib.dev_ptr(grad_k), _lib.dev_ptr(grad_v), n_val, _lib.dev_ptr(indexes.col_ptr),
+            _lib.dev_ptr(indexes._bcsc_buf), _lib.IDX_BCSC_I64, inv_t, batch, Nt, Ns, E, BH, BW, _lib.current_stream(gpu))
+        _lib.check(rc, 'spx_attention_backward_kv')
+        torch.testing.assert_close(grad_v.float(), vf.grad, **tol)
+        torch.testing.assert_close(grad_k.float(), kf.grad, **tol)
     torch.testing.assert_close(indexes.inverse(probs).float(), p_ref.detach(), **tol)
     torch.testing.assert_close(indexes.inverse(grad_scores).float(), scores.grad, **tol)
     torch.testing.assert_close(grad_q.float(), qf.grad, **tol)
