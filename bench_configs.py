@@ -131,7 +131,7 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
                     fn(*leaves).backward(grad)
 
                 n_step = min(steps, 20)
-                for fused, name in ((True, 'c3 training step, fused forward and score-gradient kernels'),
+                for fused, name in ((True, 'c3 training step, fused forward, row-side and column-side backward kernels'),
                                     (False, 'c3 training step, three operators forward and six kernels backward')):
                     att_t._fused = fused
                     sec = time_eager(torch, lambda: step(att_t), n_step, 3) / n_step
