@@ -298,3 +298,30 @@ def test_attention_backward_scores_kernel(dtype, BH, BW, E, element_mask, gpu, b
     torch.testing.assert_close(indexes.inverse(grad_scores).float(), scores.grad, **tol)
     torch.testing.assert_close(grad_q.float(), qf.grad, **tol)
     assert float(grad_q[:, :BH].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('needs', [(True, False, False), (False, True, False), (False, False, True), (True, False, True)])
+def test_attention_training_partial_gradients(needs, gpu, H=2, Nt=256, Ns=256, E=64, bh=64, bw=64):
+    """Only some of query / key / value require gradients: the fused backward returns exactly
+    those, equal to dense fp32 autograd."""
+    dtype = torch.float16
+    _, q = randn((H, Nt, E), 51, dtype)
+    _, k = randn((H, Ns, E), 52, dtype)
+    _, v = randn((H, Ns, E), 53, dtype)
+    _, g = randn((H, Nt, E), 54, dtype)
+    mask_np = ops.block_mask((Nt, Ns), (bh, bw), 0.5, seed=55)
+    mask_np[:, :bw] = 1
+    mask = torch.from_numpy(mask_np).to(gpu)
+    att = SparseAttention(mask=mask)
+    leaves = [t.to(gpu).requires_grad_(n) for t, n in zip((q, k, v), needs)]
+    att.build(train_config(bh, bw), sample_inputs=[t.detach() for t in leaves])
+    out = att(*leaves)
+    out.backward(g.to(gpu))
+    ref = [t.detach().float().requires_grad_(n) for t, n in zip(leaves, needs)]
+    scores = (ref[0] @ ref[1].transpose(1, 2) / float(np.sqrt(E))).masked_fill(mask == 0, float('-inf'))
+    (torch.softmax(scores, -1) @ ref[2]).backward(g.to(gpu).float())
+    for t, r, n in zip(leaves, ref, needs):
+        if n:
+            torch.testing.assert_close(t.grad.float(), r.grad, rtol=2e-2, atol=2e-2)
+        else:
+            assert t.grad is None
