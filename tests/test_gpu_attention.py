@@ -325,3 +325,33 @@ def test_attention_training_partial_gradients(needs, gpu, H=2, Nt=256, Ns=256, E
             torch.testing.assert_close(t.grad.float(), r.grad, rtol=2e-2, atol=2e-2)
         else:
             assert t.grad is None
+
+
+def test_attention_training_after_mask_update(gpu, H=3, Nt=256, Ns=256, E=64, bh=64, bw=64):
+    """update_mask between training steps: the fused forward and both backward kernels follow
+    the rebuilt index (BCSR and BCSC)."""
+    dtype = torch.float16
+    _, q = randn((H, Nt, E), 61, dtype)
+    _, k = randn((H, Ns, E), 62, dtype)
+    _, v = randn((H, Ns, E), 63, dtype)
+    _, g = randn((H, Nt, E), 64, dtype)
+    att = None
+    for seed in range(3):
+        mask_np = ops.block_mask((Nt, Ns), (bh, bw), 0.5, seed=70 + seed)
+        mask_np[:bh, :bw] = 1
+        mask = torch.from_numpy(mask_np).to(gpu)
+        leaves = [t.to(gpu).requires_grad_(True) for t in (q, k, v)]
+        if att is None:
+            att = SparseAttention(mask=mask)
+            att.build(train_config(bh, bw), sample_inputs=[t.detach() for t in leaves])
+        else:
+            att.update_mask(mask)
+        out = att(*leaves)
+        out.backward(g.to(gpu))
+        ref = [t.detach().float().requires_grad_(True) for t in leaves]
+        scores = (ref[0] @ ref[1].transpose(1, 2) / float(np.sqrt(E))).masked_fill(mask == 0, float('-inf'))
+        ref_out = torch.softmax(scores, -1).nan_to_num(0.0) @ ref[2]
+        ref_out.backward(g.to(gpu).float())
+        torch.testing.assert_close(out.detach().float(), ref_out.detach(), rtol=2e-2, atol=2e-2)
+        for t, r in zip(leaves, ref):
+            torch.testing.assert_close(t.grad.float(), r.grad, rtol=2e-2, atol=2e-2)
