@@ -310,9 +310,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
     const int e_begin = p.row_ptr[br];
     const int e_end = p.row_ptr[br + 1];
     u32x4 kr[NV], vr[NV];
-    int bc = 0;
+    // bc: block column of the tile in the staging registers; bc_next: the one after it, fetched
+    // a whole step before its address is needed (the wait for an index entry that is used at
+    // once would stall every step for an L2 round trip)
+    int bc = 0, bc_next = 0;
     if (e_begin < e_end) {
         bc = p.bcsr_idx[e_begin] & 0xffff;
+        bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
         const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
         for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
@@ -328,7 +332,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
         for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
         const int key0 = bc * BW;
         // next live block (the last step re-reads its own block; the copy is not used)
-        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        bc = bc_next;
+        bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
         {
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -560,7 +565,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
     bool fresh = true;
     float l_part = 0.f;
     {
+        // (the entry after next is fetched a whole step before its address is needed)
         int bc = p.bcsr_idx[e_begin] & 0xffff;
+        int bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
         {
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -572,7 +579,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
 #pragma unroll
             for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + k_dst + i * RSTEP * KP) = kr[i];
             const int key0 = bc * BW;
-            bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+            bc = bc_next;
+            bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
             {
                 const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -635,6 +643,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
 #pragma unroll
     for (int t = 0; t < ET; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     int bc = p.bcsr_idx[e_begin] & 0xffff;
+    int bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
     {
         const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -650,7 +659,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
 #pragma unroll
         for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
         const int key0 = bc * BW;
-        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        bc = bc_next;
+        bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
         {
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -868,12 +878,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
     const int e_begin = p.row_ptr[br];
     const int e_end = p.row_ptr[br + 1];
     u32x4 kr[NV], vr[NV], pr[PN];
-    int bc = 0;
+    int bc = 0, bc_next = 0;   // the entry after next is fetched a whole step before its address is needed
     if (e_begin < e_end) {
 #pragma unroll
         for (int i = 0; i < PN; ++i)
             pr[i] = *reinterpret_cast<const u32x4*>(P + (int64_t)e_begin * (16 * WAVES * BW) + wave_off + i * 512);
         bc = p.bcsr_idx[e_begin] & 0xffff;
+        bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
         const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
         for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
@@ -890,7 +901,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
 #pragma unroll
         for (int i = 0; i < PN; ++i) *reinterpret_cast<u32x4*>(ptile + pt_vec[i]) = pr[i];
         const int e_next = e + 1 < e_end ? e + 1 : e;
-        bc = p.bcsr_idx[e_next] & 0xffff;
+        bc = bc_next;
+        bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
         {
 #pragma unroll
             for (int i = 0; i < PN; ++i)
@@ -1308,9 +1320,10 @@ __global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams 
     const int e_begin = p.row_ptr[br];
     const int e_end = p.row_ptr[br + 1];
     u32x4 kr[NV], vr[NV];
-    int bc = 0;
+    int bc = 0, bc_next = 0;   // the entry after next is fetched a whole step before its address is needed
     if (e_begin < e_end) {
         bc = p.bcsr_idx[e_begin] & 0xffff;
+        bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
         const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
         for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
@@ -1326,7 +1339,8 @@ __global__ __launch_bounds__(64 * WAVES, 2) void attention_kernel_v3(AttnParams 
         for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
         const int key0 = bc * BW;
         // next live block (the last step re-reads its own block; the copy is not used)
-        bc = p.bcsr_idx[e + 1 < e_end ? e + 1 : e] & 0xffff;
+        bc = bc_next;
+        bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
         {
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
