@@ -127,7 +127,7 @@ def main():
                     help='also run one plain 256 MiB device copy, so that a rocprofv3 --pmc run of this '
                          'command shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic')
     ap.add_argument('--config', default='headline',
-                    help="'headline' (default, the one JSON line the harness reads) or one of c1..c5 / all: "
+                    help="'headline' (default, the one JSON line the harness reads) or one of c1..c5 / seqlen / all: "
                          "secondary measurements of the other benchmark configurations")
     ap.add_argument('--attention-tile-cfg', type=int, default=0,
                     help='tile configuration of the fused attention kernel in --config c3 (0 = the library\'s choice)')

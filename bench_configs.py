@@ -36,7 +36,7 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
     from sparta_amd.tesa import get_bcs_function
 
     dev = torch.device('cuda:0')
-    todo = ['c1', 'c2', 'c3', 'c4', 'c5'] if which == 'all' else [which]
+    todo = ['c1', 'c2', 'c3', 'c4', 'c5', 'seqlen'] if which == 'all' else [which]
     steps = min(steps, 100)
 
     def timed(fn):
@@ -207,3 +207,21 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
             w0 = mods[0].weight
             sec = timed(lambda: torch.matmul(x, w0.t()))
             _emit('c5 dense torch.matmul with the same FLOPs (16384x1024x4096)', sec, flops=2.0 * n_tok * K * N)
+
+        if 'seqlen' in todo:
+            # SeqlenDynamicSparseAttention: the reference test's shape (fp32) and a larger fp16 one;
+            # lengths uniform in [1, N); dense SDPA over the padded batch for comparison
+            for (B, H, N, E), dtype in (((12, 20, 256, 64), torch.float32), ((32, 12, 1024, 64), torch.float16)):
+                g = torch.Generator().manual_seed(2022)
+                q, k_, v = (torch.rand((B, H, N, E), generator=g).to(dtype).to(dev) for _ in range(3))
+                lens = np.random.default_rng(2022).integers(1, N, size=B).astype(np.int32)
+                seqlens = torch.from_numpy(lens).to(dev)
+                att = sparta.nn.SeqlenDynamicSparseAttention(global_mode=False)
+                flops = float(sum(4.0 * int(L) * int(L) * E * H for L in lens))
+                sec = timed(lambda: att(q, k_, v, seqlens))
+                name = str(dtype).replace('torch.', '')
+                _emit(f'seqlen attention {B}x{H}x{N}x{E} {name}, lengths uniform in [1, {N})', sec, flops=flops,
+                      bytes_alg=float(sum(4 * int(L) * E * H for L in lens)) * q.element_size())
+                sec = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k_, v, scale=1.0))
+                _emit(f'seqlen shape, dense torch SDPA over the padded batch ({name})', sec, flops=4.0 * B * H * N * N * E)
+

@@ -42,6 +42,8 @@ struct AttnParams {
     int bcsc_wide;        // 1: int64 entries (bcsr_pos << 32 | col << 16 | row), 0: int32 (col << 16 | row)
     void* grad_k;
     void* grad_v;
+    const int32_t* seqlens;   // sequence-length mode of the pipelined kernel: one length per `heads` entries
+    int heads;
 };
 
 template <typename T> struct AttnMma;
@@ -235,8 +237,12 @@ template <> struct AttnPack<bf16_t> {
     __device__ static bf16x8 pack(f32x8 v) { return __builtin_convertvector(v, bf16x8); }
 };
 
-template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
+// SEQ: no index and no mask bytes; entry b attends over its first L = seqlens[b / heads]
+// positions: the walk covers the key blocks below L, a key is live iff its position is, and
+// queries at or past L give zeros (block rows at or past L walk nothing).
+template <typename T, int BW, int E, int WAVES, bool HAS_MASK, bool SEQ = false>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(AttnParams p, int nbr, int batch) {
+    static_assert(!SEQ || HAS_MASK, "the sequence-length mode masks by key position");
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
     constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
@@ -307,16 +313,22 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
     const int k_sw = r16 & 7;
     const int v_src = BW * KP + (g4 * 4 + (r16 >> 2)) * VP + (r16 & 3) * 8;
 
-    const int e_begin = p.row_ptr[br];
-    const int e_end = p.row_ptr[br + 1];
+    int seq_len = 0;
+    if constexpr (SEQ) {
+        seq_len = p.seqlens[b / p.heads];
+        seq_len = seq_len < 0 ? 0 : (seq_len > p.Ns ? p.Ns : seq_len);
+    }
+    const int e_begin = SEQ ? 0 : p.row_ptr[br];
+    const int e_end = SEQ ? (br * (16 * WAVES) < seq_len ? (seq_len + BW - 1) / BW : 0) : p.row_ptr[br + 1];
+    auto column = [&](int e) { return SEQ ? e : (p.bcsr_idx[e] & 0xffff); };
     u32x4 kr[NV], vr[NV];
     // bc: block column of the tile in the staging registers; bc_next: the one after it, fetched
     // a whole step before its address is needed (the wait for an index entry that is used at
     // once would stall every step for an L2 round trip)
     int bc = 0, bc_next = 0;
     if (e_begin < e_end) {
-        bc = p.bcsr_idx[e_begin] & 0xffff;
-        bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
+        bc = column(e_begin);
+        bc_next = column(e_begin + 1 < e_end ? e_begin + 1 : e_begin);
         const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
         for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
@@ -333,7 +345,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
         const int key0 = bc * BW;
         // next live block (the last step re-reads its own block; the copy is not used)
         bc = bc_next;
-        bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
+        bc_next = column(e + 2 < e_end ? e + 2 : e_end - 1);
         {
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
@@ -342,7 +354,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
             for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
         }
         unsigned live[KT];
-        if constexpr (HAS_MASK) {
+        if constexpr (SEQ) {
+            // one byte per key of this lane, set while the key position is below the length
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const int left = seq_len - (key0 + kt * 16 + g4 * 4);   // live keys among the lane's four
+                live[kt] = left >= 4 ? 0x01010101u : left <= 0 ? 0u : (0x01010101u >> (8 * (4 - left)));
+            }
+        } else if constexpr (HAS_MASK) {
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
                 live[kt] = *reinterpret_cast<const uint32_t*>(p.mask + (int64_t)qrow * p.Ns + key0 + kt * 16 + g4 * 4);
@@ -417,7 +436,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
 
     // every accumulator row of lacc holds the row sum of query r16
     const float l_run = lacc[0];
-    const float inv_l = l_run > 0.f ? 1.f / l_run : 0.f;
+    const float inv_l = (l_run > 0.f && (!SEQ || qrow < seq_len)) ? 1.f / l_run : 0.f;
     uint64_t pieces[ET];
 #pragma unroll
     for (int t = 0; t < ET; ++t) {
@@ -459,6 +478,34 @@ static int launch_attention_v2_inst(const AttnParams& p, int batch, hipStream_t 
     }
     SPX_LAUNCH_CHECK("attention_kernel_v2");
     return 0;
+}
+
+// Sequence-length mode of the pipelined kernel: square tiles of 64 (N a multiple of 64) or 32.
+template <typename T, int TB, int E>
+static int launch_attention_v2_seq_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr int TILE = TB * (E * 4 + 32);
+    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    const int nbr = p.Nt / TB;
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_kernel_v2<T, TB, E, TB / 16, true, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_kernel_v2)");
+    }
+    hipLaunchKernelGGL((attention_kernel_v2<T, TB, E, TB / 16, true, true>), dim3((unsigned)groups), dim3(4 * TB), smem, st, p, nbr, batch);
+    SPX_LAUNCH_CHECK("attention_kernel_v2 (sequence lengths)");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_v2_seq(const AttnParams& p, int batch, int E, hipStream_t st) {
+    const int TB = p.Nt % 64 == 0 ? 64 : 32;
+    if (TB == 64 && E == 64) return launch_attention_v2_seq_inst<T, 64, 64>(p, batch, st);
+    if (TB == 64 && E == 128) return launch_attention_v2_seq_inst<T, 64, 128>(p, batch, st);
+    if (TB == 32 && E == 64) return launch_attention_v2_seq_inst<T, 32, 64>(p, batch, st);
+    if (TB == 32 && E == 128) return launch_attention_v2_seq_inst<T, 32, 128>(p, batch, st);
+    return fail(SPX_E_CONFIG, "the pipelined sequence-length kernel takes head dims 64 / 128 (got %d)", E);
 }
 
 // The pipelined kernel covers query blocks of 32 / 64 / 128, key blocks of 32 / 64 / 128
@@ -1703,6 +1750,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.probs = nullptr; p.probs_batch = 0;
     p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr; p.row_dot = nullptr;
     p.col_ptr = nullptr; p.bcsc_idx = nullptr; p.bcsc_wide = 0; p.grad_k = nullptr; p.grad_v = nullptr;
+    p.seqlens = nullptr; p.heads = 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel;
     // 3: pipelined kernel on 32x32x16 MFMAs (one wavefront per 32 queries; measured within a few
@@ -1748,6 +1796,7 @@ extern "C" int spx_attention_forward_train(int dtype, const void* q, const void*
     p.probs = probs; p.probs_batch = probs_batch_stride;
     p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr; p.row_dot = nullptr;
     p.col_ptr = nullptr; p.bcsc_idx = nullptr; p.bcsc_wide = 0; p.grad_k = nullptr; p.grad_v = nullptr;
+    p.seqlens = nullptr; p.heads = 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (dtype == SPX_F16) return launch_attention_train<_Float16>(p, batch, BW, E, st);
     return launch_attention_train<bf16_t>(p, batch, BW, E, st);
@@ -1833,10 +1882,21 @@ extern "C" int spx_attention_seqlen_forward(int dtype, const void* q, const void
     SPX_REQUIRE(q && k && v && out && seqlens, SPX_E_NULL, "a required buffer is NULL");
     SPX_REQUIRE(aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(out, 16), SPX_E_ALIGN,
                 "q, k, v, out must be 16-byte aligned");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    // 16-bit types with head dims 64 / 128 run the pipelined fused kernel in its
+    // sequence-length mode; everything else the 16 x 16 x 16 kernel below
+    if (dtype != SPX_F32 && (E == 64 || E == 128)) {
+        AttnParams ap = {};
+        ap.q = q; ap.k = k; ap.v = v; ap.out = out;
+        ap.inv_t = inv_temperature;
+        ap.Nt = N; ap.Ns = N; ap.BH = N % 64 == 0 ? 64 : 32;
+        ap.seqlens = seqlens; ap.heads = heads;
+        if (dtype == SPX_F16) return launch_attention_v2_seq<_Float16>(ap, batch * heads, E, st);
+        return launch_attention_v2_seq<bf16_t>(ap, batch * heads, E, st);
+    }
     SeqlenParams p;
     p.q = q; p.k = k; p.v = v; p.out = out; p.seqlens = seqlens;
     p.inv_t = inv_temperature; p.heads = heads; p.N = N;
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     switch (dtype) {
         case SPX_F32: return launch_attention_seqlen<float>(p, batch * heads, E, st);
         case SPX_F16: return launch_attention_seqlen<_Float16>(p, batch * heads, E, st);
