@@ -16,6 +16,18 @@ def _grid_attention(n_blocks=64, seed=2022):
     return grid
 
 
+_RESULTS = []
+
+
+def _close(torch, got, want, what, rtol=1e-2, atol=1e-2):
+    """Every measurement below is preceded by this comparison with a dense fp32 torch
+    computation of the same inputs on the GPU; a mismatch aborts the benchmark."""
+    try:
+        torch.testing.assert_close(got.float(), want.float(), rtol=rtol, atol=atol)
+    except AssertionError as exc:
+        raise AssertionError(f'{what}: result differs from the dense computation\n{exc}') from None
+
+
 def _emit(name, sec, flops=None, bytes_alg=None, extra=None):
     out = {'config': name, 'ms': sec * 1e3}
     if flops:
@@ -25,10 +37,19 @@ def _emit(name, sec, flops=None, bytes_alg=None, extra=None):
         out['algorithmic_gbs'] = bytes_alg / sec / 1e9
         out['hbm_frac'] = bytes_alg / sec / 1e9 / 8000.0
     out.update(extra or {})
-    print(json.dumps(out), flush=True)
+    _RESULTS.append(out)
+    if _emit.verbose:
+        print(json.dumps(out), flush=True)
 
 
-def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
+_emit.verbose = True
+
+
+def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brief=False, verbose=True):
+    """Runs the named configurations ('all', one name, or a list of names); every timed
+    operator is first compared with the dense computation.  `brief` leaves out the
+    comparison methods (dense torch, unfused pipelines, training steps); `verbose`
+    prints one JSON object per measurement.  Returns the list of measurements."""
     import torch
     import sparta_amd as sparta
     from oracle import ops
@@ -36,8 +57,10 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
     from sparta_amd.tesa import get_bcs_function
 
     dev = torch.device('cuda:0')
-    todo = ['c1', 'c2', 'c3', 'c4', 'c5', 'seqlen'] if which == 'all' else [which]
+    todo = ['c1', 'c2', 'c3', 'c4', 'c5', 'seqlen'] if which == 'all' else ([which] if isinstance(which, str) else list(which))
     steps = min(steps, 100)
+    del _RESULTS[:]
+    _emit.verbose = verbose
 
     def timed(fn):
         try:
@@ -56,16 +79,19 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
             lin = torch.nn.Linear(1024, 1024, device=dev)
             lin.weight.copy_((w * torch.from_numpy(mask_np)).to(dev))
             lin.bias.copy_(b.to(dev))
-            for blk in (16, 32):
+            want = torch.nn.functional.linear(x, lin.weight, lin.bias)
+            for blk in ((16,) if brief else (16, 32)):
                 op = sparta.nn.SparseLinear(lin, weight_mask=torch.from_numpy(mask_np).to(dev))
                 cfg = dict(cfg32, BLOCK_SIZE_K_VALUE=blk, BLOCK_SIZE_N_VALUE=blk)
                 op.build({'forward:C': cfg}, sample_inputs=[x])
                 nnz = op.get_sparse_indexes('B').block_nnz
+                _close(torch, op(x), want, f'c1 {blk}x{blk}', rtol=1e-4, atol=1e-4)
                 sec = timed(lambda: op(x))
                 _emit(f'c1 SparseLinear fp32 1024^3 8x8@90%, {blk}x{blk} tiles', sec, flops=2.0 * 1024 * nnz * blk * blk,
                       extra={'nnz_blocks': nnz, 'useful_gflop_8x8': 0.215})
-            sec = timed(lambda: lin(x))
-            _emit('c1 dense torch Linear fp32', sec, flops=2.0 * 1024 ** 3)
+            if not brief:
+                sec = timed(lambda: lin(x))
+                _emit('c1 dense torch Linear fp32', sec, flops=2.0 * 1024 ** 3)
 
         if 'c2' in todo:
             M = K = N = 4096
@@ -73,6 +99,7 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
             A = torch.randn((1, M, K), generator=g).half().to(dev)
             B = torch.randn((1, N, K), generator=g).half().to(dev)
             mask = torch.from_numpy(ops.block_mask((4096, 4096), (32, 32), 0.95, seed=2022)).to(dev)
+            maskf = mask.float()
             for mode in ('sdd', 'dsd', 'dds'):
                 k = SparTASparseMatMulKernel(mode=mode, biased=False, transpose_A=False, transpose_B=True, compressed=True)
                 port = {'sdd': 'A', 'dsd': 'B', 'dds': 'C'}[mode]
@@ -82,13 +109,28 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
                 idx = k.ports[port].indexes
                 args = {'sdd': (idx.convert(A), B), 'dsd': (A, idx.convert(B)), 'dds': (A, B)}[mode]
                 nnz = idx.block_nnz
+                if mode == 'sdd':
+                    want = torch.matmul(A[0].float() * maskf, B[0].float().t())
+                elif mode == 'dsd':
+                    want = torch.matmul(A[0].float(), (B[0].float() * maskf).t())
+                else:
+                    want = idx.convert(torch.matmul(A[0].float(), B[0].float().t()))
+                _close(torch, k(*args).reshape(want.shape), want, f'c2 {mode}')
+                del want
                 sec = timed(lambda: k(*args))
                 _emit(f'c2 {mode} 4096^3 fp16 32x32@95%', sec, flops=nnz * 2.0 * 4096 * 1024,
                       bytes_alg=2 * 4096 * 4096 * 2 + nnz * 2048, extra={'nnz_blocks': nnz})
-            sec = timed(lambda: torch.matmul(A[0], B[0].t()))
-            _emit('c2 dense torch.matmul fp16 4096^3', sec, flops=2.0 * 4096 ** 3)
+            if not brief:
+                sec = timed(lambda: torch.matmul(A[0], B[0].t()))
+                _emit('c2 dense torch.matmul fp16 4096^3', sec, flops=2.0 * 4096 ** 3)
+            from oracle import bcs
+            mask_np = mask.cpu().numpy()
             for both in (False, True):
                 fn = get_bcs_function(32, 32, True, both)
+                built = fn.build_indexes(mask)
+                row_ptr, bcsr, _ = bcs.build_bcsr(mask_np, 32, 32)
+                assert np.array_equal(built.row_ptr.cpu().numpy(), row_ptr), 'c2 index build: row_ptr differs from the oracle'
+                assert np.array_equal(built.BCSR_idx.cpu().numpy(), bcsr), 'c2 index build: BCSR_idx differs from the oracle'
                 sec = timed(lambda: fn.build_indexes(mask))
                 _emit(f"c2 index build 4096x4096 mask ({'BCSR+BCSC' if both else 'BCSR'})", sec, bytes_alg=4096 * 4096)
 
@@ -106,10 +148,18 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
                       sample_inputs=[q, k_, v])
             nnz = att._sparse_port.indexes.block_nnz
             flops = 2 * nnz * 2.0 * blk * blk * E * BH
+            sample = [0, 42, 95]
+            scores = torch.matmul(q[sample].float(), k_[sample].float().transpose(1, 2)) / math.sqrt(E)
+            scores.masked_fill_(mask == 0, float('-inf'))
+            want = torch.matmul(torch.softmax(scores, -1), v[sample].float())
+            del scores
+            _close(torch, att(q, k_, v)[sample], want, 'c3 fused attention (heads 0, 42, 95)')
             sec = timed(lambda: att(q, k_, v))
             _emit('c3 fused sparse attention 96x4096x64 fp16, 64x64 blocks', sec, flops=flops,
                   bytes_alg=4 * BH * N * E * 2, extra={'nnz_blocks': nnz, 'tile_cfg': attention_tile_cfg})
+        if 'c3' in todo and not brief:
             att._fused = False
+            _close(torch, att(q, k_, v)[sample], want, 'c3 three-operator pipeline (heads 0, 42, 95)')
             sec = timed(lambda: att(q, k_, v))
             _emit('c3 three-operator pipeline (dds, softmax, sdd)', sec, flops=flops)
             qq, kk, vv = (t.view(8, 12, N, E) for t in (q, k_, v))
@@ -161,7 +211,11 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
             masks1 = [topk_mask((F, D), s) for s in range(4)]
             masks2 = [topk_mask((D, F), 100 + s) for s in range(4)]
             cfg = {'forward:C': {'_impl': 'openai', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 32}}
-            for dynamic in (True, False):
+            def dense_ffn(m1, m2):
+                h = torch.relu(torch.matmul(x.float(), (l1.weight.float() * m1.float()).t())).half()
+                return torch.matmul(h.float(), (l2.weight.float() * m2.float()).t())
+
+            for dynamic in ((True,) if brief else (True, False)):
                 op1 = sparta.nn.SparseLinear(l1, weight_mask=masks1[0], dynamic=dynamic)
                 op2 = sparta.nn.SparseLinear(l2, weight_mask=masks2[0], dynamic=dynamic)
                 op1.build(cfg, sample_inputs=[x])
@@ -174,18 +228,24 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
                     op2.update_mask(weight_mask=m2)
                     return op2(torch.relu(op1(x)))
 
+                _close(torch, step(), dense_ffn(m1, m2), f'c4 dynamic={dynamic}')
                 if dynamic:
                     sec = timed(step)  # no host sync inside: capturable
+                    # a new mask in the same buffers: the next call rebuilds both indexes from it
+                    m1.copy_(masks1[2])
+                    m2.copy_(masks2[2])
+                    _close(torch, step(), dense_ffn(masks1[2], masks2[2]), 'c4 after a mask update')
                     tag = 'hip graph replay'
                 else:
                     sec = time_eager(torch, step, steps, warmup) / steps
                     tag = 'eager (one host sync per rebuild, as in the reference)'
                 _emit(f'c4 dynamic-mask FFN 8192x768->3072->768 fp16, rebuild timed, dynamic={dynamic}', sec,
-                      flops=2 * 2.0 * T * 115 * 32 * 64, extra={'timing': tag})
-            fwd_only = timed(lambda: op2(torch.relu(op1(x))))
-            _emit('c4 same FFN, masks fixed (no rebuild)', fwd_only, flops=2 * 2.0 * T * 115 * 32 * 64)
-            sec = timed(lambda: l2(torch.relu(l1(x))))
-            _emit('c4 dense torch FFN fp16', sec, flops=2 * 2.0 * T * D * F)
+                      flops=2 * 2.0 * T * 116 * 32 * 64, extra={'timing': tag})
+            if not brief:
+                fwd_only = timed(lambda: op2(torch.relu(op1(x))))
+                _emit('c4 same FFN, masks fixed (no rebuild)', fwd_only, flops=2 * 2.0 * T * 116 * 32 * 64)
+                sec = timed(lambda: l2(torch.relu(l1(x))))
+                _emit('c4 dense torch FFN fp16', sec, flops=2 * 2.0 * T * D * F)
 
         if 'c5' in todo:
             n_tok, n_exp, K, N = 16384, 8, 1024, 4096
@@ -199,14 +259,21 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
             p = np.arange(1, n_exp + 1, dtype=np.float64) ** -1.2
             ids = torch.from_numpy(np.random.default_rng(2022).choice(n_exp, size=n_tok, p=p / p.sum()).astype(np.int32)).to(dev)
             x = torch.randn((n_tok, K), generator=g).half().to(dev)
-            moe(x, ids)
+            got = moe(x, ids)
+            want = torch.empty((n_tok, N), dtype=torch.float32, device=dev)
+            for e in range(n_exp):
+                rows = (ids == e).nonzero().flatten()
+                want[rows] = torch.matmul(x[rows].float(), mods[e].weight.float().t())
+            _close(torch, got, want, 'c5 MoE forward')
+            del want, got
             sec = timed(lambda: moe(x, ids))
             _emit('c5 MoE forward 16384 tok, 1024->4096, 8 experts Zipf(1.2), index rebuild included', sec,
                   flops=2.0 * n_tok * K * N, bytes_alg=(n_tok * K + n_exp * K * N + n_tok * N) * 2,
                   extra={'expert_counts': moe.expert_count.cpu().tolist()})
-            w0 = mods[0].weight
-            sec = timed(lambda: torch.matmul(x, w0.t()))
-            _emit('c5 dense torch.matmul with the same FLOPs (16384x1024x4096)', sec, flops=2.0 * n_tok * K * N)
+            if not brief:
+                w0 = mods[0].weight
+                sec = timed(lambda: torch.matmul(x, w0.t()))
+                _emit('c5 dense torch.matmul with the same FLOPs (16384x1024x4096)', sec, flops=2.0 * n_tok * K * N)
 
         if 'seqlen' in todo:
             # SeqlenDynamicSparseAttention: the reference test's shape (fp32) and a larger fp16 one;
@@ -218,10 +285,19 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0):
                 seqlens = torch.from_numpy(lens).to(dev)
                 att = sparta.nn.SeqlenDynamicSparseAttention(global_mode=False)
                 flops = float(sum(4.0 * int(L) * int(L) * E * H for L in lens))
+                got = att(q, k_, v, seqlens)
+                for b in (0, B // 2, B - 1):
+                    L = int(lens[b])
+                    p = torch.softmax(torch.matmul(q[b, :, :L].float(), k_[b, :, :L].float().transpose(1, 2)), -1)
+                    tol = 1e-4 if dtype == torch.float32 else 1e-2
+                    _close(torch, got[b, :, :L], torch.matmul(p, v[b, :, :L].float()), f'seqlen attention b={b}', tol, tol)
+                    assert float(got[b, :, L:].abs().max()) == 0.0, 'seqlen attention: rows past the length are not zero'
                 sec = timed(lambda: att(q, k_, v, seqlens))
                 name = str(dtype).replace('torch.', '')
                 _emit(f'seqlen attention {B}x{H}x{N}x{E} {name}, lengths uniform in [1, {N})', sec, flops=flops,
                       bytes_alg=float(sum(4 * int(L) * E * H for L in lens)) * q.element_size())
-                sec = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k_, v, scale=1.0))
-                _emit(f'seqlen shape, dense torch SDPA over the padded batch ({name})', sec, flops=4.0 * B * H * N * N * E)
+                if not brief:
+                    sec = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k_, v, scale=1.0))
+                    _emit(f'seqlen shape, dense torch SDPA over the padded batch ({name})', sec, flops=4.0 * B * H * N * N * E)
+    return list(_RESULTS)
 

@@ -53,11 +53,32 @@ def matmul_data(torch, sparta, M, K, N, granularity, sparsity, dtype, device):
     return dict(A=A, B=B, C=C.to(dtype), grad_C=grad_C, grad_A=grad_A.to(dtype), grad_B=grad_B.to(dtype)), mask
 
 
-def time_fwd_bwd(torch, sparta, func, inputs, grad, targets, warmups, iters):
-    """Forward latency and (forward + backward) - forward, like profile_matmul (matmul.py:25-53)."""
+def _granularities(args):
+    return [args.granularity] if getattr(args, 'granularity', None) else GRANULARITY_LIST
+
+
+def _sparsities(args):
+    if getattr(args, 'sparsity', None) is not None:
+        return [args.sparsity]
+    return QUICK_SPARSITY if args.quick else SPARSITY_LIST
+
+
+def time_fwd_bwd(torch, sparta, func, inputs, grad, targets, warmups, iters, grad_targets=None):
+    """Forward latency and (forward + backward) - forward, like profile_matmul (matmul.py:25-53).
+    Before anything is timed the output is checked against `targets` and the input
+    gradients against `grad_targets` (the reference's bench checks both, matmul.py:30-36);
+    a mismatch raises AssertionError."""
     fwd = sparta.testing.profile(func, inputs, target_outputs=targets[:1] if targets else None,
                                  num_warmups=warmups, num_iters=iters)
     leaves = [t.detach().clone().requires_grad_(True) for t in inputs]
+    if grad_targets is not None:
+        func(*leaves).backward(grad)
+        for leaf, want in zip(leaves, grad_targets):
+            half = leaf.dtype in (torch.float16, torch.bfloat16)
+            tol = 1e-2 if half else 1e-4
+            # gradients are sums over up to thousands of products: scale the absolute bound by their size
+            scale = max(float(want.float().abs().max()), 1.0)
+            torch.testing.assert_close(leaf.grad.float(), want.float(), rtol=tol, atol=tol * scale)
 
     def both(*args):
         for leaf in leaves:
@@ -76,8 +97,8 @@ def sweep_matmul(args, torch, sparta, table_dir, device_name):
     dtype = {'fp16': torch.float16, 'fp32': torch.float32, 'bf16': torch.bfloat16}[args.dtype]
     table = None if args.tune else ct.load_config_table(table_dir, device_name)
     rows, tuned = [], []
-    for g in GRANULARITY_LIST:
-        for s in (QUICK_SPARSITY if args.quick else SPARSITY_LIST):
+    for g in _granularities(args):
+        for s in _sparsities(args):
             t0 = time.time()
             data, mask = matmul_data(torch, sparta, M, K, N, (g, g), s, dtype, 'cuda')
             dense = lambda A, B: torch.matmul(A, B.transpose(1, 2))
@@ -102,9 +123,12 @@ def sweep_matmul(args, torch, sparta, table_dir, device_name):
             else:
                 config = ct.lookup_config(table, granularity=g, sparsity=s)
                 op.build(config, sample_inputs=sample)
-            Bc = op.get_sparse_indexes('B').convert(data['B'])
+            indexes = op.get_sparse_indexes('B')
+            Bc = indexes.convert(data['B'])
+            # the gradient of the compressed operand covers the live blocks only
             lat = time_fwd_bwd(torch, sparta, op, [data['A'], Bc], data['grad_C'],
-                               [data['C']], args.warmups, args.iters)
+                               [data['C']], args.warmups, args.iters,
+                               grad_targets=[data['grad_A'], indexes.convert(data['grad_B'])])
             rows.append(('sparta_amd', M, K, N, g, s) + lat)
             print(f'matmul g={g} s={s}: dense fwd {lat_dense[0]*1e3:.1f} us bwd {lat_dense[1]*1e3:.1f} us | '
                   f'sparse fwd {lat[0]*1e3:.1f} us bwd {lat[1]*1e3:.1f} us  ({time.time()-t0:.1f} s)', flush=True)
@@ -117,8 +141,8 @@ def sweep_attention(args, torch, sparta, table_dir, device_name):
     dtype = {'fp16': torch.float16, 'fp32': torch.float32, 'bf16': torch.bfloat16}[args.dtype]
     table = None if args.tune else ct.load_config_table(table_dir, device_name)
     rows, tuned = [], []
-    for g in GRANULARITY_LIST:
-        for s in (QUICK_SPARSITY if args.quick else SPARSITY_LIST):
+    for g in _granularities(args):
+        for s in _sparsities(args):
             t0 = time.time()
             torch.manual_seed(2022)
             q = torch.rand((1, Nt, E), device='cuda').to(dtype)
@@ -135,6 +159,10 @@ def sweep_attention(args, torch, sparta, table_dir, device_name):
 
             lat_dense = time_fwd_bwd(torch, sparta, dense, [q, k, v], grad, None, args.warmups, args.iters)
             rows.append(('dense', Ns, Nt, E, g, s) + lat_dense)
+            # gradient targets from the masked dense computation in fp32
+            leaves = [t.float().requires_grad_(True) for t in (q, k, v)]
+            dense(*leaves).backward(grad.float())
+            grad_targets = [leaf.grad for leaf in leaves]
             if int(mask.sum()) == 0:
                 rows.append(('sparta_amd', Ns, Nt, E, g, s, 0.0, 0.0))
                 if args.tune:
@@ -152,7 +180,8 @@ def sweep_attention(args, torch, sparta, table_dir, device_name):
             else:
                 config = ct.lookup_config(table, granularity=g, sparsity=s)
                 op.build(config, sample_inputs=[q, k, v])
-            lat = time_fwd_bwd(torch, sparta, op, [q, k, v], grad, [want], args.warmups, args.iters)
+            lat = time_fwd_bwd(torch, sparta, op, [q, k, v], grad, [want], args.warmups, args.iters,
+                               grad_targets=grad_targets)
             rows.append(('sparta_amd', Ns, Nt, E, g, s) + lat)
             print(f'attention g={g} s={s}: dense fwd {lat_dense[0]*1e3:.1f} us bwd {lat_dense[1]*1e3:.1f} us | '
                   f'sparse fwd {lat[0]*1e3:.1f} us bwd {lat[1]*1e3:.1f} us  ({time.time()-t0:.1f} s)', flush=True)
@@ -164,6 +193,8 @@ def main():
     ap.add_argument('--op', choices=['matmul', 'attention'], default='matmul')
     ap.add_argument('--dtype', choices=['fp16', 'bf16', 'fp32'], default='fp16')
     ap.add_argument('--quick', action='store_true', help='4 sparsities per granularity instead of 12')
+    ap.add_argument('--granularity', type=int, default=None, help='run this mask granularity only')
+    ap.add_argument('--sparsity', type=float, default=None, help='run this sparsity only')
     ap.add_argument('--tune', type=int, default=0, help='tune every point with this many trials per kernel')
     ap.add_argument('--algo', choices=['rand', 'grid'], default='rand', help='search algorithm of --tune')
     ap.add_argument('--warmups', type=int, default=20)

@@ -121,7 +121,9 @@ int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
  * BCSFunctionContext.row_sum / col_sum (block_compressed.py:360-403) and
  * bcsr_val_sum_row / bcsr_val_sum_col (block_compressed.cu.j2:222-288).
  * axis 0: result [batch, H] = sum over W;  axis 1: result [batch, W] = sum
- * over H.  `result` must be zero-filled by the caller. idx as in spx_bcs_gather. */
+ * over H.  Every entry of `result` is written (zero where no block is live) and
+ * the additions follow the index order, so the sums are bit-identical from run
+ * to run (the reference adds with atomics).  idx as in spx_bcs_gather. */
 int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
                 int nnz, int batch, int H, int W, int BH, int BW, int dtype, int axis,
                 int64_t sparse_batch_stride, spx_stream_t stream);
@@ -268,9 +270,12 @@ int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const 
  * (csrc/moe_sparse_forward.cpp:7-25, csrc/moe_sparse_forward_kernel.cu.j2:58-116,
  * :120-325, :363-483) with a stable counting sort (no per-expert capacity) and a
  * gathered GEMM over a flattened (expert, row-tile) list.
- *   exp_ids int32 [n_tok], every value in [0, n_exp); expert_count int32 [n_exp];
+ *   exp_ids int32 [n_tok]; expert_count int32 [n_exp];
  *   expert_offset int32 [n_exp+1] exclusive prefix; token_perm int32 [n_tok]:
  *   token_perm[expert_offset[e] + j] = j-th token (ascending) routed to e.
+ *   Tokens whose id lies outside [0, n_exp) (the reference indexes out of bounds
+ *   for them) are listed, ascending, in token_perm[expert_offset[n_exp] .. n_tok)
+ *   and spx_moe_forward writes zero rows for them, so every row of out is defined.
  *   workspace: spx_moe_index_workspace_bytes(n_tok, n_exp) bytes, 256-byte aligned.
  *   tokens [n_tok,in_dim]; out [n_tok,out_dim];
  *   weight [n_exp,in_dim,out_dim] (weight_layout 0, the reference's stacked

@@ -33,12 +33,11 @@ def _hipcc() -> str:
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(OBJ, os.path.basename(src)[:-4] + '.o')
     if not force and os.path.exists(obj):
-        newest = max(
-            os.path.getmtime(os.path.join(d, f))
-            for d in (CSRC, os.path.join(ROOT, '..', 'include'))
-            for f in os.listdir(d)
-        )
-        if os.path.getmtime(obj) >= newest:
+        # an object is current when it is newer than its own source and every header
+        deps = [src] + [os.path.join(d, f)
+                        for d in (CSRC, os.path.join(ROOT, '..', 'include'))
+                        for f in os.listdir(d) if f.endswith(('.hpp', '.h'))]
+        if os.path.getmtime(obj) >= max(os.path.getmtime(d) for d in deps):
             return obj
     cmd = [_hipcc(), *HIPCC_FLAGS, '-c', src, '-o', obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)

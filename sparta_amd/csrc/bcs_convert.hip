@@ -114,36 +114,58 @@ struct SumParams {
     int64_t sparse_batch_stride;
 };
 
-// One workgroup per (block, batch): reduces its tile along one axis and adds the
-// BH (axis 0: one value per row) or BW (axis 1) partial sums into `result`.
+// One workgroup per (block row [axis 0] or block column [axis 1], batch): it scans the
+// index 256 entries at a time, and adds the tiles of its row / column in index order
+// (thread (o, s) owns output o and every per-th element along the reduced axis).  No
+// atomics: the order of the additions is fixed by the index, so the sums are the same
+// bits on every run, and every output is written exactly once (zero for an empty row).
 template <typename T>
 __global__ __launch_bounds__(256) void sum_kernel(SumParams p) {
     __shared__ float part[256];
-    const int i = blockIdx.x;
-    int br, bc;
-    decode_block(p.idx, p.idx_kind, i, br, bc);
-    const T* tile = reinterpret_cast<const T*>(p.sparse) + (int64_t)blockIdx.y * p.sparse_batch_stride +
-                    (int64_t)i * p.BH * p.BW;
+    __shared__ unsigned long long s_match[4];
+    const int mine = blockIdx.x;
     const int nout = p.axis == 0 ? p.BH : p.BW;   // <= 256
     const int nred = p.axis == 0 ? p.BW : p.BH;
     const int out_stride = p.axis == 0 ? p.BW : 1;
     const int red_stride = p.axis == 0 ? 1 : p.BW;
-    // threads: 256 / nout partial reducers per output
-    const int per = 256 / nout;
+    const int per = 256 / nout;  // partial reducers per output
     const int o = threadIdx.x / per;
     const int s = threadIdx.x - o * per;
+    const T* batch_base = reinterpret_cast<const T*>(p.sparse) + (int64_t)blockIdx.y * p.sparse_batch_stride;
     float acc = 0.f;
-    if (o < nout)
-        for (int k = s; k < nred; k += per)
-            acc += Elem<T>::to_float(tile[(int64_t)o * out_stride + (int64_t)k * red_stride]);
+    for (int base = 0; base < p.nnz; base += 256) {
+        const int i = base + threadIdx.x;
+        bool match = false;
+        if (i < p.nnz) {
+            int br, bc;
+            decode_block(p.idx, p.idx_kind, i, br, bc);
+            match = (p.axis == 0 ? br : bc) == mine;
+        }
+        const unsigned long long bits = __ballot(match);
+        if ((threadIdx.x & 63) == 0) s_match[threadIdx.x >> 6] = bits;
+        __syncthreads();
+        for (int w = 0; w < 4; ++w) {
+            unsigned long long todo = s_match[w];
+            while (todo) {
+                const int j = __ffsll((long long)todo) - 1;
+                todo &= todo - 1;
+                const int slot = base + w * 64 + j;  // values follow the order of this index
+                const T* tile = batch_base + (int64_t)slot * p.BH * p.BW;
+                if (o < nout)
+                    for (int k = s; k < nred; k += per)
+                        acc += Elem<T>::to_float(tile[(int64_t)o * out_stride + (int64_t)k * red_stride]);
+            }
+        }
+        __syncthreads();
+    }
     part[threadIdx.x] = acc;
     __syncthreads();
     if (threadIdx.x < nout) {
         float t = 0.f;
         for (int k = 0; k < per; ++k) t += part[threadIdx.x * per + k];
-        const int64_t pos = p.axis == 0 ? ((int64_t)blockIdx.y * p.H + (int64_t)br * p.BH + threadIdx.x)
-                                        : ((int64_t)blockIdx.y * p.W + (int64_t)bc * p.BW + threadIdx.x);
-        atomicAdd(p.result + pos, t);
+        const int64_t pos = p.axis == 0 ? ((int64_t)blockIdx.y * p.H + (int64_t)mine * p.BH + threadIdx.x)
+                                        : ((int64_t)blockIdx.y * p.W + (int64_t)mine * p.BW + threadIdx.x);
+        p.result[pos] = t;
     }
 }
 
@@ -186,7 +208,7 @@ extern "C" int spx_bcs_sum(const void* sparse, void* result, const void* idx, in
     p.idx = idx; p.idx_kind = idx_kind; p.nnz = nnz;
     p.H = H; p.W = W; p.BH = BH; p.BW = BW; p.axis = axis;
     p.sparse_batch_stride = sparse_batch_stride;
-    hipLaunchKernelGGL(sum_kernel<float>, dim3(nnz, batch, 1), dim3(256), 0,
+    hipLaunchKernelGGL(sum_kernel<float>, dim3(axis == 0 ? H / BH : W / BW, batch, 1), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(stream), p);
     SPX_LAUNCH_CHECK("sum_kernel");
     return 0;

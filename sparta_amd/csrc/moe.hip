@@ -24,6 +24,7 @@ constexpr int MOE_MAX_EXP = 2048; // LDS table capacity of the placement kernel
 // ---- index -------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, int n_tok, int n_exp,
                                                        int32_t* partial /* [n_chunk][n_exp] */) {
+    // n_exp here counts the pseudo expert that collects the tokens whose id is out of range
     extern __shared__ int hist[];
     for (int e = threadIdx.x; e < n_exp; e += 256) hist[e] = 0;
     __syncthreads();
@@ -31,8 +32,9 @@ __global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, i
     for (int i = threadIdx.x; i < MOE_CHUNK; i += 256) {
         const int t = base + i;
         if (t < n_tok) {
-            const int e = exp_ids[t];
-            if (e >= 0 && e < n_exp) atomicAdd(&hist[e], 1);
+            int e = exp_ids[t];
+            if (e < 0 || e >= n_exp - 1) e = n_exp - 1;
+            atomicAdd(&hist[e], 1);
         }
     }
     __syncthreads();
@@ -40,7 +42,9 @@ __global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, i
 }
 
 // One workgroup: exclusive scan of partial[] in (expert, chunk) order, in place;
-// also writes expert_count and expert_offset.
+// also writes expert_count [n_exp - 1] and expert_offset [n_exp] (n_exp counts the
+// pseudo expert of out-of-range ids, whose tokens follow those of the real experts, so
+// expert_offset[n_exp - 1] is the number of tokens with a valid id).
 __global__ __launch_bounds__(1024) void moe_scan_kernel(int32_t* partial, int n_chunk, int n_exp,
                                                         int32_t* expert_count, int32_t* expert_offset) {
     __shared__ int lds[32];
@@ -75,10 +79,9 @@ __global__ __launch_bounds__(1024) void moe_scan_kernel(int32_t* partial, int n_
         carry += total;
         __syncthreads();
     }
-    if (threadIdx.x == 0) expert_offset[n_exp] = carry;
     __syncthreads();
     // counts from consecutive offsets (offsets were written by this workgroup)
-    for (int e = threadIdx.x; e < n_exp; e += 1024) expert_count[e] = expert_offset[e + 1] - expert_offset[e];
+    for (int e = threadIdx.x; e + 1 < n_exp; e += 1024) expert_count[e] = expert_offset[e + 1] - expert_offset[e];
 }
 
 // Stable placement of one chunk.  Waves take 64 tokens at a time; inside a wave the
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, 
         int e = -1;
         if (t < n_tok) {
             e = exp_ids[t];
-            if (e < 0 || e >= n_exp) e = -1;
+            if (e < 0 || e >= n_exp - 1) e = n_exp - 1;  // out of range: the pseudo expert
         }
         // intra-wave rank and per-wave count of my expert
         int rank = 0, cnt = 0;
@@ -144,6 +147,52 @@ struct MoeParams {
     int w_kcontig;  // weight [E, N, K] if set, else [E, K, N]
 };
 
+// Which (expert, row tile) belongs to tile index y: one wavefront scans the per-expert
+// tile counts.  Expert n_exp is the pseudo expert of the tokens whose id was out of
+// range (token_perm[expert_offset[n_exp] .. n_tok)): its tiles are zero-filled instead
+// of multiplied.  found_e = -1 when y is past the last tile.
+template <int TM>
+__device__ __forceinline__ void moe_find_tile(const MoeParams& p, int y, int lane,
+                                              int& found_e, int& found_row0, int& found_rows) {
+    int tiles_before = 0;
+    found_e = -1; found_row0 = 0; found_rows = 0;
+    for (int e0 = 0; e0 <= p.n_exp && found_e < 0; e0 += 64) {
+        const int e = e0 + lane;
+        int cnt = 0, off = 0;
+        if (e <= p.n_exp) {
+            off = p.expert_offset[e];
+            cnt = (e < p.n_exp ? p.expert_offset[e + 1] : p.n_tok) - off;
+        }
+        const int tiles = (cnt + TM - 1) / TM;
+        const int inc = wave_inclusive_scan(tiles);
+        const int excl = tiles_before + inc - tiles;
+        const bool mine = y >= excl && y < excl + tiles;
+        const unsigned long long hit = __ballot(mine);
+        if (hit) {
+            const int src = __ffsll((long long)hit) - 1;
+            const int lt = y - __shfl(excl, src, 64);
+            found_e = e0 + src;
+            found_row0 = __shfl(off, src, 64) + lt * TM;
+            found_rows = min(TM, __shfl(cnt, src, 64) - lt * TM);
+        }
+        tiles_before += __shfl(inc, 63, 64);
+    }
+}
+
+// Zero rows token_perm[row0 .. row0 + rows) of `out`, columns n0 .. n0 + TN (16-byte stores).
+template <typename T>
+__device__ __forceinline__ void moe_zero_tile(const MoeParams& p, int row0, int rows, int n0, int TN, int nthreads) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    T* out = reinterpret_cast<T*>(p.out);
+    const int ncol = (min(n0 + TN, p.N) - n0) / VE;  // N is a multiple of VE
+    for (int v = threadIdx.x; v < rows * ncol; v += nthreads) {
+        const int r = v / ncol, c = v - r * ncol;
+        const int tok = p.token_perm[row0 + r];
+        *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n0 + c * VE) = u32x4{0u, 0u, 0u, 0u};
+    }
+}
+
 constexpr int MOE_TM = 128, MOE_TN = 128;
 // k per LDS stage: 128 bytes per row for every element type
 template <typename T> struct MoeKt { static constexpr int value = 128 / (int)sizeof(T); };
@@ -169,30 +218,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
     // ---- which (expert, row tile) is mine ------------------------------------------
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
-        const int y = blockIdx.y;
-        int tiles_before = 0;
-        int found_e = -1, found_row0 = 0, found_rows = 0;
-        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
-            const int e = e0 + lane;
-            int cnt = 0, off = 0;
-            if (e < p.n_exp) {
-                off = p.expert_offset[e];
-                cnt = p.expert_offset[e + 1] - off;
-            }
-            const int tiles = (cnt + MOE_TM - 1) / MOE_TM;
-            const int inc = wave_inclusive_scan(tiles);
-            const int excl = tiles_before + inc - tiles;
-            const bool mine = y >= excl && y < excl + tiles;
-            const unsigned long long hit = __ballot(mine);
-            if (hit) {
-                const int src = __ffsll((long long)hit) - 1;
-                const int lt = y - __shfl(excl, src, 64);
-                found_e = e0 + src;
-                found_row0 = __shfl(off, src, 64) + lt * MOE_TM;
-                found_rows = min(MOE_TM, __shfl(cnt, src, 64) - lt * MOE_TM);
-            }
-            tiles_before += __shfl(inc, 63, 64);
-        }
+        int found_e, found_row0, found_rows;
+        moe_find_tile<MOE_TM>(p, blockIdx.y, lane, found_e, found_row0, found_rows);
         if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
     }
     __syncthreads();
@@ -200,6 +227,10 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
     if (expert < 0) return;  // uniform: this tile index is past the last tile
     const int row0 = s_row0, rows = s_rows;
     const int n0 = blockIdx.x * MOE_TN;
+    if (expert == p.n_exp) {  // tokens without a valid expert id: zero rows
+        moe_zero_tile<T>(p, row0, rows, n0, MOE_TN, 256);
+        return;
+    }
 
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -402,30 +433,8 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
 
     if (threadIdx.x < 64) {
         const int lane = threadIdx.x;
-        const int y = blockIdx.y;
-        int tiles_before = 0;
-        int found_e = -1, found_row0 = 0, found_rows = 0;
-        for (int e0 = 0; e0 < p.n_exp && found_e < 0; e0 += 64) {
-            const int e = e0 + lane;
-            int cnt = 0, off = 0;
-            if (e < p.n_exp) {
-                off = p.expert_offset[e];
-                cnt = p.expert_offset[e + 1] - off;
-            }
-            const int tiles = (cnt + TM - 1) / TM;
-            const int inc = wave_inclusive_scan(tiles);
-            const int excl = tiles_before + inc - tiles;
-            const bool mine = y >= excl && y < excl + tiles;
-            const unsigned long long hit = __ballot(mine);
-            if (hit) {
-                const int src = __ffsll((long long)hit) - 1;
-                const int lt = y - __shfl(excl, src, 64);
-                found_e = e0 + src;
-                found_row0 = __shfl(off, src, 64) + lt * TM;
-                found_rows = min(TM, __shfl(cnt, src, 64) - lt * TM);
-            }
-            tiles_before += __shfl(inc, 63, 64);
-        }
+        int found_e, found_row0, found_rows;
+        moe_find_tile<TM>(p, blockIdx.y, lane, found_e, found_row0, found_rows);
         if (lane == 0) { s_expert = found_e; s_row0 = found_row0; s_rows = found_rows; }
     }
     __syncthreads();
@@ -433,6 +442,10 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
     if (expert < 0) return;
     const int row0 = s_row0, rows = s_rows;
     const int n0 = blockIdx.x * TN;
+    if (expert == p.n_exp) {  // tokens without a valid expert id: zero rows
+        moe_zero_tile<T>(p, row0, rows, n0, TN, NTH);
+        return;
+    }
 
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -606,7 +619,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
 
 template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
 static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
-    const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp;
+    const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp + 1;
     if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
     const int smem = NBUF * (TM + TN) * 128;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF>),
@@ -619,7 +632,7 @@ static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
 
 static size_t moe_index_ws(int n_tok, int n_exp) {
     const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
-    return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * n_exp * sizeof(int32_t), 256);
+    return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * (n_exp + 1) * sizeof(int32_t), 256);
 }
 
 }  // namespace spx
@@ -644,14 +657,14 @@ extern "C" int spx_moe_index(const int32_t* exp_ids, int n_tok, int n_exp,
     int32_t* partial = reinterpret_cast<int32_t*>(workspace);
     const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
     if (n_chunk > 0) {
-        hipLaunchKernelGGL(moe_hist_kernel, dim3(n_chunk), dim3(256), n_exp * sizeof(int), st, exp_ids, n_tok, n_exp, partial);
+        hipLaunchKernelGGL(moe_hist_kernel, dim3(n_chunk), dim3(256), (n_exp + 1) * sizeof(int), st, exp_ids, n_tok, n_exp + 1, partial);
         SPX_LAUNCH_CHECK("moe_hist_kernel");
     }
-    hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, st, partial, n_chunk, n_exp, expert_count, expert_offset);
+    hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, st, partial, n_chunk, n_exp + 1, expert_count, expert_offset);
     SPX_LAUNCH_CHECK("moe_scan_kernel");
     if (n_chunk > 0) {
-        hipLaunchKernelGGL(moe_place_kernel, dim3(n_chunk), dim3(256), 5 * n_exp * sizeof(int), st, exp_ids, n_tok, n_exp,
-                           partial, token_perm);
+        hipLaunchKernelGGL(moe_place_kernel, dim3(n_chunk), dim3(256), 5 * (n_exp + 1) * sizeof(int), st, exp_ids, n_tok,
+                           n_exp + 1, partial, token_perm);
         SPX_LAUNCH_CHECK("moe_place_kernel");
     }
     return 0;
@@ -695,7 +708,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
         }
 #undef SPX_MOE_DIRECT
     }
-    const int max_tiles = (n_tok + MOE_TM - 1) / MOE_TM + n_exp;
+    const int max_tiles = (n_tok + MOE_TM - 1) / MOE_TM + n_exp + 1;
     SPX_REQUIRE(max_tiles <= 65535, SPX_E_SHAPE, "too many row tiles for one launch");
     dim3 grid((out_dim + MOE_TN - 1) / MOE_TN, max_tiles, 1);
     const size_t smem = 2 * (size_t)MOE_TM * 128;

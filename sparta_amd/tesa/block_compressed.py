@@ -198,18 +198,21 @@ class BCSFunctionContext(TeSAFunctionContext):
         self._block_size = block_H * block_W
         self._BCSR = BCSR
         self._BCSC = BCSC
-        self._workspaces: Dict[Tuple[int, int, str], torch.Tensor] = {}
+        self._workspaces: Dict[Tuple[int, int], int] = {}
 
     # ---- index build ------------------------------------------------------------
     def _workspace(self, H: int, W: int, device) -> torch.Tensor:
-        key = (H, W, str(device))
-        ws = self._workspaces.get(key)
-        if ws is None:
+        """Scratch of one index build.  Taken from torch's caching allocator at every
+        build (only the byte count is cached): the allocator hands a block back out
+        only in stream order, so two operators - or two streams - that rebuild masks
+        of one shape at the same time never share the liveness / prefix buffers."""
+        key = (H, W)
+        nbytes = self._workspaces.get(key)
+        if nbytes is None:
             nbytes = _lib.load().spx_bcs_index_workspace_bytes(H, W, self._block_H, self._block_W)
             assert nbytes > 0, f'mask shape ({H}, {W}) does not fit block ({self._block_H}, {self._block_W})'
-            ws = torch.empty((nbytes,), dtype=torch.uint8, device=device)
-            self._workspaces[key] = ws
-        return ws
+            self._workspaces[key] = nbytes
+        return torch.empty((nbytes,), dtype=torch.uint8, device=device)
 
     def build_indexes(self, mask: torch.Tensor, capacity: Optional[int] = None) -> BCSIndexes:
         """mask: uint8 (or any 1-byte dtype) [H, W] on the GPU.  `capacity` bounds the
@@ -294,7 +297,7 @@ class BCSFunctionContext(TeSAFunctionContext):
         batch = int(np.prod(lead)) if lead else 1
         vals = sparse_val.contiguous().to(torch.float32)
         n_out = H if axis == 0 else W
-        result = torch.zeros((batch, n_out), dtype=torch.float32, device=vals.device)
+        result = torch.empty((batch, n_out), dtype=torch.float32, device=vals.device)
         with torch.cuda.device(vals.device):
             rc = _lib.load().spx_bcs_sum(
                 _lib.dev_ptr(vals), _lib.dev_ptr(result), _lib.dev_ptr(index), idx_kind, block_nnz,

@@ -20,6 +20,20 @@ class TeSAIndexes(abc.ABC):
     def get_mask(self) -> torch.Tensor:
         """The element mask actually covered by the index."""
 
+    def to(self, device: Any) -> 'TeSAIndexes':
+        """Move every tensor attribute to `device` (sparta/tesa/tesa_base.py:23-27; the
+        reference discards the moved copies and only updates `device`, here the
+        attributes are rebound).  Cached host-side values survive the move."""
+        self.device = torch.device(device)
+        for name, value in list(self.__dict__.items()):
+            if isinstance(value, torch.Tensor):
+                setattr(self, name, value.to(device))
+            elif isinstance(value, dict):
+                for key, item in value.items():
+                    if isinstance(item, torch.Tensor):
+                        value[key] = item.to(device)
+        return self
+
 
 class TeSAFunctionContext(abc.ABC):
     """Builds indexes for one sparsity format and converts values."""

@@ -94,7 +94,7 @@ def test_matmul_block_shapes(blocks, mode, gpu):
     # alternate dtype / transposes over the 27 block shapes to keep the suite short
     k = BLOCKS.index(blocks)
     dtype = [torch.float32, torch.float16, torch.bfloat16][k % 3]
-    run_case(gpu, mode, bool(k & 1), bool(k & 2), bool(k & 4), bool(k & 8) or True, dtype, blocks,
+    run_case(gpu, mode, bool(k & 1), bool(k & 2), bool(k & 4), bool(k & 8), dtype, blocks,
              batch=2, M=192, K=128, N=256, gran=(16, 16), sparsity=0.8, seed=k)
 
 

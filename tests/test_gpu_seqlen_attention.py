@@ -67,6 +67,24 @@ def test_seqlen_attention_shapes_and_edges(dtype, N, E, gpu, B=5, H=3):
     assert_close(out[4], full, dtype, 'full length')
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('N,E', [(256, 64), (192, 128), (96, 128), (1024, 64)])
+def test_seqlen_attention_pipelined_kernel_instantiations(dtype, N, E, gpu, H=2):
+    """16-bit types with head dim 64 / 128 run the pipelined fused kernel in its
+    sequence-length mode: key tiles of 64 (N % 64 == 0) or 32, each shape with several
+    key tiles and with lengths that end inside a tile, on a tile edge and one past it."""
+    seqlens = np.array([0, 1, 31, 32, 33, 63, 64, 65, N // 2 + 7, N - 1, N], dtype=np.int32)
+    seqlens = np.minimum(seqlens, N)
+    B = len(seqlens)
+    (q, k, v), (qn, kn, vn) = rand_qkv((B, H, N, E), 11, dtype)
+    att = SeqlenDynamicSparseAttention(global_mode=False)
+    out = att(q.to(gpu), k.to(gpu), v.to(gpu), torch.from_numpy(seqlens).to(gpu))
+    want = reference(qn, kn, vn, seqlens)
+    assert_close(out, want, dtype, f'seqlen attention (pipelined kernel) {dtype} N={N} E={E}')
+    for b, L in enumerate(seqlens):
+        assert float(out[b, :, int(L):].abs().max() if L < N else 0.0) == 0.0
+
+
 def test_seqlen_attention_rejects_bad_input(gpu):
     att = SeqlenDynamicSparseAttention(global_mode=False)
     q = torch.rand((2, 2, 48, 64), device=gpu)

@@ -210,6 +210,32 @@ def test_attention_all_ones_is_textbook():
         np.testing.assert_allclose(out[b, i], sum(p[j] * v[b, j] for j in range(6)), rtol=1e-8)
 
 
+def test_attention_masked_tiny_brute_force():
+    """Pure-Python loops over a random element mask (some rows fully masked, an explicit
+    temperature and the default sqrt(E)): live keys only in the sum, the maximum taken
+    over all keys as the reference's softmax does (sparta/testing/math.py:24), masked
+    rows exactly zero (the 1e-10 in the denominator makes them 0 / 1e-10)."""
+    import math
+    rng = np.random.default_rng(21)
+    B, Nt, Ns, E = 2, 5, 7, 3
+    q, k, v = rng.standard_normal((B, Nt, E)), rng.standard_normal((B, Ns, E)), rng.standard_normal((B, Ns, E))
+    mask = (rng.random((Nt, Ns)) < 0.5).astype(np.uint8)
+    mask[3] = 0
+    for temperature in (None, 0.7):
+        T = math.sqrt(E) if temperature is None else temperature
+        out = ops.attention_reference(q, k, v, mask, temperature=temperature)
+        for b in range(B):
+            for i in range(Nt):
+                s = [sum(q[b, i, e] * k[b, j, e] for e in range(E)) for j in range(Ns)]
+                top = max(s)
+                w = [math.exp((s[j] - top) / T) if mask[i, j] else 0.0 for j in range(Ns)]
+                tot = sum(w)
+                for e in range(E):
+                    want = sum(w[j] * v[b, j, e] for j in range(Ns)) / (tot + 1e-10)  # math.py:27
+                    assert abs(out[b, i, e] - want) < 1e-12
+        assert np.all(out[:, 3] == 0.0)
+
+
 def test_moe_reference_properties():
     rng = np.random.default_rng(14)
     tokens = rng.standard_normal((10, 6))
