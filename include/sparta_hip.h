@@ -116,6 +116,23 @@ int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
                             int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
                             void* workspace, size_t workspace_bytes, spx_stream_t stream);
 
+/* spx_bcs_index for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): no workspace argument.
+ * No counterpart in the reference.  The scratch of the two kernels lives in a device
+ * array inside the library, spx_bcs_index_static_max_bytes() = 1 MiB per GPU, held until
+ * the process ends; a mask whose workspace (spx_bcs_index_workspace_bytes) is larger is
+ * rejected with SPX_E_WORKSPACE before anything is launched (1 MiB covers about 190 000
+ * blocks, e.g. a 4096 x 4096 mask down to 16 x 8 blocks).  Nothing is allocated or
+ * freed by the call.  All calls on one GPU share that GPU's array: calls that overlap
+ * on one GPU (two streams, two threads) race and must be serialised by the caller.
+ * The first call on a device looks the array's address up (not a stream operation):
+ * make it outside graph capture.  Results are identical to spx_bcs_index. */
+size_t spx_bcs_index_static_max_bytes(void);
+int spx_bcs_index_static(const uint8_t* mask, int H, int W, int BH, int BW,
+                         int32_t* row_ptr, int32_t* bcsr_idx,
+                         int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                         int32_t* nnz_dev, int cap, spx_stream_t stream);
+
 /* Row / column sums of compressed values (fp32 accumulate), used for the bias
  * gradient of a compressed sparse-output matmul.  Replace
  * BCSFunctionContext.row_sum / col_sum (block_compressed.py:360-403) and

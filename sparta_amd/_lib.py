@@ -40,6 +40,8 @@ _SIGNATURES = {
     'spx_bcs_index_workspace_bytes': (_Z, [_I, _I, _I, _I]),
     'spx_bcs_index': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P, _Z, _P]),
     'spx_bcs_index_scheduled': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _Z, _P]),
+    'spx_bcs_index_static_max_bytes': (_Z, []),
+    'spx_bcs_index_static': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P]),
     'spx_bcs_gather': (_I, [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
     'spx_bcs_scatter': (_I, [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
     'spx_bcs_sum': (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _L, _P]),

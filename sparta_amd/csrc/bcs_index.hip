@@ -10,6 +10,7 @@
 // (sparta/tesa/templates/block_compressed.cu.j2:67-170) and the cumsum + .item()
 // glue of sparta/tesa/block_compressed.py:242-309.
 #include "common.hpp"
+#include <mutex>
 
 namespace spx {
 
@@ -522,6 +523,57 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
         hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
     SPX_LAUNCH_CHECK("emit_kernel");
     return 0;
+}
+
+// ---- index build without any allocation ---------------------------------------------
+// The workspace of spx_bcs_index lives in a file-scope device array instead of a
+// caller-provided buffer.  Every device the library runs on holds its own copy of the
+// array at its own address: the address is looked up once per device, with that device
+// current, and kept; host code never uses the array's name for anything else.
+namespace spx {
+constexpr size_t BCS_SCRATCH_BYTES = 1u << 20;
+constexpr int BCS_SCRATCH_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[BCS_SCRATCH_BYTES];
+static void* g_scratch_ptr[BCS_SCRATCH_MAX_DEVICES];
+static std::once_flag g_scratch_once[BCS_SCRATCH_MAX_DEVICES];
+static hipError_t g_scratch_err[BCS_SCRATCH_MAX_DEVICES];
+
+// Address of the current device's copy of `scratch`; NULL (and *err set) on failure.
+static void* scratch_of_current_device(hipError_t* err) {
+    int dev = -1;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= BCS_SCRATCH_MAX_DEVICES) { *err = hipErrorInvalidDevice; return nullptr; }
+    std::call_once(g_scratch_once[dev], [dev]() {
+        void* ptr = nullptr;
+        g_scratch_err[dev] = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        g_scratch_ptr[dev] = g_scratch_err[dev] == hipSuccess ? ptr : nullptr;
+    });
+    *err = g_scratch_err[dev];
+    return g_scratch_ptr[dev];
+}
+}  // namespace spx
+
+extern "C" size_t spx_bcs_index_static_max_bytes(void) { return spx::BCS_SCRATCH_BYTES; }
+
+extern "C" int spx_bcs_index_static(const uint8_t* mask, int H, int W, int BH, int BW,
+                                    int32_t* row_ptr, int32_t* bcsr_idx,
+                                    int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
+                                    int32_t* nnz_dev, int cap, spx_stream_t stream) {
+    using namespace spx;
+    int rc = check_index_shape(H, W, BH, BW);
+    if (rc) return rc;
+    const size_t need = index_workspace(H, W, BH, BW).total;
+    SPX_REQUIRE(need <= BCS_SCRATCH_BYTES, SPX_E_WORKSPACE,
+                "a (%d,%d) mask in (%d,%d) blocks needs %zu bytes of scratch, the static buffer holds %zu: "
+                "use spx_bcs_index with a caller-provided workspace", H, W, BH, BW, need, BCS_SCRATCH_BYTES);
+    hipError_t err = hipSuccess;
+    void* ptr = scratch_of_current_device(&err);
+    if (!ptr) return hip_fail(err, "hipGetSymbolAddress(scratch)");
+    // every byte of the workspace that the kernels read is written by them first, so the
+    // previous call's contents need no clearing
+    return bcs_index_impl(mask, H, W, BH, BW, row_ptr, bcsr_idx, col_ptr, bcsc_idx, bcsc_i64, nnz_dev, cap,
+                          nullptr, nullptr, ptr, BCS_SCRATCH_BYTES, stream);
 }
 
 extern "C" int spx_bcs_schedule(const int32_t* ptr, int n, int32_t* order, spx_stream_t stream) {
