@@ -121,8 +121,8 @@ int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
  * No counterpart in the reference.  The scratch of the two kernels lives in a device
  * array inside the library, spx_bcs_index_static_max_bytes() = 1 MiB per GPU, held until
  * the process ends; a mask whose workspace (spx_bcs_index_workspace_bytes) is larger is
- * rejected with SPX_E_WORKSPACE before anything is launched (1 MiB covers about 190 000
- * blocks, e.g. a 4096 x 4096 mask down to 16 x 8 blocks).  Nothing is allocated or
+ * rejected with SPX_E_WORKSPACE before anything is launched (1 MiB covers about 700 000
+ * blocks, e.g. a 4096 x 4096 mask down to 8 x 4 blocks).  Nothing is allocated or
  * freed by the call.  All calls on one GPU share that GPU's array: calls that overlap
  * on one GPU (two streams, two threads) race and must be serialised by the caller.
  * The first call on a device looks the array's address up (not a stream operation):

@@ -1,8 +1,11 @@
 // BCSR / BCSC index build for a uint8 element mask.
 //
-// Two launches, no host round trip, no atomics, canonical (sorted) order:
-//   1. liveness_kernel: streams the mask once with 16-byte loads and writes one
-//      byte per block ("any byte of the tile non-zero").  HBM-bound: H*W bytes in.
+// Two launches, no host round trip, no atomics, canonical (sorted) order.  Block grids
+// of at most 2048 row words and 2048 column words (a word = 64 blocks) take the pair
+// live_bits_kernel + emit_words_kernel described further down; larger grids and masks
+// whose rows cannot be read with 16-byte loads take the general pair:
+//   1. liveness_kernel: streams the mask once and writes one byte per block ("any byte
+//      of the tile non-zero").
 //   2. emit_kernel (one workgroup): turns the byte map into 64-block words with
 //      wavefront ballots, prefix-scans the word popcounts (which directly yields
 //      row_ptr / col_ptr and every block's rank), and writes the index arrays.
@@ -229,10 +232,94 @@ __global__ __launch_bounds__(1024) void emit_kernel(EmitParams p) {
     if (p.col_order) schedule_segments(p.col_ptr, p.Cn, p.col_order, s_bins);
 }
 
-// Fast path of the emit step for block grids of at most 2048 row words and 2048
-// column words: every thread owns two consecutive words, the prefix sums run in
-// registers + LDS, and only the final arrays touch global memory.
+// ---- fast path: block grids of at most 2048 row words and 2048 column words ----------
+// (a word = the liveness bits of 64 consecutive blocks of a block-row or block-column).
+// Two launches; at this size both are bound by launch and memory latency and by the
+// number of instructions a wavefront issues, not by bandwidth, so the layout of the work
+// is chosen to keep every dependent chain short:
+//   live_bits_kernel   one workgroup per (row word, group of mask rows): ORs the 64 x BW
+//                      bytes of each of its mask rows (16-byte loads, all independent)
+//                      and writes the 64 liveness bits as one 8-byte partial word (very
+//                      small grids split the BH mask rows of a block-row over up to eight
+//                      workgroups, whose partial words the second kernel ORs together).
+//   emit_words_kernel  one group of workgroups per requested format (BCSR side, BCSC
+//                      side), each split into `nslice` slices.  Every workgroup loads all
+//                      row words (<= 16 KB, one coalesced load per thread), prefix-sums
+//                      their popcounts in LDS and - on the BCSC side - transposes them into
+//                      column words 64 x 64 bits at a time with a six-step lane butterfly
+//                      (one wavefront per tile).  It then writes only its slice of the index
+//                      entries, one word per wavefront instruction (lane = bit, rank = word
+//                      base + popcount of the lower bits), so a dense mask still stores 64
+//                      entries per instruction.  Slice 0 of a side writes the pointer array
+//                      and nnz, the last slice the launch order.
 constexpr int EMIT_FAST_WORDS = 2048;
+
+struct BitsParams {
+    const uint8_t* mask;
+    unsigned long long* pbits;  // [Q][R * WPR] partial words, one per group of mask rows
+    int W, BH, BW, WPR, NW;
+    int log_bw;
+    int rows_per_part;          // mask rows of a block-row that one workgroup covers (BH / Q)
+};
+
+__global__ __launch_bounds__(256) void live_bits_kernel(BitsParams p) {
+    __shared__ uint32_t flags[64];
+    const int tid = threadIdx.x;
+    if (tid < 64) flags[tid] = 0;
+    __syncthreads();
+    const int wi = blockIdx.x, r = blockIdx.y, part = blockIdx.z;
+    const int64_t col0 = (int64_t)wi * 64 * p.BW;            // first mask column of the word
+    const int64_t left = p.W - col0;
+    const int nch = (int)((left < 64 * p.BW ? left : 64 * p.BW) >> 4);  // 16-byte chunks per mask row
+    const uint8_t* base = p.mask + ((int64_t)r * p.BH + (int64_t)part * p.rows_per_part) * p.W + col0;
+    const int log_nch = p.log_bw + 2;                         // log2 of the chunks of a full word
+    const int nrows = p.rows_per_part;
+
+    auto mark = [&](int chunk, uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3) {
+        if (p.BW >= 16) {
+            if (a0 | a1 | a2 | a3) flags[(chunk << 4) >> p.log_bw] = 1;
+        } else if (p.BW == 8) {
+            if (a0 | a1) flags[chunk * 2] = 1;
+            if (a2 | a3) flags[chunk * 2 + 1] = 1;
+        } else {  // BW == 4
+            if (a0) flags[chunk * 4] = 1;
+            if (a1) flags[chunk * 4 + 1] = 1;
+            if (a2) flags[chunk * 4 + 2] = 1;
+            if (a3) flags[chunk * 4 + 3] = 1;
+        }
+    };
+    if (log_nch <= 8) {
+        // a thread keeps one chunk column and walks the mask rows 256 >> log_nch apart
+        const int chunk = tid & ((1 << log_nch) - 1);
+        const int rstep = 256 >> log_nch;
+        if (chunk < nch) {
+            uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+            const uint8_t* src = base + (int64_t)chunk * 16;
+#pragma unroll 8
+            for (int row = tid >> log_nch; row < nrows; row += rstep) {
+                const vec16 v = *reinterpret_cast<const vec16*>(src + (int64_t)row * p.W);
+                a0 |= v.x; a1 |= v.y; a2 |= v.z; a3 |= v.w;
+            }
+            mark(chunk, a0, a1, a2, a3);
+        }
+    } else {
+        for (int chunk = tid; chunk < nch; chunk += 256) {
+            uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+            const uint8_t* src = base + (int64_t)chunk * 16;
+#pragma unroll 8
+            for (int row = 0; row < nrows; ++row) {
+                const vec16 v = *reinterpret_cast<const vec16*>(src + (int64_t)row * p.W);
+                a0 |= v.x; a1 |= v.y; a2 |= v.z; a3 |= v.w;
+            }
+            mark(chunk, a0, a1, a2, a3);
+        }
+    }
+    __syncthreads();
+    if (tid < 64) {
+        const unsigned long long word = __ballot(flags[tid] != 0);
+        if (tid == 0) p.pbits[(int64_t)part * p.NW + (int64_t)r * p.WPR + wi] = word;
+    }
+}
 
 __device__ __forceinline__ int block_exclusive_scan_1024(int v, int* lds, int* total) {
     const int lane = lane_id();
@@ -252,134 +339,160 @@ __device__ __forceinline__ int block_exclusive_scan_1024(int v, int* lds, int* t
     return before + inc - v;
 }
 
-__global__ __launch_bounds__(1024) void emit_fast_kernel(EmitParams p) {
-    __shared__ unsigned long long s_bits[EMIT_FAST_WORDS];
-    __shared__ int s_base[EMIT_FAST_WORDS];
+// Launch order of n segments whose lengths are base[(i + 1) * stride] - base[i * stride]
+// (base in LDS, `total` closing the last one): descending length, bucketed at 255.
+// Segments of equal length come out in the order their lanes reach the LDS counter:
+// any order of them is as good for scheduling, the result only has to be a permutation.
+__device__ void schedule_from_lds(const int* base, int stride, int n, int total, int32_t* order, int* bins) {
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) bins[i] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int c = (i + 1 < n ? base[(i + 1) * stride] : total) - base[i * stride];
+        atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        int carry = 0;
+        for (int b0 = 0; b0 < 256; b0 += 64) {
+            const int v = bins[b0 + threadIdx.x];
+            const int inc = wave_inclusive_scan(v);
+            bins[b0 + threadIdx.x] = carry + inc - v;
+            carry += __shfl(inc, 63, 64);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int c = (i + 1 < n ? base[(i + 1) * stride] : total) - base[i * stride];
+        order[atomicAdd(&bins[255 - (c < 255 ? c : 255)], 1)] = i;
+    }
+}
+
+__device__ __forceinline__ unsigned long long shfl_xor_u64(unsigned long long x, int j) {
+    const int lo = __shfl_xor((int)(unsigned)x, j, 64);
+    const int hi = __shfl_xor((int)(unsigned)(x >> 32), j, 64);
+    return ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo;
+}
+
+// 64 x 64 bit-matrix transpose over a wavefront: lane i holds row i on entry and column i
+// on exit (bit b of the result of lane i = bit i of the input of lane b).  Six butterfly
+// steps: lanes i and i ^ j exchange the off-diagonal j x j blocks.
+__device__ __forceinline__ unsigned long long transpose_bits_64x64(unsigned long long x, int lane) {
+    unsigned long long m = 0x00000000FFFFFFFFull;
+#pragma unroll
+    for (int j = 32; j >= 1; j >>= 1) {
+        const unsigned long long y = shfl_xor_u64(x, j);
+        x = (lane & j) ? ((x & ~m) | ((y & ~m) >> j)) : ((x & m) | ((y & m) << j));
+        m ^= m << (j >> 1);
+    }
+    return x;
+}
+
+__global__ __launch_bounds__(1024) void emit_words_kernel(EmitParams p, int nslice, int sides, int nparts) {
+    __shared__ unsigned long long s_bits[EMIT_FAST_WORDS];   // row words
+    __shared__ int s_base[EMIT_FAST_WORDS];                  // exclusive prefix of their popcounts
+    __shared__ unsigned long long s_cbits[EMIT_FAST_WORDS];  // column words
+    __shared__ int s_cbase[EMIT_FAST_WORDS];
     __shared__ int s_scan[16];
     __shared__ int s_bins[256];
     const int tid = threadIdx.x;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int side = sides == 3 ? (int)blockIdx.x / nslice : (sides == 2 ? 1 : 0);  // 0 BCSR, 1 BCSC
+    const int slice = (int)blockIdx.x % nslice;
 
     // ---- row words: word g = r * WPR + wi covers columns wi*64 .. wi*64+63 of row r ----
     const int NW = p.R * p.WPR;
-    unsigned long long w[2];
-    int cnt[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int g = tid * 2 + i;
-        unsigned long long word = 0;
-        if (g < NW) {
-            const int r = g / p.WPR;
-            const int c0 = (g - r * p.WPR) * 64;
-            const uint8_t* src = p.live + (int64_t)r * p.Cn + c0;
-            const int n = p.Cn - c0 < 64 ? p.Cn - c0 : 64;
-            if ((p.Cn & 7) == 0) {
-                // liveness bytes are 0 or 1: one multiply gathers the low bit of 8 bytes
-                const unsigned long long* src8 = reinterpret_cast<const unsigned long long*>(src);
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    if (k * 8 < n) {
-                        const unsigned long long x = src8[k];
-                        word |= ((x * 0x0102040810204080ULL) >> 56) << (k * 8);
-                    }
-                }
+    unsigned long long w0 = 0, w1 = 0;  // OR of the partial words of the row groups
+    if (tid * 2 < NW) {
+        const bool pair = tid * 2 + 1 < NW && (NW & 1) == 0;  // 16-byte loads need an even pitch
+        for (int q = 0; q < nparts; ++q) {
+            const unsigned long long* src = p.wbits + (int64_t)q * NW + tid * 2;
+            if (pair) {
+                const ulonglong2 v = *reinterpret_cast<const ulonglong2*>(src);
+                w0 |= v.x; w1 |= v.y;
             } else {
-#pragma unroll 8
-                for (int k = 0; k < n; ++k) word |= (unsigned long long)(src[k] != 0) << k;
+                w0 |= src[0];
+                if (tid * 2 + 1 < NW) w1 |= src[1];
             }
         }
-        w[i] = word;
-        cnt[i] = __popcll(word);
     }
+    const int c0 = __popcll(w0), c1 = __popcll(w1);
     int nnz;
-    const int tbase = block_exclusive_scan_1024(cnt[0] + cnt[1], s_scan, &nnz);
-    int base[2] = {tbase, tbase + cnt[0]};
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int g = tid * 2 + i;
-        if (g < EMIT_FAST_WORDS) { s_bits[g] = w[i]; s_base[g] = base[i]; }
-        if (g < NW) {
-            const int r = g / p.WPR;
-            const int wi = g - r * p.WPR;
-            if (p.row_ptr && wi == 0) p.row_ptr[r] = base[i];
-            if (p.bcsr_idx) {
-                unsigned long long bits = w[i];
-                int pos = base[i];
-                while (bits) {
-                    const int c = __ffsll((long long)bits) - 1;
-                    bits &= bits - 1;
-                    if (pos < p.cap) p.bcsr_idx[pos] = (r << 16) | (wi * 64 + c);
-                    ++pos;
-                }
+    const int tbase = block_exclusive_scan_1024(c0 + c1, s_scan, &nnz);
+    s_bits[tid * 2] = w0;
+    s_bits[tid * 2 + 1] = w1;
+    s_base[tid * 2] = tbase;
+    s_base[tid * 2 + 1] = tbase + c0;
+    __syncthreads();
+
+    if (side == 0) {
+        if (slice == 0) {
+            if (tid == 0) {
+                p.nnz_dev[0] = nnz;
+                p.row_ptr[p.R] = nnz;
+            }
+            for (int r = tid; r < p.R; r += 1024) p.row_ptr[r] = s_base[r * p.WPR];
+        }
+        for (int g = slice * 16 + wave; g < NW; g += 16 * nslice) {
+            const unsigned long long bits = s_bits[g];
+            if ((bits >> lane) & 1ull) {
+                const int pos = s_base[g] + __popcll(bits & lt_mask);
+                const int r = g / p.WPR;
+                if (pos < p.cap) p.bcsr_idx[pos] = (r << 16) | ((g - r * p.WPR) * 64 + lane);
             }
         }
+        if (slice == nslice - 1 && p.row_order) schedule_from_lds(s_base, p.WPR, p.R, nnz, p.row_order, s_bins);
+        return;
     }
-    if (tid == 0) {
-        p.nnz_dev[0] = nnz;
-        if (p.row_ptr) p.row_ptr[p.R] = nnz;
-    }
-    if (p.row_order && p.row_ptr) schedule_segments(p.row_ptr, p.R, p.row_order, s_bins);
-    if (!p.col_ptr) return;
-    __syncthreads();  // s_bits / s_base complete
 
     // ---- column words: word g = c * WPC + ri covers rows ri*64 .. ri*64+63 of column c ----
     const int NWC = p.Cn * p.WPC;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int g = tid * 2 + i;
-        unsigned long long word = 0;
-        if (g < NWC) {
-            const int c = g / p.WPC;
-            const int r0 = (g - c * p.WPC) * 64;
-            const int n = p.R - r0 < 64 ? p.R - r0 : 64;
-            // bit (r, c) comes from the row words already in LDS
-            const int wi = c >> 6, cb = c & 63;
-            const unsigned long long* col = s_bits + r0 * p.WPR + wi;
-            if (n == 64) {
-#pragma unroll 16
-                for (int k = 0; k < 64; ++k) word |= ((col[k * p.WPR] >> cb) & 1ull) << k;
-            } else {
-                for (int k = 0; k < n; ++k) word |= ((col[k * p.WPR] >> cb) & 1ull) << k;
-            }
-        }
-        w[i] = word;
-        cnt[i] = __popcll(word);
+    s_cbits[tid * 2] = 0;
+    s_cbits[tid * 2 + 1] = 0;
+    __syncthreads();
+    for (int tile = wave; tile < p.WPR * p.WPC; tile += 16) {  // tile = (ri, wi): 64 rows x 64 columns
+        const int ri = tile / p.WPR, wi = tile - ri * p.WPR;
+        const int r = ri * 64 + lane;
+        const unsigned long long rows = r < p.R ? s_bits[r * p.WPR + wi] : 0ull;
+        const unsigned long long col = transpose_bits_64x64(rows, lane);
+        const int c = wi * 64 + lane;
+        if (c < p.Cn) s_cbits[c * p.WPC + ri] = col;
     }
+    __syncthreads();
+    const unsigned long long cw0 = s_cbits[tid * 2], cw1 = s_cbits[tid * 2 + 1];
     int nnz2;
-    const int cbase = block_exclusive_scan_1024(cnt[0] + cnt[1], s_scan, &nnz2);
-    base[0] = cbase;
-    base[1] = cbase + cnt[0];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int g = tid * 2 + i;
-        if (g < NWC) {
-            const int c = g / p.WPC;
-            const int ri = g - c * p.WPC;
-            if (ri == 0) p.col_ptr[c] = base[i];
-            if (p.bcsc_idx) {
-                unsigned long long bits = w[i];
-                int pos = base[i];
-                const int wi = c >> 6, cb = c & 63;
-                while (bits) {
-                    const int k = __ffsll((long long)bits) - 1;
-                    bits &= bits - 1;
-                    const int r = ri * 64 + k;
-                    if (pos < p.cap) {
-                        if (p.bcsc_i64) {
-                            const int gw = r * p.WPR + wi;
-                            const unsigned long long below = cb == 0 ? 0ull : (s_bits[gw] & (~0ull >> (64 - cb)));
-                            const long long bpos = s_base[gw] + __popcll(below);
-                            reinterpret_cast<long long*>(p.bcsc_idx)[pos] = (bpos << 32) | ((long long)c << 16) | (long long)r;
-                        } else {
-                            reinterpret_cast<int32_t*>(p.bcsc_idx)[pos] = (c << 16) | r;
-                        }
-                    }
-                    ++pos;
+    const int cb = block_exclusive_scan_1024(__popcll(cw0) + __popcll(cw1), s_scan, &nnz2);
+    s_cbase[tid * 2] = cb;
+    s_cbase[tid * 2 + 1] = cb + __popcll(cw0);
+    __syncthreads();
+    if (slice == 0) {
+        if (tid == 0) {
+            p.col_ptr[p.Cn] = nnz2;
+            if (sides == 2) p.nnz_dev[0] = nnz2;  // no BCSR side in this launch
+        }
+        for (int c = tid; c < p.Cn; c += 1024) p.col_ptr[c] = s_cbase[c * p.WPC];
+    }
+    for (int g = slice * 16 + wave; g < NWC; g += 16 * nslice) {
+        const unsigned long long bits = s_cbits[g];
+        if ((bits >> lane) & 1ull) {
+            const int pos = s_cbase[g] + __popcll(bits & lt_mask);
+            if (pos < p.cap) {
+                const int c = g / p.WPC;
+                const int r = (g - c * p.WPC) * 64 + lane;
+                if (p.bcsc_i64) {
+                    const int gw = r * p.WPR + (c >> 6);
+                    const int cl = c & 63;
+                    const unsigned long long below = cl == 0 ? 0ull : (s_bits[gw] & (~0ull >> (64 - cl)));
+                    const long long bpos = s_base[gw] + __popcll(below);
+                    reinterpret_cast<long long*>(p.bcsc_idx)[pos] = (bpos << 32) | ((long long)c << 16) | (long long)r;
+                } else {
+                    reinterpret_cast<int32_t*>(p.bcsc_idx)[pos] = (c << 16) | r;
                 }
             }
         }
     }
-    if (tid == 0) p.col_ptr[p.Cn] = nnz2;
-    if (p.col_order) schedule_segments(p.col_ptr, p.Cn, p.col_order, s_bins);
+    if (slice == nslice - 1 && p.col_order) schedule_from_lds(s_cbase, p.WPC, p.Cn, nnz2, p.col_order, s_bins);
 }
 
 __global__ __launch_bounds__(1024) void schedule_kernel(const int32_t* ptr, int n, int32_t* order) {
@@ -388,7 +501,7 @@ __global__ __launch_bounds__(1024) void schedule_kernel(const int32_t* ptr, int 
 }
 
 struct IndexWorkspace {
-    size_t live_off, wbits_off, wbase_off, cbase_off, total;
+    size_t live_off, wbits_off, wbase_off, cbase_off, pbits_off, total;
     int R, Cn, WPR, WPC;
 };
 
@@ -403,6 +516,9 @@ static IndexWorkspace index_workspace(int H, int W, int BH, int BW) {
     w.wbits_off = off; off += round_up((size_t)w.R * w.WPR * 8, 256);
     w.wbase_off = off; off += round_up((size_t)w.R * w.WPR * 4, 256);
     w.cbase_off = off; off += round_up((size_t)w.Cn * w.WPC * 4, 256);
+    // partial words of the fast path: up to 8 row groups of at most EMIT_FAST_WORDS words
+    const size_t nw = (size_t)w.R * w.WPR;
+    w.pbits_off = off; off += round_up((nw < 2048 ? nw : 2048) * 8 * 8, 256);
     w.total = off;
     return w;
 }
@@ -478,10 +594,45 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
     char* wsb = reinterpret_cast<char*>(workspace);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
+    EmitParams ep;
+    ep.live = reinterpret_cast<uint8_t*>(wsb + ws.live_off);
+    ep.wbits = reinterpret_cast<unsigned long long*>(wsb + ws.wbits_off);
+    ep.wbase = reinterpret_cast<int*>(wsb + ws.wbase_off);
+    ep.cbase = reinterpret_cast<int*>(wsb + ws.cbase_off);
+    ep.row_ptr = row_ptr; ep.bcsr_idx = bcsr_idx;
+    ep.col_ptr = col_ptr; ep.bcsc_idx = bcsc_idx; ep.bcsc_i64 = bcsc_i64;
+    ep.nnz_dev = nnz_dev; ep.cap = cap;
+    ep.R = ws.R; ep.Cn = ws.Cn; ep.WPR = ws.WPR; ep.WPC = ws.WPC;
+    ep.row_order = row_order; ep.col_order = col_order;
+
     // Widest load the mask's address and row pitch allow.
     int vec = 1;
     if (W % 16 == 0 && aligned(mask, 16)) vec = 16;
     else if (W % 4 == 0 && aligned(mask, 4)) vec = 4;
+
+    if (vec == 16 && ws.R * ws.WPR <= EMIT_FAST_WORDS && ws.Cn * ws.WPC <= EMIT_FAST_WORDS) {
+        // row groups: a power of two, at most 8, at least 4 mask rows each.  Measured on
+        // 3072 x 768 and 4096 x 4096 masks, one workgroup per word is as fast as eight, so
+        // the split only serves grids of fewer than 64 words
+        int nparts = 1;
+        while (nparts < 8 && BH / (nparts * 2) >= 4 && ws.R * ws.WPR * nparts < 64) nparts *= 2;
+        BitsParams bp;
+        bp.mask = mask;
+        bp.pbits = reinterpret_cast<unsigned long long*>(wsb + ws.pbits_off);
+        bp.W = W; bp.BH = BH; bp.BW = BW; bp.WPR = ws.WPR; bp.NW = ws.R * ws.WPR;
+        bp.log_bw = ilog2(BW);
+        bp.rows_per_part = BH / nparts;
+        ep.wbits = bp.pbits;
+        hipLaunchKernelGGL(live_bits_kernel, dim3(ws.WPR, ws.R, nparts), dim3(256), 0, st, bp);
+        SPX_LAUNCH_CHECK("live_bits_kernel");
+        const int sides = (row_ptr ? 1 : 0) | (col_ptr ? 2 : 0);
+        // enough slices that a slice writes at most ~2048 index entries
+        int nslice = (ws.R * ws.Cn + 2047) / 2048;
+        nslice = nslice < 1 ? 1 : (nslice > 8 ? 8 : nslice);
+        hipLaunchKernelGGL(emit_words_kernel, dim3(nslice * (sides == 3 ? 2 : 1)), dim3(1024), 0, st, ep, nslice, sides, nparts);
+        SPX_LAUNCH_CHECK("emit_words_kernel");
+        return 0;
+    }
 
     // Segment width: at most 256 threads * vec bytes, at least one block wide;
     // narrowed while that buys more workgroups (the launch wants >> 256 of them).
@@ -506,21 +657,7 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
     else if (vec == 4) hipLaunchKernelGGL(liveness_kernel<4>, grid, dim3(256), 0, st, lp);
     else hipLaunchKernelGGL(liveness_kernel<1>, grid, dim3(256), 0, st, lp);
     SPX_LAUNCH_CHECK("liveness_kernel");
-
-    EmitParams ep;
-    ep.live = lp.live;
-    ep.wbits = reinterpret_cast<unsigned long long*>(wsb + ws.wbits_off);
-    ep.wbase = reinterpret_cast<int*>(wsb + ws.wbase_off);
-    ep.cbase = reinterpret_cast<int*>(wsb + ws.cbase_off);
-    ep.row_ptr = row_ptr; ep.bcsr_idx = bcsr_idx;
-    ep.col_ptr = col_ptr; ep.bcsc_idx = bcsc_idx; ep.bcsc_i64 = bcsc_i64;
-    ep.nnz_dev = nnz_dev; ep.cap = cap;
-    ep.R = ws.R; ep.Cn = ws.Cn; ep.WPR = ws.WPR; ep.WPC = ws.WPC;
-    ep.row_order = row_order; ep.col_order = col_order;
-    if (ws.R * ws.WPR <= EMIT_FAST_WORDS && ws.Cn * ws.WPC <= EMIT_FAST_WORDS)
-        hipLaunchKernelGGL(emit_fast_kernel, dim3(1), dim3(1024), 0, st, ep);
-    else
-        hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
+    hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
     SPX_LAUNCH_CHECK("emit_kernel");
     return 0;
 }

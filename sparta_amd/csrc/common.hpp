@@ -78,14 +78,19 @@ template <> struct Elem<bf16_t> {
     __device__ static bf16_t from_float(float v) { bf16_t r; r.v = float_to_bf16(v); return r; }
 };
 
-// Inclusive prefix sum across the 64 lanes of a wavefront.
+// Inclusive prefix sum across the 64 lanes of a wavefront: six data-parallel steps on
+// the VALU (shifts by 1, 2, 4, 8 inside each row of 16 lanes, then lane 15 of a row
+// broadcast into the next row, then lane 31 into the upper half), no LDS traffic.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ int dpp_shift_or_zero(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
-    const int lane = lane_id();
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        int t = __shfl_up(v, d, 64);
-        if (lane >= d) v += t;
-    }
+    v += dpp_shift_or_zero<0x111, 0xf>(v);  // row_shr:1
+    v += dpp_shift_or_zero<0x112, 0xf>(v);  // row_shr:2
+    v += dpp_shift_or_zero<0x114, 0xf>(v);  // row_shr:4
+    v += dpp_shift_or_zero<0x118, 0xf>(v);  // row_shr:8
+    v += dpp_shift_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v += dpp_shift_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
     return v;
 }
 // Reductions over each aligned group of 16 lanes (a DPP "row"): four data-parallel
