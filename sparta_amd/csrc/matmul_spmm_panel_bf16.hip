@@ -1,5 +1,5 @@
-// bf16 instantiations of the panel sparse-operand matmul kernel.
-#include "matmul_spmm_panel.hpp"
+// bf16 instantiations of the panel sparse-operand matmul kernels (one workgroup per tile, and persistent).
+#include "matmul_spmm_stream.hpp"
 namespace spx {
 template <>
 int launch_spmm_panel<bf16_t>(const SpmmParams& p, int BN, int batch, int nst, hipStream_t st) {
@@ -10,5 +10,10 @@ int launch_spmm_panel<bf16_t>(const SpmmParams& p, int BN, int batch, int nst, h
         return launch_spmm_panel_impl<bf16_t, 2, true>(p, BN, batch, st);
     }
     return launch_spmm_panel_impl<bf16_t, 2, false>(p, BN, batch, st);
+}
+template <>
+int launch_spmm_stream<bf16_t>(const SpmmParams& p, int BN, int batch, hipStream_t st) {
+    if (!spmm_stream_supported<bf16_t>(p, BN)) return fail(SPX_E_CONFIG, "the persistent panel kernel needs a k-contiguous dense operand and 64-byte block rows");
+    return launch_spmm_stream_impl<bf16_t>(p, BN, batch, st);
 }
 }  // namespace spx

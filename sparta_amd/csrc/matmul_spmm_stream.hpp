@@ -1,0 +1,350 @@
+// Sparse-operand matmul, persistent variant of the panel kernel (matmul_spmm_panel.hpp)
+// for a k-contiguous dense operand with many 256-row tiles: out[m,n] = sum_k D[m,k] S[k,n].
+//
+// The panel kernel launches one workgroup per (256-row tile, block-column).  Every such
+// workgroup pays a chain of dependent loads before its first MFMA (launch order -> column
+// pointer -> index entries -> first blocks of D) and an epilogue during which it loads
+// nothing, and the workgroups of a launch generation go through these phases together,
+// so HBM, the L2 -> L1 gathers and the stores take turns instead of overlapping.  Here a
+// workgroup is a slot that stays: slot (xcd, pos) walks the tiles (m-tile 8 g + xcd,
+// block-column order[g odd ? nb-1-pos : pos]) for g = 0, 1, ... as ONE stream of steps.
+// The index entries of tile g+1 are fetched while tile g runs, the loads of its first two
+// steps are issued during the last two steps of tile g, and the stores of tile g are in
+// flight while tile g+1 gathers.  Alternating the walk direction over the launch order
+// (longest block-column first) pairs long columns with short ones, so the slots of an XCD
+// finish together.  All m-tiles of one XCD share its L2, as in the panel kernel.
+//
+// Step, LDS layout, fragment mapping and epilogue are those of the panel kernel with the
+// sparse block shared by the four wavefronts (one barrier per step).
+#pragma once
+#include "matmul_spmm_panel.hpp"
+
+namespace spx {
+
+template <typename T, int BN, int BK, bool SWAP>
+__global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(SpmmParams p, int n_mtiles) {
+    typedef typename PanelMma<T>::M MMA;
+    typedef typename MMA::frag Frag;
+    constexpr int KC = PanelMma<T>::KC;
+    constexpr int CH = BK / KC;          // steps per block
+    constexpr int NT = BN / 16;
+    constexpr int ROWS = 80;             // private LDS rows (64 bytes each) per wave
+    constexpr int SH_BYTES = 2 * BN * 64;  // shared, double-buffered S tile
+    constexpr int E16 = 16 / (int)sizeof(T);
+    static_assert(BK % KC == 0, "block depth must be a multiple of the step");
+
+    __shared__ __align__(16) char lds_all[4 * ROWS * 64 + SH_BYTES];
+
+    const int nb = p.Nc / BN;
+    const int xcd = (int)blockIdx.x % kPanelXcd;
+    const int pos = (int)blockIdx.x / kPanelXcd;  // [0, nb)
+    if (xcd >= n_mtiles) return;
+    const int n_tiles = (n_mtiles - xcd + kPanelXcd - 1) / kPanelXcd;
+    const int64_t b = blockIdx.y;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15;
+    const int g4 = lane >> 4;
+    char* lds = lds_all + wave * (ROWS * 64);
+    char* wsh = lds_all + 4 * ROWS * 64;
+
+    const T* D = reinterpret_cast<const T*>(p.D) + b * p.d_batch;
+    const T* S = reinterpret_cast<const T*>(p.S) + b * p.s_batch;
+
+    // coalesced load mapping: lane -> (row within a 16-row group, 16-byte chunk).  Element
+    // offsets from the first row of a tile fit 32 bits (checked on the host); the last
+    // m-tile may be partial: its rows past the end re-read the last row and are never stored.
+    const int lrow = lane >> 2;
+    const int lchk = lane & 3;
+    const int last_rows = p.Mc - (n_mtiles - 1) * 256;  // rows of the last m-tile (1..256)
+    int roff[4];  // byte offset of this lane's chunk from the start of a tile's first row
+    int wofs[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int row = wave * 64 + q * 16 + lrow;
+        roff[q] = (row * (int)p.d_ld + lchk * E16) * (int)sizeof(T);
+        const int lr = q * 16 + lrow;
+        wofs[q] = lr * 64 + ((lchk ^ ((lr >> 2) & 3)) << 4);
+    }
+    // shared S tile: this wave stages chunks wave*BN .. wave*BN+BN-1 of the BN*4 chunks
+    // (k-contiguous S: chunk = (n row, 16-byte piece of its 64 bytes of k); otherwise a chunk
+    // is 16 bytes of n at one k and is transposed on its way into LDS)
+    const int sh_chunk = wave * BN + lane;
+    const int sh_row = sh_chunk >> 2, sh_chk = sh_chunk & 3;
+    const bool sh_active = lane < BN;
+    const int sh_k = sh_chunk / (BN / E16), sh_n0 = (sh_chunk % (BN / E16)) * E16;
+    const int sofs = sh_row * 64 + ((sh_chk ^ ((sh_row >> 2) & 3)) << 4);
+    int aofs[4], bofs[NT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = i * 16 + r16;
+        aofs[i] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int row = t * 16 + r16;
+        bofs[t] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
+    }
+    const int64_t sld = p.compressed ? (p.s_kcontig ? BK : BN) : p.s_ld;
+    const int64_t sh_toff = p.s_kcontig ? (int64_t)sh_row * sld + sh_chk * E16 : (int64_t)sh_k * sld + sh_n0;
+
+    // ---- per-tile state: the tile being computed and the one after it -------------------
+    struct Tile {
+        int mt, j, e_begin, n_it;   // uniform
+        int kb_vec, slot_vec;       // lane l: k-block and value slot of index entry l (first 64)
+    };
+    auto load_tile = [&](int g, Tile& t) {
+        t.mt = g * kPanelXcd + xcd;
+        const int o = (g & 1) ? nb - 1 - pos : pos;
+        t.j = p.sched ? p.sched[o] : o;
+        t.e_begin = p.ptr[t.j];
+        const int n_blk = p.ptr[t.j + 1] - t.e_begin;
+        t.n_it = n_blk * CH;
+        t.kb_vec = 0;
+        t.slot_vec = 0;
+        if (lane < n_blk) {
+            if (p.idx_kind == SPX_IDX_BCSC_I64) {
+                const long long v = reinterpret_cast<const long long*>(p.idx)[t.e_begin + lane];
+                t.kb_vec = (int)(v & 0xffff);
+                t.slot_vec = (int)(v >> 32);
+            } else {
+                t.kb_vec = reinterpret_cast<const int32_t*>(p.idx)[t.e_begin + lane] & 0xffff;
+                t.slot_vec = t.e_begin + lane;
+            }
+        }
+    };
+    Tile cur, nxt;
+    load_tile(0, cur);
+    if (n_tiles > 1) load_tile(1, nxt); else nxt = cur;
+
+    // Loads of one step of tile t into a stage (dreg: 4 x 16 bytes of D per lane, sreg: this
+    // lane's piece of the shared S block).  A step past the end (live == false) loads one
+    // fixed line per instruction and is never accumulated: the number of loads in flight is
+    // the same on every path, so each wait covers only the oldest stage.
+    auto issue = [&](const Tile& t, int it, bool live, u32x4 (&dreg)[4], u32x4& sreg) {
+        const int er = it / CH;
+        const int ch = it % CH;
+        int kb;
+        int64_t slot;
+        if (er < 64) {
+            kb = __builtin_amdgcn_readlane(t.kb_vec, er);
+            slot = __builtin_amdgcn_readlane(t.slot_vec, er);
+        } else if (p.idx_kind == SPX_IDX_BCSC_I64) {
+            const long long v = reinterpret_cast<const long long*>(p.idx)[t.e_begin + er];
+            kb = (int)(v & 0xffff);
+            slot = v >> 32;
+        } else {
+            kb = reinterpret_cast<const int32_t*>(p.idx)[t.e_begin + er] & 0xffff;
+            slot = t.e_begin + er;
+        }
+        const int koff = kb * BK + ch * KC;
+        // buffer loads: the tile's first row is the (scalar) base, the k offset a scalar
+        // offset and the lane's place in the tile a 32-bit register - no 64-bit address
+        // arithmetic per load.  A step that is not live reads the tile's first bytes.
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T*>(D + (int64_t)(live ? t.mt : 0) * 256 * p.d_ld), 0, 0x7fffffff, 0x00020000);
+        const int soff = live ? koff * (int)sizeof(T) : 0;
+        if (live && t.mt == n_mtiles - 1 && last_rows < 256) {
+            // partial last m-tile: rows past the end re-read its last row
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int row = wave * 64 + q * 16 + lrow;
+                const int voff = ((row < last_rows ? row : last_rows - 1) * (int)p.d_ld + lchk * E16) * (int)sizeof(T);
+                dreg[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dreg[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? roff[q] : 0, soff, 0);
+        }
+        const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN) + (p.s_kcontig ? ch * KC : ch * KC * BN)
+                                     : (p.s_kcontig ? S + (int64_t)t.j * BN * p.s_ld + koff
+                                                    : S + (int64_t)koff * p.s_ld + (int64_t)t.j * BN);
+        if (sh_active) sreg = *reinterpret_cast<const u32x4*>(live ? sblk + sh_toff : S);
+    };
+
+    f32x4 acc[4][NT];
+    u32x4 d0[4], d1[4], s0, s1;
+    s0 = s1 = u32x4{0u, 0u, 0u, 0u};
+
+    // One step: stage -> LDS, refill the stage with the step two ahead (which may belong to
+    // the next tile), barrier for the shared S tile, MFMAs.
+    auto step = [&](int it, int n_pad, bool have_next, u32x4 (&dreg)[4], u32x4& sreg) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(lds + wofs[q]) = dreg[q];
+        char* sdst = wsh + (it & 1) * (BN * 64);
+        if (sh_active) {
+            if (p.s_kcontig) {
+                *reinterpret_cast<u32x4*>(sdst + sofs) = sreg;
+            } else {
+                union { u32x4 v4; T e[E16]; } u;
+                u.v4 = sreg;
+#pragma unroll
+                for (int i = 0; i < E16; ++i) {
+                    const int n = sh_n0 + i;
+                    *reinterpret_cast<T*>(sdst + n * 64 + (((sh_k / E16) ^ ((n >> 2) & 3)) << 4) +
+                                          (sh_k % E16) * (int)sizeof(T)) = u.e[i];
+                }
+            }
+        }
+        {
+            const int ahead = it + 2;
+            if (ahead < n_pad) {
+                const bool live = ahead < cur.n_it;
+                issue(cur, live ? ahead : 0, live, dreg, sreg);
+            } else {
+                const int nit = ahead - n_pad;
+                const bool live = have_next && nit < nxt.n_it;
+                issue(nxt, live ? nit : 0, live, dreg, sreg);
+            }
+        }
+        __syncthreads();  // the S tile of this step is complete
+        if (it < cur.n_it) {
+            Frag af[4], bf[NT];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const Frag*>(lds + aofs[i]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) bf[t] = *reinterpret_cast<const Frag*>(sdst + bofs[t]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    acc[i][t] = SWAP ? MMA::mma(bf[t], af[i], acc[i][t]) : MMA::mma(af[i], bf[t], acc[i][t]);
+        }
+    };
+
+    issue(cur, 0, 0 < cur.n_it, d0, s0);
+    issue(cur, cur.n_it > 1 ? 1 : 0, 1 < cur.n_it, d1, s1);
+
+    const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
+    T* out = reinterpret_cast<T*>(p.out) + b * p.o_batch;
+    T* eT = reinterpret_cast<T*>(lds);
+
+    for (int g = 0; g < n_tiles; ++g) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[i][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // every tile runs an even number of steps, at least two (the surplus ones are idle),
+        // so that the stage a step uses is fixed by its position in its tile
+        const int n_pad = cur.n_it < 2 ? 2 : (cur.n_it + 1) & ~1;
+        const bool have_next = g + 1 < n_tiles;
+        for (int it = 0; it < n_pad; it += 2) {
+            step(it, n_pad, have_next, d0, s0);
+            step(it + 1, n_pad, have_next, d1, s1);
+        }
+
+        // ---- epilogue of tile g: registers -> private LDS -> 16-byte row-contiguous stores
+        // (LDS instructions of one wave execute in order, so the region can be reused
+        // without a barrier once the last fragment reads have been issued)
+        const int m0 = cur.mt * 256 + wave * 64;
+        const int j = cur.j;
+        if constexpr (SWAP) {
+            // out[m][n], n contiguous.  One 16-row slab per pass: LDS [16][BN + pad].
+            constexpr int LDE = BN + E16;
+            constexpr int CPR = BN / E16;  // 16-byte chunks per row
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    T vals[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float v = acc[i][t][q];
+                        const int n = j * BN + t * 16 + g4 * 4 + q;
+                        if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m0 + i * 16 + r16 < p.Mc ? m0 + i * 16 + r16 : 0) : n]);
+                        vals[q] = Elem<T>::from_float(v);
+                    }
+                    T* dst = eT + r16 * LDE + t * 16 + g4 * 4;
+                    if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                    else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+                }
+#pragma unroll
+                for (int c0 = 0; c0 < 16 * CPR; c0 += 64) {
+                    const int c = c0 + lane;
+                    const int row = c / CPR;
+                    const int chunk = c % CPR;
+                    const int m = m0 + i * 16 + row;
+                    if (c < 16 * CPR && m < p.Mc)
+                        __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(eT + row * LDE + chunk * E16),
+                                                    reinterpret_cast<u32x4*>(out + (int64_t)m * p.o_ld + (int64_t)j * BN + chunk * E16));
+                }
+            }
+        } else {
+            // out[n][m], m contiguous.  One 16-column slab per pass: LDS [16 n][64 m + pad].
+            constexpr int LDE = 64 + E16;
+            constexpr int CPR = 64 / E16;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    T vals[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float v = acc[i][t][q];
+                        const int m = m0 + i * 16 + g4 * 4 + q;
+                        if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m < p.Mc ? m : 0) : j * BN + t * 16 + r16]);
+                        vals[q] = Elem<T>::from_float(v);
+                    }
+                    T* dst = eT + r16 * LDE + i * 16 + g4 * 4;
+                    if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
+                    else *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(vals);
+                }
+#pragma unroll
+                for (int c0 = 0; c0 < 16 * CPR; c0 += 64) {
+                    const int c = c0 + lane;
+                    const int nrow = c / CPR;
+                    const int chunk = c % CPR;
+                    const int m = m0 + chunk * E16;
+                    if (m < p.Mc)
+                        __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(eT + nrow * LDE + chunk * E16),
+                                                    reinterpret_cast<u32x4*>(out + ((int64_t)j * BN + t * 16 + nrow) * p.o_ld + m));
+                }
+            }
+        }
+
+        // ---- move on: tile g+1 becomes current, the index entries of tile g+2 are fetched --
+        cur = nxt;
+        if (g + 2 < n_tiles) load_tile(g + 2, nxt);
+    }
+}
+
+template <typename T>
+bool spmm_stream_supported(const SpmmParams& p, int BN) {
+    const int kc = 64 / (int)sizeof(T);
+    // element offsets inside a 256-row tile are kept in 32 bits
+    return p.d_kcontig && p.BK % kc == 0 && (BN == 16 || BN == 32 || BN == 64) &&
+           p.d_ld * 256 + 64 < (int64_t)0x7fffffff / (int)sizeof(T);
+}
+
+template <typename T, int BN, int BK, bool SWAP>
+static int launch_spmm_stream_inst(const SpmmParams& p, int batch, hipStream_t st) {
+    const int n_mtiles = (p.Mc + 255) / 256;
+    const int64_t nblocks = (int64_t)kPanelXcd * (p.Nc / BN);
+    if (nblocks > 0x7fffffffLL) return fail(SPX_E_SHAPE, "problem too large for one launch");
+    hipLaunchKernelGGL((spmm_stream_kernel<T, BN, BK, SWAP>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st, p, n_mtiles);
+    SPX_LAUNCH_CHECK("spmm_stream_kernel");
+    return 0;
+}
+
+template <typename T>
+int launch_spmm_stream_impl(const SpmmParams& p, int BN, int batch, hipStream_t st) {
+    const bool swap = p.out_ncontig != 0;
+#define SPX_STREAM_CASE(bn, bk)                                                              \
+    if (BN == bn && p.BK == bk) {                                                            \
+        if constexpr (bk % (64 / (int)sizeof(T)) == 0) {                                     \
+            return swap ? launch_spmm_stream_inst<T, bn, bk, true>(p, batch, st)             \
+                        : launch_spmm_stream_inst<T, bn, bk, false>(p, batch, st);           \
+        }                                                                                    \
+    }
+    SPX_STREAM_CASE(16, 16) SPX_STREAM_CASE(16, 32) SPX_STREAM_CASE(16, 64)
+    SPX_STREAM_CASE(32, 16) SPX_STREAM_CASE(32, 32) SPX_STREAM_CASE(32, 64)
+    SPX_STREAM_CASE(64, 16) SPX_STREAM_CASE(64, 32) SPX_STREAM_CASE(64, 64)
+#undef SPX_STREAM_CASE
+    return fail(SPX_E_CONFIG, "block (%d,%d) not supported by the persistent panel kernel", p.BK, BN);
+}
+
+template <typename T>
+int launch_spmm_stream(const SpmmParams& p, int BN, int batch, hipStream_t st);
+
+}  // namespace spx

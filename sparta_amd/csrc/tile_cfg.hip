@@ -20,6 +20,7 @@ static const spx_tile_cfg kSpmmCfgs[] = {
     {7, 256, 0, 4, 2, 16, 7, "panel-256-sharedS"},
     {8, 64, 0, 4, 2, 16, 7, "panel-64-ksplit"},
     {9, 64, 0, 4, 2, 64, 6, "thin-dense-operand"},
+    {10, 256, 0, 4, 2, 16, 7, "panel-256-persistent"},
 };
 static const spx_tile_cfg kDdsCfgs[] = {
     {0, 0, 0, 4, 1, 16, 7, "auto"},

@@ -98,7 +98,7 @@ def test_matmul_block_shapes(blocks, mode, gpu):
              batch=2, M=192, K=128, N=256, gran=(16, 16), sparsity=0.8, seed=k)
 
 
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6, 7, 8, 10])
 @pytest.mark.parametrize('mode', ['sdd', 'dsd'])
 @pytest.mark.parametrize('compressed', [False, True])
 @pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 64, 32)),
@@ -112,6 +112,20 @@ def test_matmul_tile_configs(tile_cfg, mode, compressed, dtype, blocks, gpu):
     run_case(gpu, mode, False, True, True, compressed, dtype, blocks, batch=2,
              M=320 if mode == 'dsd' else 192, K=256, N=192 if mode == 'dsd' else 328, gran=(16, 16),
              sparsity=0.7, seed=11, tile_cfg=tile_cfg)
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd'])
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 64, 64)),
+                                          (torch.float32, (16, 16, 16)), (torch.float16, (32, 64, 32))])
+def test_matmul_persistent_kernel_walks_several_tiles(mode, compressed, dtype, blocks, gpu):
+    """Tile config 10 with seventeen 256-row tiles of the dense operand, the last one
+    partial: three tiles for the workgroups of the first XCD, two for the others; block
+    columns of zero, one (odd step count) and several live blocks; both output layouts."""
+    dense_rows = 16 * 256 + 104 if mode == 'dsd' else 16 * 256 + 128
+    M, N = (dense_rows, 192) if mode == 'dsd' else (192, dense_rows)
+    run_case(gpu, mode, False, True, True, compressed, dtype, blocks, batch=2, M=M, K=256, N=N,
+             gran=blocks[:2] if mode == 'sdd' else (blocks[2], blocks[1]), sparsity=0.75, seed=17, tile_cfg=10)
 
 
 @pytest.mark.parametrize('tile_cfg', [1, 2])
