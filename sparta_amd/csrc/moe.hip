@@ -414,19 +414,26 @@ __device__ __forceinline__ void lds_direct_load16(const void* g, uint32_t lds_wa
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(g) : "memory", "m0");
 }
 
-template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
-__global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void moe_gemm_direct_kernel(MoeParams p) {
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN>
+__global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 : 2) void moe_gemm_direct_kernel(MoeParams p) {
+    static_assert(!BKN || sizeof(T) == 2, "the [K, N] weight layout is read with 16-bit LDS transpose loads");
     constexpr int NTH = 64 * WAVES;
     constexpr int WGN = WAVES / WGM;
     constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
     constexpr int NTT = TN / WGN / 16;  // 16-column tiles per wave
     constexpr int VE = 16 / (int)sizeof(T);
-    constexpr int KT = MoeKt<T>::value;   // 128 bytes of k per row and stage
-    constexpr int A_LOADS = TM * 8 / NTH;
-    constexpr int B_LOADS = TN * 8 / NTH;
-    constexpr int RSTEP = NTH / 8;        // tile rows between a thread's vectors (a multiple of 8)
-    constexpr int A_BYTES = TM * 128;
-    constexpr int BUF = (TM + TN) * 128;
+    constexpr int KT = KTB / (int)sizeof(T);  // k per row and stage (KTB = 64 or 128 bytes)
+    constexpr int CPR = KTB / 16;             // 16-byte chunks per LDS row
+    constexpr int A_LOADS = TM * CPR / NTH;
+    constexpr int B_LOADS = TN * CPR / NTH;
+    constexpr int RSTEP = NTH / CPR;          // tile rows between a thread's vectors
+    constexpr int A_BYTES = TM * KTB;
+    constexpr int BUF = (TM + TN) * KTB;
+    // chunk c of row r sits at position c ^ swz(r): rows of 128 bytes use the low three bits
+    // of the row, rows of 64 bytes bits 2..3 (sixteen lanes of a 16-byte read then touch
+    // sixteen different 16-byte bank groups)
+    auto swz = [](int row) { return KTB == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
+    auto lds_off = [&](int row, int chunk) { return (row * CPR + (chunk ^ swz(row))) * 16; };
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) char smem[];
     __shared__ int s_expert, s_row0, s_rows;
@@ -456,13 +463,13 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
     const T* X = reinterpret_cast<const T*>(p.tokens);
     const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
 
-    // staging map: every wavefront instruction fills 8 consecutive LDS rows (1 KB); lane l
-    // lands at position l % 8 of row l / 8, so it fetches the chunk that the swizzle
-    // keeps at that position: (l % 8) ^ (row % 8)
-    const int srow = threadIdx.x >> 3;
-    const int chunk = (threadIdx.x & 7) ^ (srow & 7);
+    // staging map: every wavefront instruction fills 1 KB of consecutive LDS rows (8 or 16);
+    // lane l lands at position l % CPR of row l / CPR, so it fetches the chunk that the
+    // swizzle keeps at that position
+    const int srow = threadIdx.x / CPR;
+    const int chunk = (threadIdx.x % CPR) ^ swz(srow);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
-    const uint32_t st_dst = __builtin_amdgcn_readfirstlane(lds_base + (wave * 8) * 128);
+    const uint32_t st_dst = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
     const T* a_src[A_LOADS];
 #pragma unroll
     for (int q = 0; q < A_LOADS; ++q) {
@@ -470,20 +477,40 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
         const int tok = p.token_perm[row0 + (r < rows ? r : rows - 1)];
         a_src[q] = X + (int64_t)tok * p.K + chunk * VE;
     }
+    // Weight tile.  [N, K] storage (k contiguous): rows of KTB bytes like the token tile.
+    // [K, N] storage (BKN, the stacked weight.T of the reference): the stage is kept as
+    // KT k-rows of TN * 2 bytes; a wavefront instruction fills 1 KB of them linearly, the
+    // 32-byte units of a k-row are XOR-swizzled by its low two bits (the source address
+    // carries the swizzle), and the k-contiguous MFMA fragments come out of LDS transpose
+    // reads, sixteen lanes fetching four k-rows of sixteen columns at a time.
+    constexpr int RB = TN * (int)sizeof(T);   // BKN: bytes of a k-row in LDS
+    constexpr int CB = RB / 16;               // BKN: 16-byte slots of a k-row
     const T* b_src[B_LOADS];
 #pragma unroll
     for (int q = 0; q < B_LOADS; ++q) {
-        const int r = srow + RSTEP * q;
-        const int n = n0 + r < p.N ? n0 + r : p.N - 1;
-        b_src[q] = W + (int64_t)n * p.K + chunk * VE;
+        if constexpr (BKN) {
+            const int slot = q * NTH + (int)threadIdx.x;
+            const int kr = slot / CB, c = slot % CB;
+            int n = n0 + ((((c >> 1) ^ (kr & 3)) << 1) | (c & 1)) * VE;
+            if (n + VE > p.N) n = p.N - VE;   // columns past the end re-read valid data; never stored
+            b_src[q] = W + (int64_t)kr * p.N + n;
+        } else {
+            const int r = srow + RSTEP * q;
+            const int n = n0 + r < p.N ? n0 + r : p.N - 1;
+            b_src[q] = W + (int64_t)n * p.K + chunk * VE;
+        }
     }
-    auto issue_stage = [&](int s) {
+    // load q of stage s (q < A_LOADS: token rows, else weight rows)
+    auto issue_one = [&](int s, int q) {
         const uint32_t dst = st_dst + (uint32_t)((s % NBUF) * BUF);
         const int k = s * KT;
+        if (q < A_LOADS) lds_direct_load16(a_src[q] + k, dst + q * RSTEP * KTB);
+        else if constexpr (BKN) lds_direct_load16(b_src[q - A_LOADS] + (int64_t)k * p.N, dst + A_BYTES + (q - A_LOADS) * NTH * 16);
+        else lds_direct_load16(b_src[q - A_LOADS] + k, dst + A_BYTES + (q - A_LOADS) * RSTEP * KTB);
+    };
+    auto issue_stage = [&](int s) {
 #pragma unroll
-        for (int q = 0; q < A_LOADS; ++q) lds_direct_load16(a_src[q] + k, dst + q * RSTEP * 128);
-#pragma unroll
-        for (int q = 0; q < B_LOADS; ++q) lds_direct_load16(b_src[q] + k, dst + A_BYTES + q * RSTEP * 128);
+        for (int q = 0; q < A_LOADS + B_LOADS; ++q) issue_one(s, q);
     };
 
     // 2-byte types: 32 x 32 x 16 MFMAs (twice the sustained rate of the 16 x 16 x 32 ones)
@@ -505,15 +532,24 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
 
     const int n_st = p.K / KT;
     constexpr int L = A_LOADS + B_LOADS;   // loads per thread and stage
-    issue_stage(0);
-    if (NBUF > 2 && n_st > 1) issue_stage(1);
+#pragma unroll
+    for (int s0 = 0; s0 < NBUF - 1; ++s0)
+        if (s0 < n_st) issue_stage(s0);
 
     for (int s = 0; s < n_st; ++s) {
         // stage s has landed once at most the loads of the stages after it are outstanding
-        if (NBUF > 2 && s + 1 < n_st) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L) : "memory");
+        // (NBUF - 2 of them, fewer at the end of the walk)
+        const int newer = n_st - 1 - s < NBUF - 2 ? n_st - 1 - s : NBUF - 2;
+        if (NBUF > 3 && newer == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L) : "memory");
+        else if (NBUF > 2 && newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();   // everyone's part of stage s is in LDS; the buffer of stage s - 1 is free
-        if (s + NBUF - 1 < n_st) issue_stage(s + NBUF - 1);
+        // The loads of stage s + NBUF - 1 go out a few at a time between the MFMA groups of
+        // this stage (16-bit types): issued in one burst right after the barrier, the
+        // sixteen wavefronts queue up behind the address unit (one 1 KB instruction per 16
+        // clocks) with the matrix cores idle.
+        const bool more = s + NBUF - 1 < n_st;
+        if (!WIDE && more) issue_stage(s + NBUF - 1);
         const char* cur = smem + (s % NBUF) * BUF;
         const char* As = cur;
         const char* Bs = cur + A_BYTES;
@@ -524,15 +560,33 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
             auto read_frags = [&](int c, int slot) {
 #pragma unroll
                 for (int i = 0; i < MTW; ++i)
-                    af[slot][i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + moe_lds_off<T>(wrow + i * 32 + l32, c * 2 + h2));
+                    af[slot][i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + lds_off(wrow + i * 32 + l32, c * 2 + h2));
 #pragma unroll
-                for (int t = 0; t < NTW; ++t)
-                    bf[slot][t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 32 + l32, c * 2 + h2));
+                for (int t = 0; t < NTW; ++t) {
+                    if constexpr (BKN) {
+                        typedef short s16x8_t __attribute__((ext_vector_type(8)));
+                        typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
+                        const int kr = c * 16 + 8 * h2 + (r16 >> 2);             // and kr + 4
+                        const int unit = (wcol + t * 32 + 16 * ((lane >> 4) & 1)) >> 4;
+                        const char* at = Bs + kr * RB + ((unit ^ (kr & 3)) << 5) + ((r16 & 3) << 3);
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at));
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at + 4 * RB));
+                        bf[slot][t] = __builtin_bit_cast(typename MmaW<T>::frag,
+                                                         (s16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                    } else {
+                        bf[slot][t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + lds_off(wcol + t * 32 + l32, c * 2 + h2));
+                    }
+                }
             };
+            constexpr int LPS = (L + KSTEPS - 1) / KSTEPS;  // loads per k-step
             read_frags(0, 0);
 #pragma unroll
             for (int c = 0; c < KSTEPS; ++c) {
                 if (c + 1 < KSTEPS) read_frags(c + 1, (c + 1) & 1);
+                if (more) {
+#pragma unroll
+                    for (int q = c * LPS; q < (c + 1) * LPS && q < L; ++q) issue_one(s + NBUF - 1, q);
+                }
                 __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of this step's MFMAs
 #pragma unroll
                 for (int i = 0; i < MTW; ++i)
@@ -545,10 +599,10 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
                 typename Mma16<T>::frag af[MT], bf[NTT];
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
-                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + moe_lds_off<T>(wrow + i * 16 + r16, kc / VE + g4));
+                    af[i] = *reinterpret_cast<const typename Mma16<T>::frag*>(As + lds_off(wrow + i * 16 + r16, kc / VE + g4));
 #pragma unroll
                 for (int t = 0; t < NTT; ++t)
-                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + moe_lds_off<T>(wcol + t * 16 + r16, kc / VE + g4));
+                    bf[t] = *reinterpret_cast<const typename Mma16<T>::frag*>(Bs + lds_off(wcol + t * 16 + r16, kc / VE + g4));
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -617,17 +671,26 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF > 640 ? 1 : 2) void mo
     }
 }
 
-template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF>
-static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN>
+static int launch_moe_direct_inst(const MoeParams& p, hipStream_t st) {
     const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp + 1;
     if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
-    const int smem = NBUF * (TM + TN) * 128;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF>),
+    // the epilogue stages every wavefront's (TM / WGM) x 64 output tile as rows of 128 bytes
+    const int epi = sizeof(T) == 2 ? WAVES * (TM / WGM) * 128 : 0;
+    const int smem = NBUF * (TM + TN) * KTB > epi ? NBUF * (TM + TN) * KTB : epi;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF, KTB, BKN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_direct_kernel)");
-    hipLaunchKernelGGL((moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
+    hipLaunchKernelGGL((moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF, KTB, BKN>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
     SPX_LAUNCH_CHECK("moe_gemm_direct_kernel");
     return 0;
+}
+
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB>
+static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
+    if (p.w_kcontig) return launch_moe_direct_inst<T, TM, TN, WAVES, WGM, NBUF, KTB, false>(p, st);
+    if constexpr (sizeof(T) == 2) return launch_moe_direct_inst<T, TM, TN, WAVES, WGM, NBUF, KTB, true>(p, st);
+    else return fail(SPX_E_CONFIG, "fp32 weights stored [E, in, out] run through tile config 1");
 }
 
 static size_t moe_index_ws(int n_tok, int n_exp) {
@@ -675,7 +738,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -691,16 +754,25 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
     p.w_kcontig = weight_layout == 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    // tile_cfg 0: 2 for k-contiguous weights, else 1; 1: 128x128 tiles staged through
-    // registers (any weight layout); 2, 3: 128x128 (four wavefronts, two workgroups per
-    // CU) and 256x256 (eight wavefronts) tiles filled by LDS-direct loads (k-contiguous
-    // weights only).  2 measured best on the benchmark shapes.
-    if (tile_cfg == 0) tile_cfg = p.w_kcontig ? 2 : 1;
+    // tile_cfg 1: 128x128 tiles staged through registers (any dtype and weight layout);
+    // 2 / 3 / 4: tiles filled by LDS-direct loads - 128x128 with four wavefronts (two
+    // workgroups per CU), 256x256 with eight wavefronts of 128x64, 256x256 with sixteen
+    // wavefronts of 64x64 - for 16-bit types in either weight layout and fp32 with
+    // k-contiguous weights.  0 picks 4 when the problem has enough 256x256 tiles to fill
+    // the device (it moves half the bytes from L2 to the CUs, which is what bounds the
+    // 128x128 kernel), else 2; fp32 [E, in, out] weights take 1.
+    const bool direct_ok = p.w_kcontig || es == 2;
+    if (tile_cfg == 0) {
+        const int64_t big_tiles = (int64_t)((n_tok + 255) / 256) * ((out_dim + 255) / 256);
+        tile_cfg = !direct_ok ? 1 : (es == 2 && big_tiles >= 512 ? 4 : 2);
+    }
+    SPX_REQUIRE(tile_cfg <= 4, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg >= 2) {
-        SPX_REQUIRE(p.w_kcontig, SPX_E_CONFIG, "tile config %d needs weight_layout 1", tile_cfg);
-#define SPX_MOE_DIRECT(T)                                                          \
-        if (tile_cfg == 2) return launch_moe_direct<T, 128, 128, 4, 2, 2>(p, st);  \
-        return launch_moe_direct<T, 256, 256, 8, 2, 2>(p, st);
+        SPX_REQUIRE(direct_ok, SPX_E_CONFIG, "tile config %d takes fp32 weights in layout 1 only", tile_cfg);
+#define SPX_MOE_DIRECT(T)                                                                  \
+        if (tile_cfg == 2) return launch_moe_direct<T, 128, 128, 4, 2, 2, 128>(p, st);     \
+        if (tile_cfg == 3) return launch_moe_direct<T, 256, 256, 8, 2, 2, 128>(p, st);     \
+        return launch_moe_direct<T, 256, 256, 16, 4, 2, 128>(p, st);
         switch (dtype) {
             case SPX_F32: SPX_MOE_DIRECT(float)
             case SPX_F16: SPX_MOE_DIRECT(_Float16)

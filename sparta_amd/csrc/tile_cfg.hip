@@ -45,6 +45,7 @@ static const spx_tile_cfg kMoeCfgs[] = {
     {1, 128, 128, 4, 1, 0, 7, "gather-128x128"},
     {2, 128, 128, 4, 2, 0, 7, "gather-128x128-lds-direct"},
     {3, 256, 256, 8, 2, 0, 7, "gather-256x256-lds-direct"},
+    {4, 256, 256, 16, 2, 0, 7, "gather-256x256-direct-16-waves"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {

@@ -31,33 +31,11 @@ class DynamicSparseMoE(torch.nn.Module):
             # [n_exp, in, out]: each expert's weight transposed once, up front
             stacked = torch.stack([m.weight.t() for m in exp_modules]).contiguous()
         self.weight = torch.nn.Parameter(stacked)
-        # [n_exp, out, in] copy (in contiguous): the layout the GEMM kernel reads fastest,
-        # in the dtype of the tokens.  Rebuilt whenever the parameter's storage, version
-        # counter, dtype or device differ from what the copy was made from, and dropped
-        # by every .to() / .half() / .cuda() of the module.
-        self._weight_nk = None
-        self._weight_nk_key = None
         self._workspace = torch.zeros(0, dtype=torch.uint8, device=self.device)
         i32 = dict(dtype=torch.int32, device=self.device)
         self.expert_count = torch.zeros(self.num_exps, **i32)
         self.expert_offset = torch.zeros(self.num_exps + 1, **i32)
         self.sparse_index = torch.zeros(0, **i32)  # token permutation, sized at first call
-
-    def _apply(self, fn, *args, **kwargs):
-        self._weight_nk = None
-        self._weight_nk_key = None
-        return super()._apply(fn, *args, **kwargs)
-
-    def _kernel_weight(self, dtype: torch.dtype) -> torch.Tensor:
-        """The [n_exp, out, in] copy of `weight` in `dtype`, rebuilt when the parameter's
-        storage, version counter, dtype or device changed."""
-        w = self.weight
-        key = (w.data_ptr(), w._version, w.dtype, str(w.device), dtype)
-        if self._weight_nk is None or self._weight_nk_key != key:
-            with torch.no_grad():
-                self._weight_nk = w.detach().transpose(1, 2).to(dtype).contiguous()
-            self._weight_nk_key = key
-        return self._weight_nk
 
     def forward(self, tokens: torch.Tensor, exp_ids: torch.Tensor):
         n_tok = tokens.shape[0]
@@ -72,7 +50,6 @@ class DynamicSparseMoE(torch.nn.Module):
         ws_bytes = lib.spx_moe_index_workspace_bytes(n_tok, self.num_exps)
         if self._workspace.numel() < ws_bytes:
             self._workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=tokens.device)
-        weight = self._kernel_weight(tokens.dtype)
         stream = _lib.current_stream(tokens.device)
         rc = lib.spx_moe_index(_lib.dev_ptr(exp_ids.contiguous()), n_tok, self.num_exps,
                                _lib.dev_ptr(self.expert_count), _lib.dev_ptr(self.expert_offset),
@@ -81,8 +58,13 @@ class DynamicSparseMoE(torch.nn.Module):
         _lib.check(rc, 'spx_moe_index')
         tokens = tokens.contiguous()
         out = torch.empty((n_tok, self.out_hidden), dtype=tokens.dtype, device=tokens.device)
+        # the stacked [n_exp, in, out] parameter is what the kernel reads (weight layout 0):
+        # there is no second copy that could go stale when the parameter is written to
+        weight = self.weight.detach()
+        if weight.dtype != tokens.dtype:
+            weight = weight.to(tokens.dtype)
         rc = lib.spx_moe_forward(_lib.dtype_code(tokens.dtype), _lib.dev_ptr(tokens),
-                                 _lib.dev_ptr(weight), 1, _lib.dev_ptr(out),
+                                 _lib.dev_ptr(weight.contiguous()), 0, _lib.dev_ptr(out),
                                  _lib.dev_ptr(self.expert_offset), _lib.dev_ptr(self.sparse_index),
                                  n_tok, self.in_hidden, self.out_hidden, self.num_exps, 0, stream)
         _lib.check(rc, 'spx_moe_forward')

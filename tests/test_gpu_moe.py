@@ -98,15 +98,16 @@ def test_moe_golden_vectors(gpu):
 
 
 def test_moe_weight_layouts_agree(gpu):
-    """The [E, in, out] layout of the reference's stacked weight gives the same
-    result as the [E, out, in] copy the operator feeds the kernel."""
+    """The [E, in, out] layout of the reference's stacked weight (what the operator feeds
+    the kernels) gives the same result as an [E, out, in] copy of it."""
     from sparta_amd import _lib
     moe, w = make_moe(4, 128, 256, torch.float16, gpu)
     ids = torch.from_numpy(np.random.default_rng(0).integers(0, 4, 700).astype(np.int32)).to(gpu)
     x = torch.rand((700, 128), dtype=torch.float16, device=gpu)
     want = moe(x, ids)
     out = torch.empty_like(want)
-    rc = _lib.load().spx_moe_forward(_lib.F16, _lib.dev_ptr(x), _lib.dev_ptr(moe.weight.detach()), 0,
+    w_nk = moe.weight.detach().transpose(1, 2).contiguous()
+    rc = _lib.load().spx_moe_forward(_lib.F16, _lib.dev_ptr(x), _lib.dev_ptr(w_nk), 1,
                                      _lib.dev_ptr(out), _lib.dev_ptr(moe.expert_offset),
                                      _lib.dev_ptr(moe.sparse_index), 700, 128, 256, 4, 0,
                                      _lib.current_stream(gpu))
@@ -114,25 +115,71 @@ def test_moe_weight_layouts_agree(gpu):
     assert torch.equal(out, want)
 
 
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3])
+def test_moe_follows_in_place_weight_updates(gpu):
+    """The operator reads its stacked parameter at every call: writes through `.data`
+    (which do not advance the version counter), `.half()` and optimizer-style updates
+    all show up in the next forward."""
+    moe, w = make_moe(3, 128, 136, torch.float32, gpu)
+    ids_np = np.random.default_rng(3).integers(0, 3, 300).astype(np.int32)
+    check_forward(moe, w, 300, ids_np, torch.float32, gpu, 5)
+    with torch.no_grad():
+        moe.weight.data.mul_(-0.5)
+        moe.weight.data[1].add_(0.25)
+    w2 = w * -0.5
+    w2[1] += 0.25
+    check_forward(moe, w2, 300, ids_np, torch.float32, gpu, 6)
+    moe.half()
+    w3 = moe.weight.detach().to(torch.float64).cpu().numpy()
+    check_forward(moe, w3, 300, ids_np, torch.float16, gpu, 7)
+
+
+def test_moe_out_of_range_ids_give_zero_rows(gpu):
+    """Tokens whose expert id is negative or >= n_exp (the reference indexes out of bounds
+    for them) get zero output rows and are listed, ascending, behind the routed tokens."""
+    n_exp, n_tok = 4, 1000
+    moe, w = make_moe(n_exp, 128, 256, torch.float16, gpu)
+    rng = np.random.default_rng(11)
+    ids_np = rng.integers(0, n_exp, n_tok).astype(np.int32)
+    bad = rng.choice(n_tok, 77, replace=False)
+    ids_np[bad[:40]] = -3
+    ids_np[bad[40:]] = n_exp + 2
+    data = torch.from_numpy(rng.random((n_tok, 128), dtype=np.float32)).half()
+    out = torch.full((n_tok, 256), float('nan'), dtype=torch.float16, device=gpu)
+    got = moe(data.to(gpu), torch.from_numpy(ids_np).to(gpu))
+    valid = (ids_np >= 0) & (ids_np < n_exp)
+    want = np.zeros((n_tok, 256))
+    want[valid] = ops.moe_reference(data.to(torch.float64).numpy()[valid], w, ids_np[valid])
+    assert_close(got, want, torch.float16, 'moe with out-of-range ids')
+    assert float(got[torch.from_numpy(~valid).to(gpu)].abs().max()) == 0.0
+    offset = moe.expert_offset.cpu().numpy()
+    assert offset[n_exp] == valid.sum()
+    assert np.array_equal(moe.sparse_index[offset[n_exp]:n_tok].cpu().numpy(), np.sort(bad))
+
+
+@pytest.mark.parametrize('layout', [0, 1])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4])
 @pytest.mark.parametrize('dtype,n_tok,in_dims,out_dims', [
     (torch.float16, 3000, 256, 520), (torch.bfloat16, 1500, 128, 256), (torch.float32, 700, 96, 136),
-    (torch.float16, 5, 64, 64)])
-def test_moe_tile_configs(tile_cfg, dtype, n_tok, in_dims, out_dims, gpu):
-    """Every gathered-GEMM variant through the C ABI on the same routing (one stage, two
-    stages and more; ragged last tiles in both directions; an empty expert)."""
+    (torch.float16, 5, 64, 64), (torch.float16, 2500, 192, 776)])
+def test_moe_tile_configs(layout, tile_cfg, dtype, n_tok, in_dims, out_dims, gpu):
+    """Every gathered-GEMM variant through the C ABI, in both weight layouts, on the same
+    routing (one stage, two stages and more; ragged last tiles in both directions; an
+    empty expert)."""
     from sparta_amd import _lib
+    if dtype == torch.float32 and layout == 0 and tile_cfg != 1:
+        pytest.skip('fp32 weights stored [E, in, out] run through tile config 1')
     n_exp = 5
     moe, w = make_moe(n_exp, in_dims, out_dims, dtype, gpu)
     ids_np = np.random.default_rng(n_tok).choice([0, 1, 2, 4], size=n_tok, p=[0.6, 0.2, 0.15, 0.05]).astype(np.int32)
     x = torch.from_numpy(np.random.default_rng(1).random((n_tok, in_dims), dtype=np.float32)).to(dtype)
     xg = x.to(gpu)
-    moe(xg, torch.from_numpy(ids_np).to(gpu))  # builds the index and the [E, out, in] weight copy
+    moe(xg, torch.from_numpy(ids_np).to(gpu))  # builds the index
+    weight = moe.weight.detach() if layout == 0 else moe.weight.detach().transpose(1, 2).contiguous()
     out = torch.full((n_tok, out_dims), float('nan'), dtype=dtype, device=gpu)
-    rc = _lib.load().spx_moe_forward(_lib.dtype_code(dtype), _lib.dev_ptr(xg), _lib.dev_ptr(moe._weight_nk), 1,
+    rc = _lib.load().spx_moe_forward(_lib.dtype_code(dtype), _lib.dev_ptr(xg), _lib.dev_ptr(weight), layout,
                                      _lib.dev_ptr(out), _lib.dev_ptr(moe.expert_offset),
                                      _lib.dev_ptr(moe.sparse_index), n_tok, in_dims, out_dims, n_exp, tile_cfg,
                                      _lib.current_stream(gpu))
     _lib.check(rc, 'spx_moe_forward')
     want = ops.moe_reference(x.to(torch.float64).numpy(), w, ids_np)
-    assert_close(out, want, dtype, f'moe tile config {tile_cfg} {dtype}')
+    assert_close(out, want, dtype, f'moe tile config {tile_cfg} layout {layout} {dtype}')
