@@ -480,8 +480,9 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
     // Weight tile.  [N, K] storage (k contiguous): rows of KTB bytes like the token tile.
     // [K, N] storage (BKN, the stacked weight.T of the reference): the stage is kept as
     // KT k-rows of TN * 2 bytes; a wavefront instruction fills 1 KB of them linearly, the
-    // 32-byte units of a k-row are XOR-swizzled by its low two bits (the source address
-    // carries the swizzle), and the k-contiguous MFMA fragments come out of LDS transpose
+    // 32-byte units of a k-row are XOR-swizzled by twice its low two bits (the source
+    // address carries the swizzle; the two 16-lane groups that read neighbouring units of
+    // the same four k-rows then cover eight different units), and the k-contiguous MFMA fragments come out of LDS transpose
     // reads, sixteen lanes fetching four k-rows of sixteen columns at a time.
     constexpr int RB = TN * (int)sizeof(T);   // BKN: bytes of a k-row in LDS
     constexpr int CB = RB / 16;               // BKN: 16-byte slots of a k-row
@@ -491,7 +492,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
         if constexpr (BKN) {
             const int slot = q * NTH + (int)threadIdx.x;
             const int kr = slot / CB, c = slot % CB;
-            int n = n0 + ((((c >> 1) ^ (kr & 3)) << 1) | (c & 1)) * VE;
+            int n = n0 + ((((c >> 1) ^ ((kr & 3) << 1)) << 1) | (c & 1)) * VE;
             if (n + VE > p.N) n = p.N - VE;   // columns past the end re-read valid data; never stored
             b_src[q] = W + (int64_t)kr * p.N + n;
         } else {
@@ -568,7 +569,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                         typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
                         const int kr = c * 16 + 8 * h2 + (r16 >> 2);             // and kr + 4
                         const int unit = (wcol + t * 32 + 16 * ((lane >> 4) & 1)) >> 4;
-                        const char* at = Bs + kr * RB + ((unit ^ (kr & 3)) << 5) + ((r16 & 3) << 3);
+                        const char* at = Bs + kr * RB + ((unit ^ ((kr & 3) << 1)) << 5) + ((r16 & 3) << 3);
                         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at));
                         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at + 4 * RB));
                         bf[slot][t] = __builtin_bit_cast(typename MmaW<T>::frag,
