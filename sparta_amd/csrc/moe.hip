@@ -145,38 +145,94 @@ struct MoeParams {
     const int32_t* token_perm;
     int n_tok, K, N, n_exp;
     int w_kcontig;  // weight [E, N, K] if set, else [E, K, N]
+    int split;      // 0: one launch; 1 / 2: first / second launch of a split (see moe_find_tile)
+    int round_rows; // split: 256-row tiles that one round of the big-tile launch covers
 };
 
 // Which (expert, row tile) belongs to tile index y: one wavefront scans the per-expert
 // tile counts.  Expert n_exp is the pseudo expert of the tokens whose id was out of
 // range (token_perm[expert_offset[n_exp] .. n_tok)): its tiles are zero-filled instead
 // of multiplied.  found_e = -1 when y is past the last tile.
+//
+// split (MoeParams::split): a launch of big (256-row) tiles leaves most CUs idle during
+// its last round when the number of row tiles is a little over a multiple of the row
+// tiles one round takes (round_rows).  The work can therefore go out as two launches:
+// split 1 = the 256-row tiles below the last multiple of round_rows (whole rounds),
+// split 2 = the remaining row tiles cut into 128-row halves for the small-tile kernel,
+// which fills the device with them.  Both launches derive the same boundary from the
+// device-side expert counts.
 template <int TM>
 __device__ __forceinline__ void moe_find_tile(const MoeParams& p, int y, int lane,
                                               int& found_e, int& found_row0, int& found_rows) {
+    const int TS = p.split ? 256 : TM;      // tile height the row tiles are counted in
+    int half = 0;
+    if (p.split == 2) { half = y & 1; y >>= 1; }
     int tiles_before = 0;
-    found_e = -1; found_row0 = 0; found_rows = 0;
-    for (int e0 = 0; e0 <= p.n_exp && found_e < 0; e0 += 64) {
+    int fe = -1, frow0 = 0, frows = 0, fy = -1;
+    for (int e0 = 0; e0 <= p.n_exp && (fe < 0 || p.split); e0 += 64) {
         const int e = e0 + lane;
         int cnt = 0, off = 0;
         if (e <= p.n_exp) {
             off = p.expert_offset[e];
             cnt = (e < p.n_exp ? p.expert_offset[e + 1] : p.n_tok) - off;
         }
-        const int tiles = (cnt + TM - 1) / TM;
+        const int tiles = (cnt + TS - 1) / TS;
         const int inc = wave_inclusive_scan(tiles);
         const int excl = tiles_before + inc - tiles;
-        const bool mine = y >= excl && y < excl + tiles;
-        const unsigned long long hit = __ballot(mine);
-        if (hit) {
-            const int src = __ffsll((long long)hit) - 1;
-            const int lt = y - __shfl(excl, src, 64);
-            found_e = e0 + src;
-            found_row0 = __shfl(off, src, 64) + lt * TM;
-            found_rows = min(TM, __shfl(cnt, src, 64) - lt * TM);
+        // split 2 counts y from the boundary, which is only known after the whole scan:
+        // remember every expert's range and pick afterwards (n_exp <= 64 in one pass)
+        if (p.split != 2) {
+            const bool mine = y >= excl && y < excl + tiles;
+            const unsigned long long hit = __ballot(mine);
+            if (hit && fe < 0) {
+                const int src = __ffsll((long long)hit) - 1;
+                const int lt = y - __shfl(excl, src, 64);
+                fe = e0 + src; fy = y;
+                frow0 = __shfl(off, src, 64) + lt * TS;
+                frows = min(TS, __shfl(cnt, src, 64) - lt * TS);
+            }
         }
         tiles_before += __shfl(inc, 63, 64);
     }
+    int boundary = tiles_before;  // first row tile of the second launch
+    if (p.split) {
+        const int rem = tiles_before % p.round_rows;
+        // a last round that is mostly full stays with the big tiles
+        if (rem * 10 <= p.round_rows * 6) boundary = tiles_before - rem;
+    }
+    if (p.split == 1 && fy >= boundary) fe = -1;
+    if (p.split == 2) {
+        const int yb = boundary + y;
+        fe = -1;
+        int before = 0;
+        for (int e0 = 0; e0 <= p.n_exp && fe < 0 && yb < tiles_before; e0 += 64) {
+            const int e = e0 + lane;
+            int cnt = 0, off = 0;
+            if (e <= p.n_exp) {
+                off = p.expert_offset[e];
+                cnt = (e < p.n_exp ? p.expert_offset[e + 1] : p.n_tok) - off;
+            }
+            const int tiles = (cnt + 255) / 256;
+            const int inc = wave_inclusive_scan(tiles);
+            const int excl = before + inc - tiles;
+            const unsigned long long hit = __ballot(yb >= excl && yb < excl + tiles);
+            if (hit) {
+                const int src = __ffsll((long long)hit) - 1;
+                const int lt = yb - __shfl(excl, src, 64);
+                const int r0 = lt * 256 + half * 128;
+                const int left = __shfl(cnt, src, 64) - r0;
+                if (left > 0) {
+                    fe = e0 + src;
+                    frow0 = __shfl(off, src, 64) + r0;
+                    frows = min(128, left);
+                } else {
+                    break;  // the upper half of a row tile with at most 128 rows
+                }
+            }
+            before += __shfl(inc, 63, 64);
+        }
+    }
+    found_e = fe; found_row0 = frow0; found_rows = frows;
 }
 
 // Zero rows token_perm[row0 .. row0 + rows) of `out`, columns n0 .. n0 + TN (16-byte stores).
@@ -674,7 +730,8 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
 
 template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN>
 static int launch_moe_direct_inst(const MoeParams& p, hipStream_t st) {
-    const int tiles = (p.n_tok + TM - 1) / TM + p.n_exp + 1;
+    // split 2 covers at most one round of 256-row tiles, as 128-row halves
+    const int tiles = p.split == 2 ? 2 * p.round_rows : (p.n_tok + TM - 1) / TM + p.n_exp + 1;
     if (tiles > 65535) return fail(SPX_E_SHAPE, "too many row tiles for one launch");
     // the epilogue stages every wavefront's (TM / WGM) x 64 output tile as rows of 128 bytes
     const int epi = sizeof(T) == 2 ? WAVES * (TM / WGM) * 128 : 0;
@@ -739,7 +796,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -754,6 +811,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     p.expert_offset = expert_offset; p.token_perm = token_perm;
     p.n_tok = n_tok; p.K = in_dim; p.N = out_dim; p.n_exp = n_exp;
     p.w_kcontig = weight_layout == 1;
+    p.split = 0; p.round_rows = 1;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // tile_cfg 1: 128x128 tiles staged through registers (any dtype and weight layout);
     // 2 / 3 / 4: tiles filled by LDS-direct loads - 128x128 with four wavefronts (two
@@ -761,16 +819,36 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     // wavefronts of 64x64 - for 16-bit types in either weight layout and fp32 with
     // k-contiguous weights.  0 picks 4 when the problem has enough 256x256 tiles to fill
     // the device (it moves half the bytes from L2 to the CUs, which is what bounds the
-    // 128x128 kernel), else 2; fp32 [E, in, out] weights take 1.
+    // 128x128 kernel), else 2; fp32 [E, in, out] weights take 1.  5 = 4 for the whole
+    // rounds of 256-row tiles plus 2 for the row tiles of a thinly filled last round
+    // (two launches, see moe_find_tile); 0 picks it in place of 4.
     const bool direct_ok = p.w_kcontig || es == 2;
     if (tile_cfg == 0) {
         const int64_t big_tiles = (int64_t)((n_tok + 255) / 256) * ((out_dim + 255) / 256);
-        tile_cfg = !direct_ok ? 1 : (es == 2 && big_tiles >= 512 ? 4 : 2);
+        tile_cfg = !direct_ok ? 1 : (es == 2 && big_tiles >= 512 ? 5 : 2);
     }
-    SPX_REQUIRE(tile_cfg <= 4, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg >= 2) {
         SPX_REQUIRE(direct_ok, SPX_E_CONFIG, "tile config %d takes fp32 weights in layout 1 only", tile_cfg);
+        if (tile_cfg == 5) {
+            static int n_cu = 0;
+            if (n_cu == 0) {
+                int dev = 0;
+                hipDeviceProp_t prop;
+                if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n_cu = prop.multiProcessorCount;
+                if (n_cu <= 0) n_cu = 256;
+            }
+            const int ntn = (out_dim + 255) / 256;
+            p.round_rows = n_cu / ntn > 0 ? n_cu / ntn : 1;
+        }
 #define SPX_MOE_DIRECT(T)                                                                  \
+        if (tile_cfg == 5) {                                                               \
+            p.split = 1;                                                                   \
+            const int rc = launch_moe_direct<T, 256, 256, 16, 4, 2, 128>(p, st);           \
+            if (rc) return rc;                                                             \
+            p.split = 2;                                                                   \
+            return launch_moe_direct<T, 128, 128, 4, 2, 2, 128>(p, st);                    \
+        }                                                                                  \
         if (tile_cfg == 2) return launch_moe_direct<T, 128, 128, 4, 2, 2, 128>(p, st);     \
         if (tile_cfg == 3) return launch_moe_direct<T, 256, 256, 8, 2, 2, 128>(p, st);     \
         return launch_moe_direct<T, 256, 256, 16, 4, 2, 128>(p, st);

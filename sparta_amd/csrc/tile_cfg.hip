@@ -46,6 +46,7 @@ static const spx_tile_cfg kMoeCfgs[] = {
     {2, 128, 128, 4, 2, 0, 7, "gather-128x128-lds-direct"},
     {3, 256, 256, 8, 2, 0, 7, "gather-256x256-lds-direct"},
     {4, 256, 256, 16, 2, 0, 7, "gather-256x256-direct-16-waves"},
+    {5, 256, 256, 16, 2, 0, 7, "gather-256x256-plus-128-tail"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {

@@ -157,7 +157,7 @@ def test_moe_out_of_range_ids_give_zero_rows(gpu):
 
 
 @pytest.mark.parametrize('layout', [0, 1])
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5])
 @pytest.mark.parametrize('dtype,n_tok,in_dims,out_dims', [
     (torch.float16, 3000, 256, 520), (torch.bfloat16, 1500, 128, 256), (torch.float32, 700, 96, 136),
     (torch.float16, 5, 64, 64), (torch.float16, 2500, 192, 776)])
