@@ -379,17 +379,28 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
                 s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
             }
         }
-        float tmax = -1e30f;
+        // masked scores drop to -1e30 once (exp2 of it is 0); a block whose mask bytes are all
+        // 1 for this wavefront - every block of a block-granular pattern - skips the selects
+        if constexpr (HAS_MASK) {
+            unsigned all = live[0];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+            for (int kt = 1; kt < KT; ++kt) all &= live[kt];
+            if (__builtin_amdgcn_ballot_w64(all != 0x01010101u) != 0) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                if constexpr (HAS_MASK) {
-                    if ((live[kt] >> (8 * q)) & 0xffu) tmax = fmaxf(tmax, s[kt][q]);
-                } else {
-                    tmax = fmaxf(tmax, s[kt][q]);
-                }
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) s[kt][q] = ((live[kt] >> (8 * q)) & 0xffu) ? s[kt][q] : -1e30f;
             }
+        }
+        float part[KT];   // independent three-way maxima first, then a short chain over the rest
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) part[kt] = max3f(s[kt][0], s[kt][1], s[kt][2]);
+        float tmax = max3f(part[0], part[1], s[0][3]);
+#pragma unroll
+        for (int kt = 2; kt < KT; kt += 2) tmax = max3f(tmax, part[kt], part[kt + 1]);
+#pragma unroll
+        for (int kt = 1; kt + 1 < KT; kt += 2) tmax = max3f(tmax, s[kt][3], s[kt + 1][3]);
+        tmax = fmaxf(tmax, s[KT - 1][3]);
         tmax = xor32_max(xor16_max(tmax));
         const bool any_live = tmax > -1e29f;
         if (__builtin_amdgcn_ballot_w64(any_live && (fresh || tmax > RESCALE_LOG2)) != 0) {
@@ -411,9 +422,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int kt = 2 * kp + (j >> 2), q = j & 3;
-                float x = __builtin_amdgcn_exp2f(s[kt][q]);
-                if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
-                pv[j] = x;
+                pv[j] = __builtin_amdgcn_exp2f(s[kt][q]);
             }
             pf[kp] = AttnPack<T>::pack(pv);
             // row sums of the rounded probabilities: an all-ones tile in place of V^T

@@ -124,6 +124,8 @@ __device__ __forceinline__ void swap_rows16(float& a, float& b) {
 __device__ __forceinline__ void swap_halves32(float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
 }
+// three-way maximum; nested like this it compiles to one v_max3_f32
+__device__ __forceinline__ float max3f(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 // max / sum over the lanes l, l^16, l^32, l^48 (every lane gets the result)
 __device__ __forceinline__ float xor16_max(float v) { float a = v, b = v; swap_rows16(a, b); return fmaxf(a, b); }
 __device__ __forceinline__ float xor32_max(float v) { float a = v, b = v; swap_halves32(a, b); return fmaxf(a, b); }

@@ -1,10 +1,13 @@
 // MoE sparse forward: out[t,:] = tokens[t,:] . W[exp_ids[t]].
 //
-//  spx_moe_index   stable counting sort of the tokens by expert, three launches,
-//                  no atomics on global memory, no per-expert capacity, no host
-//                  round trip: (1) per-chunk histograms, (2) one workgroup scans
-//                  them in (expert, chunk) order, (3) every chunk places its
-//                  tokens in ascending order behind its scanned base.
+//  spx_moe_index   stable counting sort of the tokens by expert, no atomics on
+//                  global memory, no per-expert capacity, no host round trip:
+//                  (1) per-chunk histograms, (2) an exclusive scan of them in
+//                  (expert, chunk) order, (3) every chunk places its tokens in
+//                  ascending order behind its scanned base.  A table of at most
+//                  1024 (chunk, expert) counts is scanned by every placement
+//                  workgroup itself (two launches); larger ones get a scan
+//                  launch of their own.
 //  spx_moe_forward one gathered GEMM over a flattened (expert, 128-row tile) list:
 //                  a workgroup looks its tile up in the prefix of per-expert tile
 //                  counts, gathers its token rows through token_perm, and walks
@@ -18,18 +21,19 @@
 
 namespace spx {
 
-constexpr int MOE_CHUNK = 1024;   // tokens per workgroup in the index kernels
+constexpr int MOE_CHUNK = 1024;   // most tokens per workgroup in the index kernels (a multiple of 256)
+constexpr int MOE_FUSED_TABLE = 1024;  // (chunk, expert) counts a placement workgroup scans itself
 constexpr int MOE_MAX_EXP = 2048; // LDS table capacity of the placement kernel
 
 // ---- index -------------------------------------------------------------------
-__global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, int n_tok, int n_exp,
+__global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, int n_tok, int n_exp, int chunk,
                                                        int32_t* partial /* [n_chunk][n_exp] */) {
     // n_exp here counts the pseudo expert that collects the tokens whose id is out of range
     extern __shared__ int hist[];
     for (int e = threadIdx.x; e < n_exp; e += 256) hist[e] = 0;
     __syncthreads();
-    const int base = blockIdx.x * MOE_CHUNK;
-    for (int i = threadIdx.x; i < MOE_CHUNK; i += 256) {
+    const int base = blockIdx.x * chunk;
+    for (int i = threadIdx.x; i < chunk; i += 256) {
         const int t = base + i;
         if (t < n_tok) {
             int e = exp_ids[t];
@@ -86,19 +90,59 @@ __global__ __launch_bounds__(1024) void moe_scan_kernel(int32_t* partial, int n_
 
 // Stable placement of one chunk.  Waves take 64 tokens at a time; inside a wave the
 // rank among equal experts comes from ballots, between waves from a small table.
-__global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, int n_tok, int n_exp,
-                                                        const int32_t* base_of /* scanned partial */,
-                                                        int32_t* token_perm) {
+// FUSED: `counts` holds the raw per-chunk histograms (at most MOE_FUSED_TABLE of them);
+// every workgroup scans them in (expert, chunk) order itself and workgroup 0 also writes
+// expert_offset and expert_count.  Otherwise `counts` was scanned by moe_scan_kernel.
+template <bool FUSED>
+__global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, int n_tok, int n_exp, int chunk,
+                                                        const int32_t* counts, int32_t* token_perm,
+                                                        int32_t* expert_count, int32_t* expert_offset) {
     extern __shared__ int sm[];
     int* running = sm;               // [n_exp] tokens of expert e already placed by this chunk
     int* wavecnt = sm + n_exp;       // [4][n_exp] tokens of expert e in the current pass, per wave
+    __shared__ int tab[FUSED ? MOE_FUSED_TABLE : 1];
+    __shared__ int wave_total[4];
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < 5 * n_exp; i += 256) sm[i] = 0;
+    if constexpr (FUSED) {
+        // entries 4 tid .. 4 tid + 3 of the (expert, chunk) order
+        const int n_chunk = gridDim.x;
+        const int n = n_chunk * n_exp;
+        int v[4], sum = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = threadIdx.x * 4 + j;
+            v[j] = 0;
+            if (i < n) {
+                const int e = i / n_chunk, c = i - e * n_chunk;
+                v[j] = counts[c * n_exp + e];
+            }
+            sum += v[j];
+        }
+        const int inc = wave_inclusive_scan(sum);
+        if (lane == 63) wave_total[wave] = inc;
+        __syncthreads();
+        int excl = inc - sum;
+        for (int w = 0; w < wave; ++w) excl += wave_total[w];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = threadIdx.x * 4 + j;
+            if (i < n) tab[i] = excl;
+            excl += v[j];
+        }
+        __syncthreads();
+        if (blockIdx.x == 0) {
+            for (int e = threadIdx.x; e < n_exp; e += 256) {
+                expert_offset[e] = tab[e * n_chunk];
+                if (e + 1 < n_exp) expert_count[e] = tab[(e + 1) * n_chunk] - tab[e * n_chunk];
+            }
+        }
+    }
     __syncthreads();
-    const int chunk0 = blockIdx.x * MOE_CHUNK;
+    const int chunk0 = blockIdx.x * chunk;
     const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    for (int pass = 0; pass < MOE_CHUNK; pass += 256) {
+    for (int pass = 0; pass < chunk; pass += 256) {
         const int t = chunk0 + pass + threadIdx.x;
         int e = -1;
         if (t < n_tok) {
@@ -125,7 +169,8 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, 
         if (e >= 0) {
             int before = running[e];
             for (int w = 0; w < wave; ++w) before += wavecnt[w * n_exp + e];
-            token_perm[base_of[(int64_t)blockIdx.x * n_exp + e] + before + rank] = t;
+            const int base = FUSED ? tab[e * gridDim.x + blockIdx.x] : counts[(int64_t)blockIdx.x * n_exp + e];
+            token_perm[base + before + rank] = t;
         }
         __syncthreads();
         if (leader) {
@@ -751,8 +796,22 @@ static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
     else return fail(SPX_E_CONFIG, "fp32 weights stored [E, in, out] run through tile config 1");
 }
 
+// Tokens per workgroup of the index kernels: the smallest multiple of 256 (up to MOE_CHUNK)
+// whose table of (chunk, expert) counts the placement workgroups can scan themselves;
+// MOE_CHUNK with a scan launch when there is none.
+static int moe_index_chunk(int n_tok, int n_exp, bool* fused) {
+    for (int chunk = 256; chunk <= MOE_CHUNK; chunk += 256) {
+        const int64_t n_chunk = (n_tok + chunk - 1) / chunk;
+        if (n_chunk * (n_exp + 1) <= MOE_FUSED_TABLE) { *fused = true; return chunk; }
+    }
+    *fused = false;
+    return MOE_CHUNK;
+}
+
 static size_t moe_index_ws(int n_tok, int n_exp) {
-    const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
+    bool fused;
+    const int chunk = moe_index_chunk(n_tok, n_exp, &fused);
+    const int n_chunk = (n_tok + chunk - 1) / chunk;
     return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * (n_exp + 1) * sizeof(int32_t), 256);
 }
 
@@ -776,16 +835,25 @@ extern "C" int spx_moe_index(const int32_t* exp_ids, int n_tok, int n_exp,
     SPX_REQUIRE(aligned(workspace, 256), SPX_E_ALIGN, "workspace must be 256-byte aligned");
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     int32_t* partial = reinterpret_cast<int32_t*>(workspace);
-    const int n_chunk = (n_tok + MOE_CHUNK - 1) / MOE_CHUNK;
+    bool fused;
+    const int chunk = moe_index_chunk(n_tok, n_exp, &fused);
+    const int n_chunk = (n_tok + chunk - 1) / chunk;
     if (n_chunk > 0) {
-        hipLaunchKernelGGL(moe_hist_kernel, dim3(n_chunk), dim3(256), (n_exp + 1) * sizeof(int), st, exp_ids, n_tok, n_exp + 1, partial);
+        hipLaunchKernelGGL(moe_hist_kernel, dim3(n_chunk), dim3(256), (n_exp + 1) * sizeof(int), st, exp_ids, n_tok, n_exp + 1, chunk, partial);
         SPX_LAUNCH_CHECK("moe_hist_kernel");
     }
-    hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, st, partial, n_chunk, n_exp + 1, expert_count, expert_offset);
-    SPX_LAUNCH_CHECK("moe_scan_kernel");
+    if (!fused || n_chunk == 0) {
+        hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, st, partial, n_chunk, n_exp + 1, expert_count, expert_offset);
+        SPX_LAUNCH_CHECK("moe_scan_kernel");
+    }
     if (n_chunk > 0) {
-        hipLaunchKernelGGL(moe_place_kernel, dim3(n_chunk), dim3(256), 5 * (n_exp + 1) * sizeof(int), st, exp_ids, n_tok,
-                           n_exp + 1, partial, token_perm);
+        const size_t smem = 5 * (n_exp + 1) * sizeof(int);
+        if (fused)
+            hipLaunchKernelGGL(moe_place_kernel<true>, dim3(n_chunk), dim3(256), smem, st, exp_ids, n_tok, n_exp + 1, chunk, partial,
+                               token_perm, expert_count, expert_offset);
+        else
+            hipLaunchKernelGGL(moe_place_kernel<false>, dim3(n_chunk), dim3(256), smem, st, exp_ids, n_tok, n_exp + 1, chunk, partial,
+                               token_perm, expert_count, expert_offset);
         SPX_LAUNCH_CHECK("moe_place_kernel");
     }
     return 0;
