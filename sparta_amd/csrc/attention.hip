@@ -237,6 +237,37 @@ template <> struct AttnPack<bf16_t> {
     __device__ static bf16x8 pack(f32x8 v) { return __builtin_convertvector(v, bf16x8); }
 };
 
+// Scores of masked keys drop to -1e30 (exp2 of it is exactly 0, so nothing is selected
+// afterwards).  live[kt] holds the mask bytes of the lane's four keys of tile kt; a tile
+// whose bytes are all 1 for the whole wavefront - every tile of a block-granular pattern -
+// skips the selects.
+template <int KT>
+__device__ __forceinline__ void mask_scores(f32x4 (&s)[KT], const unsigned (&live)[KT]) {
+    unsigned all = live[0];
+#pragma unroll
+    for (int kt = 1; kt < KT; ++kt) all &= live[kt];
+    if (__builtin_amdgcn_ballot_w64(all != 0x01010101u) != 0) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) s[kt][q] = ((live[kt] >> (8 * q)) & 0xffu) ? s[kt][q] : -1e30f;
+    }
+}
+// Maximum of the lane's 4 * KT scores: independent three-way maxima, then a short chain
+// (fmaxf in a select per value costs three v_max_f32 each on MFMA results).
+template <int KT>
+__device__ __forceinline__ float lane_max(const f32x4 (&s)[KT]) {
+    float part[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) part[kt] = max3f(s[kt][0], s[kt][1], s[kt][2]);
+    float m = max3f(part[0], part[1], s[0][3]);
+#pragma unroll
+    for (int kt = 2; kt < KT; kt += 2) m = max3f(m, part[kt], part[kt + 1]);
+#pragma unroll
+    for (int kt = 1; kt + 1 < KT; kt += 2) m = max3f(m, s[kt][3], s[kt + 1][3]);
+    return fmaxf(m, s[KT - 1][3]);
+}
+
 // SEQ: no index and no mask bytes; entry b attends over its first L = seqlens[b / heads]
 // positions: the walk covers the key blocks below L, a key is live iff its position is, and
 // queries at or past L give zeros (block rows at or past L walk nothing).
@@ -379,28 +410,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
                 s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
             }
         }
-        // masked scores drop to -1e30 once (exp2 of it is 0); a block whose mask bytes are all
-        // 1 for this wavefront - every block of a block-granular pattern - skips the selects
-        if constexpr (HAS_MASK) {
-            unsigned all = live[0];
-#pragma unroll
-            for (int kt = 1; kt < KT; ++kt) all &= live[kt];
-            if (__builtin_amdgcn_ballot_w64(all != 0x01010101u) != 0) {
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) s[kt][q] = ((live[kt] >> (8 * q)) & 0xffu) ? s[kt][q] : -1e30f;
-            }
-        }
-        float part[KT];   // independent three-way maxima first, then a short chain over the rest
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) part[kt] = max3f(s[kt][0], s[kt][1], s[kt][2]);
-        float tmax = max3f(part[0], part[1], s[0][3]);
-#pragma unroll
-        for (int kt = 2; kt < KT; kt += 2) tmax = max3f(tmax, part[kt], part[kt + 1]);
-#pragma unroll
-        for (int kt = 1; kt + 1 < KT; kt += 2) tmax = max3f(tmax, s[kt][3], s[kt + 1][3]);
-        tmax = fmaxf(tmax, s[KT - 1][3]);
+        if constexpr (HAS_MASK) mask_scores<KT>(s, live);
+        float tmax = lane_max<KT>(s);
         tmax = xor32_max(xor16_max(tmax));
         const bool any_live = tmax > -1e29f;
         if (__builtin_amdgcn_ballot_w64(any_live && (fresh || tmax > RESCALE_LOG2)) != 0) {
@@ -659,17 +670,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
                     s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
                 }
             }
-            float tmax = -1e30f;
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if constexpr (HAS_MASK) {
-                        if ((live[kt] >> (8 * q)) & 0xffu) tmax = fmaxf(tmax, s[kt][q]);
-                    } else {
-                        tmax = fmaxf(tmax, s[kt][q]);
-                    }
-                }
+            if constexpr (HAS_MASK) mask_scores<KT>(s, live);
+            float tmax = lane_max<KT>(s);
             tmax = xor32_max(xor16_max(tmax));
             const bool any_live = tmax > -1e29f;
             if (__builtin_amdgcn_ballot_w64(any_live && (fresh || tmax > RESCALE_LOG2)) != 0) {
@@ -684,9 +686,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    float x = __builtin_amdgcn_exp2f(s[kt][q]);
-                    if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
-                    l_part += x;
+                    l_part += __builtin_amdgcn_exp2f(s[kt][q]);
                 }
         }
     }
@@ -741,6 +741,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
                 s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
             }
         }
+        if constexpr (HAS_MASK) mask_scores<KT>(s, live);
         Frag pf[KT / 2];
 #pragma unroll
         for (int kp = 0; kp < KT / 2; ++kp) {
@@ -748,9 +749,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int kt = 2 * kp + (j >> 2), q = j & 3;
-                float x = __builtin_amdgcn_exp2f(s[kt][q]) * inv_l;
-                if constexpr (HAS_MASK) x = ((live[kt] >> (8 * q)) & 0xffu) ? x : 0.f;
-                pv[j] = x;
+                pv[j] = __builtin_amdgcn_exp2f(s[kt][q]) * inv_l;
             }
             pf[kp] = AttnPack<T>::pack(pv);
             const s16x8 bits = __builtin_bit_cast(s16x8, pf[kp]);
