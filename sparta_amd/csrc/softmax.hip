@@ -220,23 +220,40 @@ __device__ __forceinline__ int64_t vector_offset(const SoftmaxParams& p, const R
 // LPR lanes share a row (16: four rows per wavefront, for rows of up to 16 * SMV_CACHE
 // vectors; 64: one row per wavefront, any length).
 template <int LPR> __device__ __forceinline__ float group_reduce_max(float v) {
-    v = row16_reduce_max(v);
-    if constexpr (LPR == 64) {
-        v = fmaxf(v, __shfl_xor(v, 16, 64));
-        v = fmaxf(v, __shfl_xor(v, 32, 64));
-    }
+    v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror: 8 lanes
+    if constexpr (LPR >= 16) v = fmaxf(v, dpp_move<0x140>(v));  // row_mirror: 16 lanes
+    if constexpr (LPR >= 32) v = fmaxf(v, __shfl_xor(v, 16, 64));
+    if constexpr (LPR == 64) v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
 }
 template <int LPR> __device__ __forceinline__ float group_reduce_sum(float v) {
-    v = row16_reduce_sum(v);
-    if constexpr (LPR == 64) {
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
-    }
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    if constexpr (LPR >= 16) v += dpp_move<0x140>(v);
+    if constexpr (LPR >= 32) v += __shfl_xor(v, 16, 64);
+    if constexpr (LPR == 64) v += __shfl_xor(v, 32, 64);
     return v;
 }
 
-template <typename T, bool BACKWARD, int LPR>
+// Maximum of VE values as nested three-way maxima (one v_max3_f32 each).
+template <int VE>
+__device__ __forceinline__ float vec_max(const float* f) {
+    float m = max3f(f[0], f[1], f[2]);
+    if constexpr (VE == 8) {
+        m = max3f(m, f[3], f[4]);
+        m = max3f(m, f[5], f[6]);
+        return fmaxf(m, f[7]);
+    } else {
+        return fmaxf(m, f[3]);
+    }
+}
+
+// HAS_MASK = false: every entry of a live block takes part (p.mask is NULL) and no mask
+// word is read or tested.
+template <typename T, bool BACKWARD, int LPR, bool HAS_MASK>
 __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParams p) {
     constexpr int VE = SmVec<T>::VE;
     constexpr int RPW = 64 / LPR;
@@ -259,56 +276,72 @@ __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParam
     const T* x = reinterpret_cast<const T*>(p.x) + boff;
     const T* yin = BACKWARD ? reinterpret_cast<const T*>(p.y_in) + boff : nullptr;
     T* out = reinterpret_cast<T*>(p.out) + boff;
+    auto on = [](mask_t m, int i) { return !HAS_MASK || ((m >> (8 * i)) & 0xff) != 0; };
+    auto mask_at = [&](int64_t off) { return HAS_MASK ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0; };
 
     float cache[SMV_CACHE][VE];
     float ycache[BACKWARD ? SMV_CACHE : 1][VE];
-    mask_t live[SMV_CACHE];
+    mask_t live[HAS_MASK ? SMV_CACHE : 1];
     int64_t offs[SMV_CACHE];
 #pragma unroll
     for (int t = 0; t < SMV_CACHE; ++t) {
         const int v = lane + LPR * t;
-        live[t] = 0;
         offs[t] = 0;
+        if constexpr (HAS_MASK) live[t] = 0;
         if (v < nvec) {
             offs[t] = vector_offset<VE>(p, rv, v, log_vpb);
-            live[t] = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + offs[t]) : ~(mask_t)0;
+            if constexpr (HAS_MASK) live[t] = mask_at(offs[t]);
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + offs[t]), cache[t]);
             if (BACKWARD) SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + offs[t]), ycache[t]);
         }
     }
     if (!BACKWARD) {
+        // exp((x - max) / T) as exp2(x * c + nb): one fused multiply-add per entry
+        const float c = p.inv_t * 1.4426950408889634f;
         float vmax = -INFINITY;
 #pragma unroll
-        for (int t = 0; t < SMV_CACHE; ++t)
+        for (int t = 0; t < SMV_CACHE; ++t) {
+            if (lane + LPR * t < nvec) {
+                if constexpr (HAS_MASK) {
 #pragma unroll
-            for (int i = 0; i < VE; ++i)
-                if ((live[t] >> (8 * i)) & 0xff) vmax = fmaxf(vmax, cache[t][i]);
+                    for (int i = 0; i < VE; ++i)
+                        if (on(live[t], i)) vmax = fmaxf(vmax, cache[t][i]);
+                } else {
+                    vmax = fmaxf(vmax, vec_max<VE>(cache[t]));
+                }
+            }
+        }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
             const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
-            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            const mask_t m = mask_at(off);
             float f[VE];
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), f);
 #pragma unroll
             for (int i = 0; i < VE; ++i)
-                if ((m >> (8 * i)) & 0xff) vmax = fmaxf(vmax, f[i]);
+                if (on(m, i)) vmax = fmaxf(vmax, f[i]);
         }
         vmax = group_reduce_max<LPR>(vmax);
+        const float nb = vmax == -INFINITY ? 0.f : -vmax * c;   // a row without live entries sums to 0
         float sum = 0.f;
 #pragma unroll
-        for (int t = 0; t < SMV_CACHE; ++t)
+        for (int t = 0; t < SMV_CACHE; ++t) {
+            if (lane + LPR * t < nvec) {
 #pragma unroll
-            for (int i = 0; i < VE; ++i) {
-                cache[t][i] = ((live[t] >> (8 * i)) & 0xff) ? __expf((cache[t][i] - vmax) * p.inv_t) : 0.f;
-                sum += cache[t][i];
+                for (int i = 0; i < VE; ++i) {
+                    const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(cache[t][i], c, nb));
+                    cache[t][i] = HAS_MASK ? (on(live[t], i) ? e : 0.f) : e;
+                    sum += cache[t][i];
+                }
             }
+        }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
             const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
-            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            const mask_t m = mask_at(off);
             float f[VE];
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), f);
 #pragma unroll
             for (int i = 0; i < VE; ++i)
-                if ((m >> (8 * i)) & 0xff) sum += __expf((f[i] - vmax) * p.inv_t);
+                if (on(m, i)) sum += __builtin_amdgcn_exp2f(__builtin_fmaf(f[i], c, nb));
         }
         sum = group_reduce_sum<LPR>(sum);
         const float inv = sum > 0.f ? 1.f / sum : 0.f;
@@ -322,35 +355,38 @@ __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParam
         }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
             const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
-            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            const mask_t m = mask_at(off);
             float f[VE];
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), f);
 #pragma unroll
             for (int i = 0; i < VE; ++i)
-                f[i] = ((m >> (8 * i)) & 0xff) ? __expf((f[i] - vmax) * p.inv_t) * inv : 0.f;
+                f[i] = on(m, i) ? __builtin_amdgcn_exp2f(__builtin_fmaf(f[i], c, nb)) * inv : 0.f;
             *reinterpret_cast<vec16*>(out + off) = SmVec<T>::pack(f);
         }
     } else {
         // cache holds grad_y, ycache holds y; grad_x = inv_t * y * (grad_y - sum(y * grad_y))
         float dot = 0.f;
 #pragma unroll
-        for (int t = 0; t < SMV_CACHE; ++t)
+        for (int t = 0; t < SMV_CACHE; ++t) {
+            if (lane + LPR * t < nvec) {
 #pragma unroll
-            for (int i = 0; i < VE; ++i) {
-                const bool on = (live[t] >> (8 * i)) & 0xff;
-                ycache[t][i] = on ? ycache[t][i] : 0.f;
-                cache[t][i] = on ? ycache[t][i] * cache[t][i] : 0.f;
-                dot += cache[t][i];
+                for (int i = 0; i < VE; ++i) {
+                    if constexpr (HAS_MASK) ycache[t][i] = on(live[t], i) ? ycache[t][i] : 0.f;
+                    cache[t][i] = ycache[t][i] * cache[t][i];
+                    if constexpr (HAS_MASK) cache[t][i] = on(live[t], i) ? cache[t][i] : 0.f;
+                    dot += cache[t][i];
+                }
             }
+        }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
             const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
-            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            const mask_t m = mask_at(off);
             float g[VE], yv[VE];
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), g);
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + off), yv);
 #pragma unroll
             for (int i = 0; i < VE; ++i)
-                if ((m >> (8 * i)) & 0xff) dot += yv[i] * g[i];
+                if (on(m, i)) dot += yv[i] * g[i];
         }
         dot = group_reduce_sum<LPR>(dot);
 #pragma unroll
@@ -363,13 +399,13 @@ __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParam
         }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
             const int64_t off = vector_offset<VE>(p, rv, v, log_vpb);
-            const mask_t m = p.mask ? *reinterpret_cast<const mask_t*>(p.mask + off) : ~(mask_t)0;
+            const mask_t m = mask_at(off);
             float g[VE], yv[VE];
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + off), g);
             SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + off), yv);
 #pragma unroll
             for (int i = 0; i < VE; ++i)
-                g[i] = ((m >> (8 * i)) & 0xff) ? p.inv_t * (yv[i] * g[i] - yv[i] * dot) : 0.f;
+                g[i] = on(m, i) ? p.inv_t * (yv[i] * g[i] - yv[i] * dot) : 0.f;
             *reinterpret_cast<vec16*>(out + off) = SmVec<T>::pack(g);
         }
     }
@@ -411,8 +447,10 @@ static int launch_softmax(int dtype, int compressed, const void* x, const void* 
         dim3 vgrid((H + rows_per_group - 1) / rows_per_group, batch, 1);
         dim3 vblock(64 * SMV_ROWS);
 #define SPX_SMV(T) \
-        if (narrow) hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 16>), vgrid, vblock, 0, st, p); \
-        else hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 64>), vgrid, vblock, 0, st, p);
+        if (narrow && mask) hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 16, true>), vgrid, vblock, 0, st, p); \
+        else if (narrow) hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 16, false>), vgrid, vblock, 0, st, p); \
+        else if (mask) hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 64, true>), vgrid, vblock, 0, st, p); \
+        else hipLaunchKernelGGL((softmax_vec_kernel<T, BACKWARD, 64, false>), vgrid, vblock, 0, st, p);
         switch (dtype) {
             case SPX_F32: SPX_SMV(float) break;
             case SPX_F16: SPX_SMV(_Float16) break;
