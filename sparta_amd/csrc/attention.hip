@@ -1085,7 +1085,10 @@ static int launch_attention_bwd_row(const AttnParams& p, int batch, int BW, int 
 // The score gradient never goes to memory: P is read once here and once by the row-side
 // kernel, instead of P and dS being read by two separate products after dS was written.
 template <typename T, int BH, int E, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void attention_bwd_col_kernel(AttnParams p, int nbc, int batch) {
+// second launch bound: wavefronts per SIMD the register budget is sized for (small tiles fit
+// 168 VGPRs; the default budget made the compiler park accumulators in AGPRs and copy them
+// back and forth every step)
+__global__ __launch_bounds__(64 * WAVES, (BH * E <= 64 * 64 || BH == 32) ? 3 : (BH * E <= 128 * 64 ? 2 : 1)) void attention_bwd_col_kernel(AttnParams p, int nbc, int batch) {
     constexpr int BW = 16 * WAVES;
     constexpr int NT = 64 * WAVES;
     constexpr int QT = BH / 16, ET = E / 16, EC = E / 32;
