@@ -96,6 +96,49 @@ def test_moe_golden_vectors(gpu):
     assert np.array_equal(moe.expert_offset.cpu().numpy(), GOLD['moe_offset'])
     assert_close(out, GOLD['moe_out'], torch.float16, 'moe golden')
 
+@pytest.mark.parametrize('n_tok,n_exp', [
+    (700, 3),          # 256-token chunks, count table scanned by the placement workgroups
+    (16384, 8),        # 64 chunks x 9 counts
+    (50000, 8),        # 512-token chunks
+    (100000, 8),       # 1024-token chunks, still within the 1024-entry table
+    (4096, 200),       # many experts: 1024-token chunks, 4 x 201 counts
+    (200000, 8),       # table too large: separate scan launch
+    (30000, 200),      # separate scan launch, many experts
+    (257, 1),
+])
+def test_moe_index_launch_paths(n_tok, n_exp, gpu):
+    """spx_moe_index through the C ABI on routings that take every chunk size of the
+    two-launch path and the three-launch path, ids outside [0, n_exp) included: counts,
+    offsets and the stable permutation are bit-exact against the oracle."""
+    from sparta_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(n_tok + n_exp)
+    p = np.arange(1, n_exp + 1, dtype=np.float64) ** -1.2
+    ids_np = rng.choice(n_exp, size=n_tok, p=p / p.sum()).astype(np.int32)
+    bad = rng.random(n_tok) < 0.01
+    ids_np[bad] = rng.choice([-3, n_exp, n_exp + 7], size=int(bad.sum()))
+    ids = torch.from_numpy(ids_np).to(gpu)
+    count = torch.full((n_exp,), -1, dtype=torch.int32, device=gpu)
+    offset = torch.full((n_exp + 1,), -1, dtype=torch.int32, device=gpu)
+    perm = torch.full((n_tok,), -1, dtype=torch.int32, device=gpu)
+    ws = torch.empty(max(lib.spx_moe_index_workspace_bytes(n_tok, n_exp), 256), dtype=torch.uint8, device=gpu)
+    for _ in range(2):  # the workspace is reused as it was left
+        _lib.check(lib.spx_moe_index(_lib.dev_ptr(ids), n_tok, n_exp, _lib.dev_ptr(count), _lib.dev_ptr(offset),
+                                     _lib.dev_ptr(perm), _lib.dev_ptr(ws), ws.numel(), _lib.current_stream(gpu)),
+                   'spx_moe_index')
+    valid = (ids_np >= 0) & (ids_np < n_exp)
+    key = np.where(valid, ids_np, n_exp)                  # out-of-range ids sort behind every expert
+    want_count = np.bincount(key, minlength=n_exp + 1)[:n_exp].astype(np.int32)
+    want_offset = np.zeros(n_exp + 1, dtype=np.int32)
+    np.cumsum(want_count, out=want_offset[1:])
+    want_perm = np.argsort(key, kind='stable').astype(np.int32)
+    c2, o2, p2 = ops.moe_index_reference(ids_np[valid], n_exp)
+    assert np.array_equal(want_count, c2) and np.array_equal(want_offset, o2)   # the oracle on the valid ids
+    assert np.array_equal(count.cpu().numpy(), want_count)
+    assert np.array_equal(offset.cpu().numpy(), want_offset)
+    assert np.array_equal(perm.cpu().numpy(), want_perm)
+    assert np.array_equal(np.flatnonzero(valid)[p2], want_perm[:int(valid.sum())])
+
 
 def test_moe_weight_layouts_agree(gpu):
     """The [E, in, out] layout of the reference's stacked weight (what the operator feeds
