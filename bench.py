@@ -128,7 +128,8 @@ def main():
                          'command shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic')
     ap.add_argument('--config', default='headline',
                     help="'headline' (default, the one JSON line the harness reads) or one of c1..c5 / seqlen / all: "
-                         "secondary measurements of the other benchmark configurations")
+                         "secondary measurements of the other benchmark configurations; 'ceilings': what plain "
+                         "read-only, write-only and copy kernels reach on this machine")
     ap.add_argument('--no-secondary', action='store_true',
                     help="leave out the 'secondary' object (the other benchmark configurations, each checked "
                          'against the dense computation before it is timed) and the cold-operand variant')

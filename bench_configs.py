@@ -1,5 +1,5 @@
 """Secondary measurements for the benchmark configurations other than the headline
-line of bench.py: `python bench.py --config c1|c2|c3|c4|c5|all`.  Prints one JSON
+line of bench.py: `python bench.py --config c1|c2|c3|c4|c5|seqlen|ceilings|all`.  Prints one JSON
 object per measurement.  Inputs are synthetic, generated on the CPU with fixed
 seeds and copied to the GPU."""
 import json
@@ -70,6 +70,18 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
 
     cfg32 = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32}
     with torch.no_grad():
+        if 'ceilings' in todo:
+            # What plain streaming kernels (torch's own) reach on this machine, for reading the
+            # HBM fractions of the memory-bound kernels: a read-only reduction, a write-only
+            # fill and a copy, each over 1 GiB (four times the last-level cache).
+            n = 1 << 28
+            src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
+            dst = torch.empty_like(src)
+            for name, fn, nbytes in (('ceiling: read-only torch.sum over 1 GiB', lambda: torch.sum(src), 4 * n),
+                                     ('ceiling: write-only fill of 1 GiB', lambda: dst.fill_(1.0), 4 * n),
+                                     ('ceiling: copy of 1 GiB (read + write)', lambda: dst.copy_(src), 8 * n)):
+                _emit(name, timed(fn), bytes_alg=nbytes)
+            del src, dst
         if 'c1' in todo:
             g = torch.Generator().manual_seed(2022)
             x = torch.rand((1024, 1024), generator=g).to(dev)

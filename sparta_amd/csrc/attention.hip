@@ -188,27 +188,6 @@ __global__ __launch_bounds__(512) void attention_kernel(AttnParams p) {
     }
 }
 
-// Store a wave's 16 x W output tile (W 2-byte elements per row, rows contiguous in memory)
-// from the MFMA layout, where lane (r16, g4) holds the four elements 16 t + 4 g4 .. + 3 of
-// row r16 as pieces[t]: the pieces pass through a wave-private LDS tile and reach memory as
-// whole 16-byte vectors.  8-byte pieces stored directly arrive as partial cache lines and
-// cost about twice the time.
-template <int W>
-__device__ __forceinline__ void wave_rows_store(char* tile, void* dst, const uint64_t* pieces) {
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    constexpr int PP = W * 2 + 16;
-    const int lane = lane_id();
-    const int r16 = lane & 15, g4 = lane >> 4;
-#pragma unroll
-    for (int t = 0; t < W / 16; ++t) *reinterpret_cast<uint64_t*>(tile + r16 * PP + t * 32 + g4 * 8) = pieces[t];
-#pragma unroll
-    for (int i = 0; i < W / 32; ++i) {
-        const int c = i * 64 + lane;
-        *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst) + c * 16) =
-            *reinterpret_cast<const u32x4*>(tile + (c / (W / 8)) * PP + (c % (W / 8)) * 16);
-    }
-}
-
 // ---- pipelined variant ------------------------------------------------------------------
 // Same mathematics and register layout as attention_kernel, rebuilt around the
 // instruction budget of a block step:

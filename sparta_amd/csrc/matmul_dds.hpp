@@ -666,6 +666,169 @@ static int launch_dds_row_inst(const DdsParams& p, int batch, hipStream_t st) {
     return 0;
 }
 
+// ---- short-K variant for 16-bit types and compressed output: a wavefront per 16 rows --------
+// The workgroup-wide kernel above spends a block step in two barriers and an fp32 round
+// trip through LDS, and - like every kernel here that loads and stores in the same loop -
+// it pays for the fact that loads and stores share one in-order completion counter
+// (vmcnt) on this chip: waiting for a prefetched panel also waits for the output stores
+// issued before it, so the 308 MB of scores of the attention shape and the work that
+// produces them ran one after the other (90 us = 48 us with the stores removed + the 45 us
+// a plain fill of the same size takes).  This kernel separates the two streams by
+// wavefront:
+//   * WAVES compute wavefronts own 16 rows of the block row each for the whole walk: A
+//     fragments in registers (loaded once), products taken transposed (B rows as the first
+//     MFMA operand) so that a lane ends up with four consecutive n of one output row; the
+//     wave passes its 16 x BN tile through a private LDS tile and stores whole 16-byte
+//     vectors - 16 complete, contiguous rows of the compressed block.  They never wait on
+//     vmcnt inside the loop.
+//   * one more wavefront only loads: the B panel of step i + 2 goes global -> LDS
+//     (global_load_lds_dwordx4, the XOR swizzle applied to the source address) into one of
+//     three buffers while steps i and i + 1 are computed; its waits see loads only.
+//   * one barrier per step hands a panel over; workgroup L runs on XCD L % 8 and every
+//     batch entry (whose B operand all of its block rows share) stays within one XCD's L2.
+// Needs row_ptr, k-contiguous operands, K of 64 or 128 and the compressed output layout.
+template <typename T, int BN, int K, int WAVES, bool HAS_BIAS>
+__global__ __launch_bounds__(64 * (WAVES + 1)) void dds_rowq_kernel(DdsParams p, int batch) {
+    static_assert(sizeof(T) == 2, "16-bit types only");
+    constexpr int BM = 16 * WAVES;
+    constexpr int KT = BN / 16, EC = K / 32;
+    constexpr int KP = K * 2;                 // bytes per staged B row
+    constexpr int PANEL = BN * KP;
+    constexpr int CPR = KP / 16;              // 16-byte chunks per B row
+    constexpr int NVL = PANEL / 1024;         // loader instructions per panel (1 KB each)
+    constexpr int RPI = 1024 / KP;            // panel rows per loader instruction
+    constexpr int NBUF = 3;
+    constexpr int OT = 16 * (BN * 2 + 16);    // a wavefront's output tile
+    static_assert(PANEL % 1024 == 0 && RPI >= 1, "panel is not a whole number of loader instructions");
+    typedef typename Mma32<T>::frag Frag;
+    extern __shared__ __align__(16) char smem[];
+
+    const int nbr = p.M / BM;
+    const int L = blockIdx.x;
+    const int slot = L >> 3;
+    const int64_t b = (int64_t)(slot / nbr) * 8 + (L & 7);
+    const int bi = slot % nbr;
+    if (b >= batch) return;
+    const int e_begin = p.row_ptr[bi];
+    const int n_blk = p.row_ptr[bi + 1] - e_begin;
+    if (n_blk <= 0) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    // block columns of the row: lane l holds entry l; longer rows read the rest from the index
+    int bj_vec = 0;
+    if (lane < n_blk) bj_vec = p.idx[e_begin + lane] & 0xffff;
+    auto column = [&](int i) {
+        return i < 64 ? __builtin_amdgcn_readlane(bj_vec, i) : (p.idx[e_begin + i] & 0xffff);
+    };
+
+    if (wave == WAVES) {
+        // ---- loader ---------------------------------------------------------------------------
+        const T* B = reinterpret_cast<const T*>(p.B) + b * p.b_batch;
+        const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+        // lane l of instruction q lands at byte q * 1024 + l * 16 of the panel: row q * RPI + l / CPR,
+        // position l % CPR, which holds chunk position ^ (row & 7)
+        const int lrow = lane / CPR;
+        const int lchunk = (lane % CPR) ^ (lrow & 7);   // RPI is 8 or 4 and q * RPI keeps row & 7 only if RPI == 8
+        auto issue_panel = [&](int i) {
+            const int bj = column(i);
+            const uint32_t dst = lds_base + (uint32_t)((i % NBUF) * PANEL);
+#pragma unroll
+            for (int q = 0; q < NVL; ++q) {
+                const int row = q * RPI + lrow;
+                const int chunk = RPI == 8 ? lchunk : ((lane % CPR) ^ (row & 7));
+                lds_direct_load16(B + ((int64_t)bj * BN + row) * p.b_ld + chunk * 8, dst + q * 1024);
+            }
+        };
+        issue_panel(0);
+        if (n_blk > 1) issue_panel(1);
+        for (int i = 0; i < n_blk; ++i) {
+            // panel i must have landed; panel i + 1 may still be on its way
+            if (i + 1 < n_blk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NVL) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (i + 2 < n_blk) issue_panel(i + 2);   // its buffer was read in step i - 1
+        }
+        return;
+    }
+
+    // ---- compute wavefronts -----------------------------------------------------------------
+    const T* A = reinterpret_cast<const T*>(p.A) + b * p.a_batch;
+    const T* biasT = HAS_BIAS ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
+    T* C = reinterpret_cast<T*>(p.C) + b * p.c_batch;
+    Frag af[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) af[c] = Mma32<T>::load(A + ((int64_t)bi * BM + wave * 16 + r16) * p.a_ld + c * 32 + g4 * 8);
+    const int k_src = r16 * KP, k_sw = r16 & 7;
+    char* const otile = smem + NBUF * PANEL + wave * OT;
+    for (int i = 0; i < n_blk; ++i) {
+        const char* buf = smem + (i % NBUF) * PANEL;
+        __syncthreads();   // panel i is complete
+        uint64_t pieces[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag bf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * KP + (((c * 4 + g4) ^ k_sw) << 4));
+                acc = Mma32<T>::mma(bf, af[c], acc);   // lane: row r16, columns kt * 16 + g4 * 4 .. + 3
+            }
+            if constexpr (HAS_BIAS) {
+                // the lane's four bias entries are 8 contiguous bytes
+                union { uint64_t u; T t[4]; } bv;
+                bv.u = *reinterpret_cast<const uint64_t*>(biasT + column(i) * BN + kt * 16 + g4 * 4);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc[q] += Elem<T>::to_float(bv.t[q]);
+            }
+            T vals[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(acc[q]);
+            pieces[kt] = *reinterpret_cast<const uint64_t*>(vals);
+        }
+        wave_rows_store<BN>(otile, C + (int64_t)(e_begin + i) * (BM * BN) + wave * 16 * BN, pieces);
+    }
+}
+
+template <typename T, int BN, int K, int WAVES>
+static int launch_dds_rowq_inst(const DdsParams& p, int batch, hipStream_t st) {
+    const size_t smem = (size_t)3 * BN * K * 2 + (size_t)WAVES * 16 * (BN * 2 + 16);
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * (p.M / (16 * WAVES));
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_rowq_kernel<T, BN, K, WAVES, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_rowq_kernel<T, BN, K, WAVES, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(dds_rowq_kernel)");
+    }
+    if (p.bias) hipLaunchKernelGGL((dds_rowq_kernel<T, BN, K, WAVES, true>), dim3((unsigned)groups), dim3(64 * (WAVES + 1)), smem, st, p, batch);
+    else hipLaunchKernelGGL((dds_rowq_kernel<T, BN, K, WAVES, false>), dim3((unsigned)groups), dim3(64 * (WAVES + 1)), smem, st, p, batch);
+    SPX_LAUNCH_CHECK("dds_rowq_kernel");
+    return 0;
+}
+
+template <typename T>
+static bool dds_rowq_ok(const DdsParams& p, int BM, int BN) {
+    if constexpr (sizeof(T) != 2) return false;
+    return p.row_ptr && p.a_kcontig && p.b_kcontig && p.compressed && (p.K == 64 || p.K == 128) &&
+           (BM == 32 || BM == 64) && (BN == 32 || BN == 64) && p.a_ld % 8 == 0 && p.b_ld % 8 == 0 &&
+           (!p.bias || (aligned(p.bias, 8) && p.bias_batch % 4 == 0));
+}
+
+template <typename T>
+static int launch_dds_rowq(const DdsParams& p, int BM, int BN, int batch, hipStream_t st) {
+    if constexpr (sizeof(T) == 2) {
+#define SPX_DDS_ROWQ_CASE(bm, bn) \
+        if (BM == bm && BN == bn) return p.K == 64 ? launch_dds_rowq_inst<T, bn, 64, bm / 16>(p, batch, st) \
+                                                   : launch_dds_rowq_inst<T, bn, 128, bm / 16>(p, batch, st);
+        SPX_DDS_ROWQ_CASE(32, 32) SPX_DDS_ROWQ_CASE(32, 64) SPX_DDS_ROWQ_CASE(64, 32) SPX_DDS_ROWQ_CASE(64, 64)
+#undef SPX_DDS_ROWQ_CASE
+    }
+    return fail(SPX_E_CONFIG, "the wavefront-per-16-rows kernel takes 16-bit types and 32 / 64-wide blocks");
+}
+
 // The block-row kernel covers 32 / 64-wide blocks with K * sizeof(T) of 128 or 256 bytes.
 template <typename T>
 static bool dds_row_ok(const DdsParams& p, int BM, int BN) {
@@ -714,10 +877,15 @@ static int launch_dds_inst(const DdsParams& p, int nnz_bound, int batch, hipStre
 //           2 = pipelined (register ring + two LDS buffers).
 template <typename T>
 int launch_dds_impl(const DdsParams& p, int BM, int BN, int nnz_bound, int batch, int tile_cfg, hipStream_t st) {
-    if (tile_cfg < 0 || tile_cfg > 3) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    if (tile_cfg < 0 || tile_cfg > 4) return fail(SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     const int pipe = dds_pipe_ok<T>(p, BM, BN);
     const bool row = dds_row_ok<T>(p, BM, BN);
-    if (tile_cfg == 0) tile_cfg = row ? 3 : (pipe ? 2 : 1);
+    const bool rowq = dds_rowq_ok<T>(p, BM, BN);
+    if (tile_cfg == 0) tile_cfg = rowq ? 4 : (row ? 3 : (pipe ? 2 : 1));
+    if (tile_cfg == 4) {
+        if (!rowq) return fail(SPX_E_CONFIG, "tile config 4 needs a 16-bit type, row_ptr, k-contiguous operands, compressed output, 32/64-wide blocks and K of 64 or 128");
+        return launch_dds_rowq<T>(p, BM, BN, batch, st);
+    }
     if (tile_cfg == 3) {
         if (!row) return fail(SPX_E_CONFIG, "tile config 3 needs row_ptr, k-contiguous operands, 32/64-wide blocks and K of 128 or 256 bytes");
         return launch_dds_row<T>(p, BM, BN, batch, st);

@@ -97,36 +97,46 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
             slot = e;
         }
     };
-    u32x4 sr[NVS], dr[NVD];
-    auto issue = [&](int kb, int64_t slot) {
+    // Index entries of the block-column: lane l holds entry l (broadcast with readlane, so
+    // no step waits for an index load); longer columns read the rest from the index.
+    const int n_blk = e_end - e_begin;
+    int kb_vec = 0, slot_vec = 0;
+    if (lane < n_blk) {
+        int kb0; int64_t slot0;
+        entry(e_begin + lane, kb0, slot0);
+        kb_vec = kb0; slot_vec = (int)slot0;
+    }
+    auto entry_at = [&](int i, int& kb, int64_t& slot) {
+        const int ii = i < n_blk ? i : n_blk - 1;   // steps past the end re-read the last block; the copy is not used
+        if (ii < 64) {
+            kb = __builtin_amdgcn_readlane(kb_vec, ii);
+            slot = __builtin_amdgcn_readlane(slot_vec, ii);
+        } else {
+            entry(e_begin + ii, kb, slot);
+        }
+    };
+    auto issue = [&](int i, u32x4 (&sr)[NVS], u32x4 (&dr)[NVD]) {
+        int kb; int64_t slot;
+        entry_at(i, kb, slot);
         const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN)
                       : ST           ? S + (int64_t)kb * BK * p.s_ld + (int64_t)j * BN
                                      : S + (int64_t)j * BN * p.s_ld + (int64_t)kb * BK;
 #pragma unroll
-        for (int i = 0; i < NVS; ++i) sr[i] = *reinterpret_cast<const u32x4*>(sblk + s_row[i] * sld + s_chunk[i] * 8);
+        for (int i2 = 0; i2 < NVS; ++i2) sr[i2] = *reinterpret_cast<const u32x4*>(sblk + s_row[i2] * sld + s_chunk[i2] * 8);
 #pragma unroll
-        for (int i = 0; i < NVD; ++i)
-            dr[i] = *reinterpret_cast<const u32x4*>(D + ((int64_t)kb * BK + d_row[i]) * p.d_ld + d_chunk[i] * 8);
+        for (int i2 = 0; i2 < NVD; ++i2)
+            dr[i2] = *reinterpret_cast<const u32x4*>(D + ((int64_t)kb * BK + d_row[i2]) * p.d_ld + d_chunk[i2] * 8);
     };
-    // (kb, slot) of the block in the staging registers and of the one after it, fetched a
-    // whole step before its address is needed
-    int kb = 0, kb_next = 0;
-    int64_t slot = 0, slot_next = 0;
-    if (e_begin < e_end) {
-        entry(e_begin, kb, slot);
-        entry(e_begin + 1 < e_end ? e_begin + 1 : e_begin, kb_next, slot_next);
-        issue(kb, slot);
-    }
-    for (int e = e_begin; e < e_end; ++e) {
-        char* buf = smem + ((e - e_begin) & 1) * TILE;
+    // Two register stages: the S block and D tile of step i + 2 are requested while step i is
+    // staged and computed (a block is a dependent HBM round trip; one step of lead left
+    // every step waiting for it).
+    auto step = [&](int i, u32x4 (&sr)[NVS], u32x4 (&dr)[NVD]) {
+        char* buf = smem + (i & 1) * TILE;
 #pragma unroll
-        for (int i = 0; i < NVS; ++i) *reinterpret_cast<u32x4*>(buf + s_dst[i]) = sr[i];
+        for (int i2 = 0; i2 < NVS; ++i2) *reinterpret_cast<u32x4*>(buf + s_dst[i2]) = sr[i2];
 #pragma unroll
-        for (int i = 0; i < NVD; ++i) *reinterpret_cast<u32x4*>(buf + S_BYTES + d_row[i] * VP + d_chunk[i] * 16) = dr[i];
-        // next live block (the last step re-reads its own block; the copy is not used)
-        kb = kb_next; slot = slot_next;
-        entry(e + 2 < e_end ? e + 2 : e_end - 1, kb_next, slot_next);
-        issue(kb, slot);
+        for (int i2 = 0; i2 < NVD; ++i2) *reinterpret_cast<u32x4*>(buf + S_BYTES + d_row[i2] * VP + d_chunk[i2] * 16) = dr[i2];
+        issue(i + 2, sr, dr);
         __syncthreads();   // the tile is complete; everyone is done with the buffer written next
 
 #pragma unroll
@@ -147,6 +157,15 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
                 acc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), sf, acc[t]);
             }
         }
+    };
+    u32x4 s0[NVS], d0[NVD], s1[NVS], d1[NVD];
+    if (n_blk > 0) {
+        issue(0, s0, d0);
+        issue(1, s1, d1);
+    }
+    for (int i = 0; i < n_blk; i += 2) {
+        step(i, s0, d0);
+        if (i + 1 < n_blk) step(i + 1, s1, d1);
     }
 
     // lane holds out[m = t*16 + g4*4 + q][n = j*BN + wave*16 + r16]

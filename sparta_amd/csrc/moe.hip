@@ -511,9 +511,6 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
 // M0), so no registers or LDS-store instructions are spent on staging.  NBUF LDS buffers hold stages s .. s + NBUF - 1; one barrier per
 // stage.  The loads are issued through inline assembly, which keeps the compiler from
 // serialising them against the fragment reads of the other buffers.
-__device__ __forceinline__ void lds_direct_load16(const void* g, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(g) : "memory", "m0");
-}
 
 template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN>
 __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 : 2) void moe_gemm_direct_kernel(MoeParams p) {

@@ -27,6 +27,7 @@ static const spx_tile_cfg kDdsCfgs[] = {
     {1, 0, 0, 4, 1, 16, 7, "block-per-workgroup"},
     {2, 0, 0, 4, 3, 16, 7, "block-per-workgroup-pipelined"},
     {3, 0, 0, 4, 2, 32, 7, "block-row-per-workgroup-short-k"},
+    {4, 0, 0, 4, 2, 32, 6, "wave-per-16-rows-short-k"},
 };
 static const spx_tile_cfg kSoftmaxCfgs[] = {
     {0, 4, 0, 4, 0, 4, 7, "auto"},

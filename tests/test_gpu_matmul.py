@@ -143,18 +143,29 @@ def test_matmul_dds_tile_configs(tile_cfg, K, dtype, blocks, tA, tB, gpu):
              gran=(16, 16), sparsity=0.7, seed=5, tile_cfg=tile_cfg)
 
 
-@pytest.mark.parametrize('tile_cfg', [0, 3])
+@pytest.mark.parametrize('tile_cfg', [0, 3, 4])
 @pytest.mark.parametrize('compressed', [False, True])
 @pytest.mark.parametrize('biased', [False, True])
 @pytest.mark.parametrize('dtype,blocks,K', [(torch.float16, (64, 32, 64), 64), (torch.bfloat16, (32, 32, 64), 128),
                                             (torch.float32, (64, 32, 32), 32), (torch.float16, (32, 32, 32), 128),
-                                            (torch.float32, (32, 32, 64), 64)])
+                                            (torch.float32, (32, 32, 64), 64), (torch.bfloat16, (64, 32, 32), 64)])
 def test_matmul_dds_block_row_kernel(tile_cfg, compressed, biased, dtype, blocks, K, gpu):
     """Sparse-output products whose whole K is one or two stages deep (attention scores):
-    one workgroup walks the live blocks of a block row; rows without a live block, one
+    one workgroup walks the live blocks of a block row (tile config 3, or 4: a wavefront
+    per 16 rows, 16-bit types and compressed output only); rows without a live block, one
     block and many."""
+    if tile_cfg == 4 and (dtype == torch.float32 or not compressed):
+        pytest.skip('tile config 4 takes 16-bit types and the compressed output layout')
     run_case(gpu, 'dds', False, True, biased, compressed, dtype, blocks, batch=3, M=448, K=K, N=320,
              gran=(32, 32), sparsity=0.8, seed=17, tile_cfg=tile_cfg)
+
+
+@pytest.mark.parametrize('blocks', [(64, 32, 64), (32, 32, 32)])
+def test_matmul_dds_block_rows_longer_than_a_wavefront(blocks, gpu):
+    """Block rows with more than 64 live blocks (the column list no longer fits one
+    register of a wavefront) and a batch that does not fill the eight-way numbering."""
+    run_case(gpu, 'dds', False, True, False, True, torch.float16, blocks, batch=11, M=128, K=64, N=blocks[2] * 90,
+             gran=(blocks[0], blocks[2]), sparsity=0.15, seed=23, tile_cfg=4)
 
 
 @pytest.mark.parametrize('tile_cfg', [0, 9])
