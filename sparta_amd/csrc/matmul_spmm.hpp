@@ -252,9 +252,15 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
         // problems are latency-bound and want more, shorter workgroups.
         const int64_t big_tiles = (int64_t)((p.Mc + 255) / 256) * (p.Nc / BN) * batch;
         const bool fill = big_tiles >= 512;
-        // (the persistent form, 10, measures the same as 7 on the 4096^3 problem - 30.4 against
-        // 29.4 - 31.8 us - and is left to tune())
-        if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
+        // the persistent form when its 8 * (N / BN) slots fill the device four times over, every
+        // slot walks at least two 256-row tiles and the block-columns are long: 28.4 - 28.7 us
+        // against 29.9 - 30.0 us for 7 on the 4096^3 problem (alternating runs on three
+        // machines); with fewer slots or tiles it loses (C4 layers: 28 / 34 against 20 / 21 us)
+        const int nb = p.Nc / BN;
+        if (stream_ok && panel_ok && batch == 1 && 8 * nb >= 1024 && p.Mc >= 16 * 256 && p.K / p.BK >= 32 &&
+            (BN == 16 || BN == 32 || BN == 64))
+            tile_cfg = 10;
+        else if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
         else if (ksplit_ok && !fill && p.K / p.BK >= 8) tile_cfg = 8;  // few tiles, long block-columns
         else if (panel7_ok && p.Mc >= 512 && fill) tile_cfg = 7;
         else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
