@@ -538,7 +538,7 @@ static int launch_attention_v2(const AttnParams& p, int batch, int BW, int E, hi
 // P.V MFMAs, so the output needs no final division.  One launch replaces the scores,
 // softmax and P.V operators of the forward pipeline.
 template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(AttnParams p, int nbr, int batch) {
+__global__ __launch_bounds__(64 * (WAVES + 1), 8 / WAVES) void attention_train_kernel(AttnParams p, int nbr, int batch) {
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
     constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
@@ -548,8 +548,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
     constexpr int VPR = E / 8;                // 16-byte vectors per tile row
     constexpr int NV = BW * VPR / NT;         // vectors per thread and tile
     constexpr int RSTEP = NT / VPR;           // tile rows between a thread's vectors
-    constexpr int PP = BW * 2 + 16;           // row pitch of a wave's private 16 x BW probability tile
-    constexpr int PN = BW / 32;               // 16-byte vectors of that tile per lane
+    constexpr int PROW = BW * 2;              // bytes per row of the staged probability tile (chunks XOR-swizzled by the row)
+    constexpr int PCH = BW / 8;               // 16-byte chunks per row
+    constexpr int PTILE = 16 * WAVES * PROW;  // one block of probabilities
     static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
     typedef typename Mma32<T>::frag Frag;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -574,7 +575,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
     T* O = reinterpret_cast<T*>(p.out) + b * (int64_t)p.Nt * E;
     T* P = reinterpret_cast<T*>(p.probs) + b * p.probs_batch;
 
-    const int qrow = br * (16 * WAVES) + wave * 16 + r16;
+    // (the store wavefront, wave == WAVES, owns no rows: it reads the first wavefront's Q rows and drops them)
+    const int qrow = br * (16 * WAVES) + (wave < WAVES ? wave : 0) * 16 + r16;
     const float c2 = p.inv_t * 1.4426950408889634f;
     Frag qf[EC];
 #pragma unroll
@@ -592,15 +594,47 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
     const int k_src = r16 * KP;
     const int k_sw = r16 & 7;
     const int v_src = BW * KP + (g4 * 4 + (r16 >> 2)) * VP + (r16 & 3) * 8;
-    char* ptile = smem + NBUF * TILE + wave * (16 * PP);
-    const int pt_piece = r16 * PP + g4 * 8;
+    char* const pstage = smem + NBUF * TILE;   // [2][PTILE]
+    auto pswz = [](int row) { return row & 7 & (PCH - 1); };
 
     const int e_begin = p.row_ptr[br];
     const int e_end = p.row_ptr[br + 1];
     if (e_begin >= e_end) {
         // no live block: zero output rows (uniform over the workgroup)
+        if (wave < WAVES) {
 #pragma unroll
-        for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = 0ull;
+            for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(O + (int64_t)qrow * E + t * 16 + g4 * 4) = 0ull;
+        }
+        return;
+    }
+    if (wave == WAVES) {
+        // ---- store wavefront: follows the barriers of the others and, one step behind them,
+        // moves every finished block of probabilities from LDS to memory as whole vectors.  It
+        // never loads from memory, and the compute wavefronts never store inside their loops:
+        // loads and stores share one completion counter per wavefront, and a wavefront that
+        // did both waited for its stores whenever it waited for a prefetched tile.
+        for (int e = e_begin; e < e_end; ++e) {   // pass 1
+            if constexpr (NBUF == 1) __syncthreads();
+            __syncthreads();
+        }
+        __syncthreads();
+        auto store_block = [&](int e) {
+            const char* tile = pstage + ((e - e_begin) & 1) * PTILE;
+#pragma unroll
+            for (int i = 0; i < PTILE / 1024; ++i) {
+                const int v = i * 64 + lane;       // vector v of the block: row v / PCH, chunk v % PCH
+                const int row = v / PCH, c = v % PCH;
+                __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(tile + row * PROW + ((c ^ pswz(row)) << 4)),
+                                            reinterpret_cast<u32x4*>(P + (int64_t)e * (16 * WAVES * BW) + v * 8));
+            }
+        };
+        for (int e = e_begin; e < e_end; ++e) {   // pass 2
+            if constexpr (NBUF == 1) __syncthreads();
+            __syncthreads();
+            if (e > e_begin) store_block(e - 1);
+        }
+        __syncthreads();
+        store_block(e_end - 1);
         return;
     }
     u32x4 kr[NV], vr[NV];
@@ -732,18 +766,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
             }
             pf[kp] = AttnPack<T>::pack(pv);
             const s16x8 bits = __builtin_bit_cast(s16x8, pf[kp]);
-            *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp) * 32) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
-            *reinterpret_cast<s16x4*>(ptile + pt_piece + (2 * kp + 1) * 32) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
+            // 16 keys are 32 bytes = two chunks of the row; the lane's four keys are half a chunk
+            char* prow = pstage + ((e - e_begin) & 1) * PTILE + (wave * 16 + r16) * PROW + (g4 & 1) * 8;
+            const int sw = pswz(wave * 16 + r16);
+            *reinterpret_cast<s16x4*>(prow + ((((2 * kp) * 2 + (g4 >> 1)) ^ sw) << 4)) = __builtin_shufflevector(bits, bits, 0, 1, 2, 3);
+            *reinterpret_cast<s16x4*>(prow + ((((2 * kp + 1) * 2 + (g4 >> 1)) ^ sw) << 4)) = __builtin_shufflevector(bits, bits, 4, 5, 6, 7);
         }
-        // The wave's 16 rows of the block are 32 * BW contiguous bytes of P: written as whole
-        // 16-byte vectors out of the wave's private tile (8-byte pieces straight from the
-        // MFMA layout reach memory as partial lines, at half the rate).
-#pragma unroll
-        for (int i = 0; i < PN; ++i) {
-            const int c = i * 64 + lane;
-            *reinterpret_cast<u32x4*>(P + (int64_t)e * (16 * WAVES * BW) + wave * (16 * BW) + c * 8) =
-                *reinterpret_cast<const u32x4*>(ptile + (c / (BW / 8)) * PP + (c % (BW / 8)) * 16);
-        }
+        // (the store wavefront writes this block's probabilities to memory during the next step)
 #pragma unroll
         for (int t = 0; t < ET; ++t) {
 #pragma unroll
@@ -765,8 +794,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
         for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(oacc[t][q]);
         pieces[t] = *reinterpret_cast<const uint64_t*>(vals);
     }
+    __syncthreads();   // the last block of probabilities is staged; the K / V tiles are dead
     if constexpr (WAVES * 16 * (E * 2 + 16) <= NBUF * TILE) {
-        __syncthreads();   // the K / V tiles are dead: their space carries the output tiles
         wave_rows_store<E>(smem + wave * (16 * (E * 2 + 16)), O + (int64_t)(qrow - r16) * E, pieces);
     } else {
 #pragma unroll
@@ -777,7 +806,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_train_kernel(
 template <typename T, int BW, int E, int WAVES>
 static int launch_attention_train_inst(const AttnParams& p, int batch, hipStream_t st) {
     constexpr int TILE = BW * (E * 4 + 32);
-    constexpr size_t smem = (2 * TILE <= 64 * 1024 ? 2 * TILE : TILE) + WAVES * 16 * (BW * 2 + 16);
+    constexpr size_t smem = (2 * TILE <= 64 * 1024 ? 2 * TILE : TILE) + 2 * WAVES * 16 * (BW * 2);   // K / V tiles + two staged blocks of P
     const int nbr = p.Nt / p.BH;
     const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
     if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
@@ -787,14 +816,14 @@ static int launch_attention_train_inst(const AttnParams& p, int batch, hipStream
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
             if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_train_kernel)");
         }
-        hipLaunchKernelGGL((attention_train_kernel<T, BW, E, WAVES, true>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+        hipLaunchKernelGGL((attention_train_kernel<T, BW, E, WAVES, true>), dim3((unsigned)groups), dim3(64 * (WAVES + 1)), smem, st, p, nbr, batch);
     } else {
         if (smem > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_train_kernel<T, BW, E, WAVES, false>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
             if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_train_kernel)");
         }
-        hipLaunchKernelGGL((attention_train_kernel<T, BW, E, WAVES, false>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+        hipLaunchKernelGGL((attention_train_kernel<T, BW, E, WAVES, false>), dim3((unsigned)groups), dim3(64 * (WAVES + 1)), smem, st, p, nbr, batch);
     }
     SPX_LAUNCH_CHECK("attention_train_kernel");
     return 0;
@@ -916,7 +945,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
     if (e_begin < e_end) {
 #pragma unroll
         for (int i = 0; i < PN; ++i)
-            pr[i] = *reinterpret_cast<const u32x4*>(P + (int64_t)e_begin * (16 * WAVES * BW) + wave_off + i * 512);
+            pr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P + (int64_t)e_begin * (16 * WAVES * BW) + wave_off + i * 512));   // P is read once
         bc = p.bcsr_idx[e_begin] & 0xffff;
         bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
         const int64_t off = (int64_t)bc * BW * E;
@@ -940,7 +969,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
         {
 #pragma unroll
             for (int i = 0; i < PN; ++i)
-                pr[i] = *reinterpret_cast<const u32x4*>(P + (int64_t)e_next * (16 * WAVES * BW) + wave_off + i * 512);
+                pr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P + (int64_t)e_next * (16 * WAVES * BW) + wave_off + i * 512));
             const int64_t off = (int64_t)bc * BW * E;
 #pragma unroll
             for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
@@ -1148,7 +1177,8 @@ __global__ __launch_bounds__(64 * WAVES, (BH * E <= 64 * 64 || BH == 32) ? 3 : (
 #pragma unroll
         for (int i = 0; i < NVD; ++i) q_r[i] = *reinterpret_cast<const u32x4*>(Q + off + i * NT * 8);
 #pragma unroll
-        for (int i = 0; i < NVP; ++i) p_r[i] = *reinterpret_cast<const u32x4*>(P + pos * (int64_t)(BH * BW) + i * NT * 8);
+        for (int i = 0; i < NVP; ++i)   // P is read once: no need to keep it in L2
+            p_r[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P + pos * (int64_t)(BH * BW) + i * NT * 8));
 #pragma unroll
         for (int t = 0; t < QT; ++t) d_r[t] = *reinterpret_cast<const f32x4*>(Dv + qb * BH + t * 16);
     };

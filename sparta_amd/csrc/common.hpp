@@ -159,8 +159,8 @@ __device__ __forceinline__ void wave_rows_store(char* tile, void* dst, const uin
 #pragma unroll
     for (int i = 0; i < W / 32; ++i) {
         const int c = i * 64 + lane;
-        *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst) + c * 16) =
-            *reinterpret_cast<const u32x4*>(tile + (c / (W / 8)) * PP + (c % (W / 8)) * 16);
+        __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(tile + (c / (W / 8)) * PP + (c % (W / 8)) * 16),
+                                    reinterpret_cast<u32x4*>(reinterpret_cast<char*>(dst) + c * 16));
     }
 }
 
@@ -169,6 +169,18 @@ __device__ __forceinline__ void wave_rows_store(char* tile, void* dst, const uin
 // (a wave-uniform LDS byte address, passed in M0).  Counted by vmcnt like any other load.
 __device__ __forceinline__ void lds_direct_load16(const void* g, uint32_t lds_wave_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(g) : "memory", "m0");
+}
+
+// 16-byte accesses for data that is streamed once: the non-temporal hint keeps it from
+// displacing operands that other workgroups re-read from L2.
+__device__ __forceinline__ vec16 load16_stream(const void* p) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return vec16{v.x, v.y, v.z, v.w};
+}
+__device__ __forceinline__ void store16_stream(void* p, const vec16& v) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4*>(p));
 }
 
 }  // namespace spx

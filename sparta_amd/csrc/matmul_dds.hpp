@@ -117,7 +117,7 @@ __device__ __forceinline__ void dds_epilogue(const DdsParams& p, const Acc& acc,
         for (int e = 0; e < VE; ++e) u.t[e] = Elem<T>::from_float(s[e]);
         const int64_t off = p.compressed ? (int64_t)i * (BM * BN) + m * BN + n
                                          : ((int64_t)bi * BM + m) * p.N + (int64_t)bj * BN + n;
-        *reinterpret_cast<vec16*>(C + off) = u.q;
+        store16_stream(C + off, u.q);   // written once: leave the operand panels in L2
     }
 }
 

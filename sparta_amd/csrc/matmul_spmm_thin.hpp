@@ -122,7 +122,8 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
                       : ST           ? S + (int64_t)kb * BK * p.s_ld + (int64_t)j * BN
                                      : S + (int64_t)j * BN * p.s_ld + (int64_t)kb * BK;
 #pragma unroll
-        for (int i2 = 0; i2 < NVS; ++i2) sr[i2] = *reinterpret_cast<const u32x4*>(sblk + s_row[i2] * sld + s_chunk[i2] * 8);
+        for (int i2 = 0; i2 < NVS; ++i2)   // read once: do not displace the D tiles from L2
+            sr[i2] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sblk + s_row[i2] * sld + s_chunk[i2] * 8));
 #pragma unroll
         for (int i2 = 0; i2 < NVD; ++i2)
             dr[i2] = *reinterpret_cast<const u32x4*>(D + ((int64_t)kb * BK + d_row[i2]) * p.d_ld + d_chunk[i2] * 8);

@@ -291,8 +291,8 @@ __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParam
         if (v < nvec) {
             offs[t] = vector_offset<VE>(p, rv, v, log_vpb);
             if constexpr (HAS_MASK) live[t] = mask_at(offs[t]);
-            SmVec<T>::unpack(*reinterpret_cast<const vec16*>(x + offs[t]), cache[t]);
-            if (BACKWARD) SmVec<T>::unpack(*reinterpret_cast<const vec16*>(yin + offs[t]), ycache[t]);
+            SmVec<T>::unpack(load16_stream(x + offs[t]), cache[t]);
+            if (BACKWARD) SmVec<T>::unpack(load16_stream(yin + offs[t]), ycache[t]);
         }
     }
     if (!BACKWARD) {
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParam
             if (lane + LPR * t < nvec) {
 #pragma unroll
                 for (int i = 0; i < VE; ++i) cache[t][i] *= inv;
-                *reinterpret_cast<vec16*>(out + offs[t]) = SmVec<T>::pack(cache[t]);
+                store16_stream(out + offs[t], SmVec<T>::pack(cache[t]));
             }
         }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
@@ -394,7 +394,7 @@ __global__ __launch_bounds__(64 * SMV_ROWS) void softmax_vec_kernel(SoftmaxParam
             if (lane + LPR * t < nvec) {
 #pragma unroll
                 for (int i = 0; i < VE; ++i) cache[t][i] = p.inv_t * (cache[t][i] - ycache[t][i] * dot);
-                *reinterpret_cast<vec16*>(out + offs[t]) = SmVec<T>::pack(cache[t]);
+                store16_stream(out + offs[t], SmVec<T>::pack(cache[t]));
             }
         }
         for (int v = lane + LPR * SMV_CACHE; v < nvec; v += LPR) {
