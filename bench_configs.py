@@ -71,15 +71,22 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
     cfg32 = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32}
     with torch.no_grad():
         if 'ceilings' in todo:
-            # What plain streaming kernels (torch's own) reach on this machine, for reading the
+            # What plain streaming kernels (the library's probe and torch's own) reach on this machine, for reading the
             # HBM fractions of the memory-bound kernels: a read-only reduction, a write-only
             # fill and a copy, each over 1 GiB (four times the last-level cache).
             n = 1 << 28
             src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
             dst = torch.empty_like(src)
-            for name, fn, nbytes in (('ceiling: read-only torch.sum over 1 GiB', lambda: torch.sum(src), 4 * n),
-                                     ('ceiling: write-only fill of 1 GiB', lambda: dst.fill_(1.0), 4 * n),
-                                     ('ceiling: copy of 1 GiB (read + write)', lambda: dst.copy_(src), 8 * n)):
+            from sparta_amd import _lib
+            lib = _lib.load()
+            def probe(mode):
+                return lambda: _lib.check(lib.spx_stream_probe(mode, _lib.dev_ptr(src), _lib.dev_ptr(dst), 4 * n,
+                                                               _lib.current_stream(dev)), 'spx_stream_probe')
+            for name, fn, nbytes in (('ceiling: read-only pass over 1 GiB (16-byte non-temporal loads)', probe(0), 4 * n),
+                                     ('ceiling: read-only torch.sum over 1 GiB', lambda: torch.sum(src), 4 * n),
+                                     ('ceiling: write-only fill of 1 GiB (torch)', lambda: dst.fill_(1.0), 4 * n),
+                                     ('ceiling: copy of 1 GiB (16-byte non-temporal loads and stores)', probe(1), 8 * n),
+                                     ('ceiling: copy of 1 GiB (torch)', lambda: dst.copy_(src), 8 * n)):
                 _emit(name, timed(fn), bytes_alg=nbytes)
             del src, dst
         if 'c1' in todo:

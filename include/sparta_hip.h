@@ -58,6 +58,12 @@ typedef void* spx_stream_t; /* hipStream_t */
 const char* spx_last_error(void);
 int spx_version(void);
 
+/* Diagnostic, no counterpart in the reference: a plain streaming pass over `bytes` bytes
+ * with the access shape of the memory-bound kernels (16 bytes per lane, non-temporal) -
+ * mode 0 reads src (dst may be NULL), mode 1 copies src to dst.  bench.py --config ceilings
+ * times it to show which read and copy rates the machine sustains. */
+int spx_stream_probe(int mode, const void* src, void* dst, size_t bytes, spx_stream_t stream);
+
 /* ------------------------------------------------------------------------ *
  * BCSR / BCSC index build.
  * Replaces BCSFunctionContext.build_indexes / _build_BCSR_indexes /

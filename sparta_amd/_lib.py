@@ -37,6 +37,7 @@ _P, _I, _L, _F, _Z = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float, _c.c_size_t
 _SIGNATURES = {
     'spx_last_error': (_c.c_char_p, []),
     'spx_version': (_I, []),
+    'spx_stream_probe': (_I, [_I, _P, _P, _Z, _P]),
     'spx_bcs_index_workspace_bytes': (_Z, [_I, _I, _I, _I]),
     'spx_bcs_index': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P, _Z, _P]),
     'spx_bcs_index_scheduled': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _Z, _P]),
