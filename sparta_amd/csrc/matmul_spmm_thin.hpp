@@ -115,6 +115,11 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
             entry(e_begin + ii, kb, slot);
         }
     };
+    // The loads of the two register stages are issued through inline assembly and waited for
+    // with explicit counts: the compiler merges its own wait counts at the loop header and
+    // then drains every outstanding load at each step, which is exactly the lead the second
+    // stage is there to provide.  (S is read once: non-temporal, it must not displace the D
+    // tiles from L2.)
     auto issue = [&](int i, u32x4 (&sr)[NVS], u32x4 (&dr)[NVD]) {
         int kb; int64_t slot;
         entry_at(i, kb, slot);
@@ -122,22 +127,33 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
                       : ST           ? S + (int64_t)kb * BK * p.s_ld + (int64_t)j * BN
                                      : S + (int64_t)j * BN * p.s_ld + (int64_t)kb * BK;
 #pragma unroll
-        for (int i2 = 0; i2 < NVS; ++i2)   // read once: do not displace the D tiles from L2
-            sr[i2] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sblk + s_row[i2] * sld + s_chunk[i2] * 8));
+        for (int i2 = 0; i2 < NVS; ++i2)
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(sr[i2]) : "v"(sblk + s_row[i2] * sld + s_chunk[i2] * 8) : "memory");
 #pragma unroll
         for (int i2 = 0; i2 < NVD; ++i2)
-            dr[i2] = *reinterpret_cast<const u32x4*>(D + ((int64_t)kb * BK + d_row[i2]) * p.d_ld + d_chunk[i2] * 8);
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dr[i2]) : "v"(D + ((int64_t)kb * BK + d_row[i2]) * p.d_ld + d_chunk[i2] * 8) : "memory");
+    };
+    // wait until at most `newer` loads issued after this stage's are still outstanding; the
+    // stage's registers pass through the statement so that no use is scheduled before it
+    auto wait_stage = [&](u32x4 (&sr)[NVS], u32x4 (&dr)[NVD], bool other_in_flight) {
+        if (other_in_flight) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NVS + NVD) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i2 = 0; i2 < NVS; ++i2) asm volatile("" : "+v"(sr[i2]));
+#pragma unroll
+        for (int i2 = 0; i2 < NVD; ++i2) asm volatile("" : "+v"(dr[i2]));
     };
     // Two register stages: the S block and D tile of step i + 2 are requested while step i is
     // staged and computed (a block is a dependent HBM round trip; one step of lead left
     // every step waiting for it).
     auto step = [&](int i, u32x4 (&sr)[NVS], u32x4 (&dr)[NVD]) {
         char* buf = smem + (i & 1) * TILE;
+        wait_stage(sr, dr, i + 1 < n_blk);   // the other stage (step i + 1) may still be on its way
 #pragma unroll
         for (int i2 = 0; i2 < NVS; ++i2) *reinterpret_cast<u32x4*>(buf + s_dst[i2]) = sr[i2];
 #pragma unroll
         for (int i2 = 0; i2 < NVD; ++i2) *reinterpret_cast<u32x4*>(buf + S_BYTES + d_row[i2] * VP + d_chunk[i2] * 16) = dr[i2];
-        issue(i + 2, sr, dr);
+        if (i + 2 < n_blk) issue(i + 2, sr, dr);
         __syncthreads();   // the tile is complete; everyone is done with the buffer written next
 
 #pragma unroll
@@ -162,7 +178,7 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
     u32x4 s0[NVS], d0[NVD], s1[NVS], d1[NVD];
     if (n_blk > 0) {
         issue(0, s0, d0);
-        issue(1, s1, d1);
+        if (n_blk > 1) issue(1, s1, d1);
     }
     for (int i = 0; i < n_blk; i += 2) {
         step(i, s0, d0);
