@@ -6,9 +6,11 @@ linked into ``sparta_amd/lib/libsparta_hip.so``.  Run as
 """
 import concurrent.futures
 import os
+import re
 import shutil
 import subprocess
 import sys
+import tempfile
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(ROOT, 'csrc')
@@ -30,6 +32,104 @@ def _hipcc() -> str:
     return exe
 
 
+# Kernels that prefetch into registers through inline assembly (``global_load_dwordx4 %0``
+# with an explicit ``s_waitcnt vmcnt(N)`` later) rely on the compiler not touching those
+# registers while the loads are in flight.  Nothing in the language promises that: a copy
+# the register allocator inserts, or a spill, would read them before the data has arrived.
+# Translation units with such loads are therefore compiled with their device assembly kept,
+# and the assembly is checked.
+_ASM_LOAD_MARK = 'global_load_dwordx4 %0'
+
+
+def _has_register_prefetch(src: str) -> bool:
+    text = open(src).read()
+    if _ASM_LOAD_MARK in text:
+        return True
+    for name in re.findall(r'#include "([^"]+)"', text):
+        header = os.path.join(CSRC, name)
+        if os.path.exists(header) and _ASM_LOAD_MARK in open(header).read():
+            return True
+    return False
+
+
+def _registers(token: str) -> set:
+    m = re.match(r'v\[(\d+):(\d+)\]$', token)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r'v(\d+)$', token)
+    return {int(m.group(1))} if m else set()
+
+
+def check_inflight_registers(asm: str) -> list:
+    """Scan device assembly for compiler-generated instructions that touch a VGPR between the
+    inline-assembly load that targets it and the inline-assembly wait that covers it.
+
+    The text of each kernel is walked in order.  An inline ``global_load_dwordx4`` makes its
+    destination registers pending; an inline ``s_waitcnt vmcnt(N)`` leaves the N newest loads
+    pending (loads complete in order); a compiler ``s_waitcnt vmcnt(0)``, an unconditional
+    branch or the end of the kernel clears the state (what follows in the text is not what
+    runs next).  Returns a list of (kernel, line number, instruction).
+    """
+    findings = []
+    kernel, pending, in_asm = None, [], False
+    for number, line in enumerate(asm.split('\n'), 1):
+        m = re.match(r'^(_Z\w+):', line)
+        if m:
+            kernel, pending = m.group(1), []
+            continue
+        text = line.strip()
+        if kernel is None or not text or text[0] in '.;' and not text.startswith(';;#ASM'):
+            continue
+        if text.startswith(';;#ASMSTART'):
+            in_asm = True
+            continue
+        if text.startswith(';;#ASMEND'):
+            in_asm = False
+            continue
+        if in_asm:
+            if text.startswith('global_load_dwordx4'):
+                pending.append(_registers(text.split()[1].rstrip(',')))
+            elif text.startswith('s_waitcnt') and 'vmcnt' in text:
+                n = int(re.search(r'vmcnt\((\d+)\)', text).group(1))
+                pending = pending[len(pending) - n:] if n else []
+            continue
+        if text.startswith('s_endpgm'):
+            kernel = None
+            continue
+        if text.startswith(('s_branch', 's_setpc')) or (text.startswith('s_waitcnt') and 'vmcnt(0)' in text):
+            pending = []
+            continue
+        if not pending:
+            continue
+        used = set()
+        for token in re.findall(r'v\[\d+:\d+\]|v\d+', text):
+            used |= _registers(token)
+        if used & set().union(*pending):
+            findings.append((kernel, number, text))
+    return findings
+
+
+def _compile_checked(src: str, obj: str) -> None:
+    """Compile with the intermediate files kept (in a scratch directory) and check the device
+    assembly the object was assembled from."""
+    with tempfile.TemporaryDirectory() as tmp:
+        cmd = [_hipcc(), *HIPCC_FLAGS, '-save-temps=cwd', '-c', src, '-o', obj]
+        proc = subprocess.run(cmd, capture_output=True, text=True, cwd=tmp)
+        if proc.returncode != 0:
+            raise RuntimeError(f'hipcc failed on {src}:\n{proc.stderr}')
+        listings = [f for f in os.listdir(tmp) if f.endswith('.s') and 'amdgcn' in f]
+        if not listings:
+            raise RuntimeError(f'no device assembly was kept for {src}; the register prefetch cannot be checked')
+        for name in listings:
+            findings = check_inflight_registers(open(os.path.join(tmp, name)).read())
+            if findings:
+                os.remove(obj)
+                shown = '\n'.join(f'  {k}: line {n}: {t}' for k, n, t in findings[:20])
+                raise RuntimeError(
+                    f'{src}: the compiler touches registers that inline-assembly loads are still filling '
+                    f'({len(findings)} instructions); restructure the prefetch or lower the register pressure:\n{shown}')
+
+
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(OBJ, os.path.basename(src)[:-4] + '.o')
     if not force and os.path.exists(obj):
@@ -39,6 +139,9 @@ def _compile(src: str, force: bool) -> str:
                         for f in os.listdir(d) if f.endswith(('.hpp', '.h'))]
         if os.path.getmtime(obj) >= max(os.path.getmtime(d) for d in deps):
             return obj
+    if _has_register_prefetch(src):
+        _compile_checked(src, obj)
+        return obj
     cmd = [_hipcc(), *HIPCC_FLAGS, '-c', src, '-o', obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:

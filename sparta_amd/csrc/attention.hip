@@ -854,8 +854,19 @@ static int launch_attention_train(const AttnParams& p, int batch, int BW, int E,
 // layout of P and fed to the dQ MFMAs.  Masked entries have P = 0 and so dS = 0: no mask is
 // needed.  dK and dV stay with the sparse-operand matmul kernels (dK = dS^T Q, dV = P^T dO).
 // Replaces three launches of the operator pipeline's backward (dP, softmax backward, dQ).
+// Wavefronts per SIMD the register budget is sized for: no more than the LDS footprint lets
+// a CU hold (two-wavefront workgroups with large tiles spilled under the budget of four).
+template <int BW, int E, int WAVES>
+constexpr int bwd_row_waves_per_simd() {
+    constexpr int TILE = BW * (E * 4 + 32);
+    constexpr int smem = (2 * TILE <= 64 * 1024 ? 2 * TILE : TILE) + WAVES * 16 * (BW * 2 + 16);
+    constexpr int by_lds = (160 * 1024 / smem * WAVES + 3) / 4;
+    constexpr int cap = 8 / WAVES;
+    return by_lds < 1 ? 1 : (by_lds < cap ? by_lds : cap);
+}
+
 template <typename T, int BW, int E, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kernel(AttnParams p, int nbr, int batch) {
+__global__ __launch_bounds__(64 * WAVES, (bwd_row_waves_per_simd<BW, E, WAVES>())) void attention_bwd_row_kernel(AttnParams p, int nbr, int batch) {
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
     constexpr int RP = E * 2;                 // pitch of the row-read tile (V): 16-byte chunks XOR-swizzled by row % 8
@@ -867,6 +878,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
     constexpr int RSTEP = NT / VPR;
     constexpr int PP = BW * 2 + 16;           // row pitch of a wave's private 16 x BW probability tile
     constexpr int PN = BW / 32;               // 16-byte vectors of that tile per lane
+    constexpr int NSTG = (PN + 2 * NV) * 4 <= 48 ? 2 : 1;   // register stages of the prefetch
     static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
     typedef typename Mma32<T>::frag Frag;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -939,43 +951,68 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
     const int64_t wave_off = (int64_t)wave * (16 * BW) + lane * 8;   // elements, inside a block
 
     const int e_begin = p.row_ptr[br];
-    const int e_end = p.row_ptr[br + 1];
-    u32x4 kr[NV], vr[NV], pr[PN];
-    int bc = 0, bc_next = 0;   // the entry after next is fetched a whole step before its address is needed
-    if (e_begin < e_end) {
+    const int n_blk = p.row_ptr[br + 1] - e_begin;
+    // Block columns of the row: lane l holds entry l (broadcast with readlane, so no step
+    // waits for an index load); longer rows read the rest from the index.
+    int bc_vec = 0;
+    if (lane < n_blk) bc_vec = p.bcsr_idx[e_begin + lane] & 0xffff;
+    auto col_at = [&](int i) {
+        return i < 64 ? __builtin_amdgcn_readlane(bc_vec, i) : (p.bcsr_idx[e_begin + i] & 0xffff);
+    };
+    // Two register stages: the P block and the K / V tiles of step i + 2 are requested while
+    // step i is staged and computed.  A step's MFMA work is a fraction of a memory round
+    // trip, so one step of lead left every step waiting.  The loads go through inline
+    // assembly and are waited for with explicit counts: the compiler merges its own wait
+    // counts at the loop header and would drain both stages at every step.  (Shapes whose
+    // tiles take more than 48 registers per thread keep one stage of ordinary loads.)
+    auto issue = [&](int i, u32x4 (&pr)[PN], u32x4 (&vr)[NV], u32x4 (&kr)[NV]) {
+        const int64_t off = (int64_t)col_at(i) * BW * E;
+        const T* pblk = P + (int64_t)(e_begin + i) * (16 * WAVES * BW) + wave_off;
+        if constexpr (NSTG == 2) {
 #pragma unroll
-        for (int i = 0; i < PN; ++i)
-            pr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P + (int64_t)e_begin * (16 * WAVES * BW) + wave_off + i * 512));   // P is read once
-        bc = p.bcsr_idx[e_begin] & 0xffff;
-        bc_next = p.bcsr_idx[e_begin + 1 < e_end ? e_begin + 1 : e_begin] & 0xffff;
-        const int64_t off = (int64_t)bc * BW * E;
+            for (int i2 = 0; i2 < PN; ++i2)   // P is read once: non-temporal
+                asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(pr[i2]) : "v"(pblk + i2 * 512) : "memory");
 #pragma unroll
-        for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+            for (int i2 = 0; i2 < NV; ++i2)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(vr[i2]) : "v"(Vg + off + i2 * NT * 8) : "memory");
 #pragma unroll
-        for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
-    }
-    for (int e = e_begin; e < e_end; ++e) {
-        char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
-        if constexpr (NBUF == 1) __syncthreads();
+            for (int i2 = 0; i2 < NV; ++i2)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kr[i2]) : "v"(Kg + off + i2 * NT * 8) : "memory");
+        } else {
 #pragma unroll
-        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + r_dst + i * RSTEP * RP) = vr[i];
+            for (int i2 = 0; i2 < PN; ++i2) pr[i2] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(pblk + i2 * 512));
 #pragma unroll
-        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + t_dst + i * RSTEP * TP) = kr[i];
+            for (int i2 = 0; i2 < NV; ++i2) vr[i2] = *reinterpret_cast<const u32x4*>(Vg + off + i2 * NT * 8);
 #pragma unroll
-        for (int i = 0; i < PN; ++i) *reinterpret_cast<u32x4*>(ptile + pt_vec[i]) = pr[i];
-        const int e_next = e + 1 < e_end ? e + 1 : e;
-        bc = bc_next;
-        bc_next = p.bcsr_idx[e + 2 < e_end ? e + 2 : e_end - 1] & 0xffff;
-        {
-#pragma unroll
-            for (int i = 0; i < PN; ++i)
-                pr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P + (int64_t)e_next * (16 * WAVES * BW) + wave_off + i * 512));
-            const int64_t off = (int64_t)bc * BW * E;
-#pragma unroll
-            for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
-#pragma unroll
-            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+            for (int i2 = 0; i2 < NV; ++i2) kr[i2] = *reinterpret_cast<const u32x4*>(Kg + off + i2 * NT * 8);
         }
+    };
+    // Wait until only the other stage is outstanding; the stage's registers pass through the
+    // statement so that no use is scheduled before it.  With dS stored everything is drained:
+    // stores share the counter and need not complete in order with the loads.
+    auto wait_stage = [&](int i, u32x4 (&pr)[PN], u32x4 (&vr)[NV], u32x4 (&kr)[NV]) {
+        if constexpr (NSTG == 1) return;   // plain loads: the compiler waits where the registers are used
+        if (i + 1 < n_blk && !store_ds) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PN + 2 * NV) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i2 = 0; i2 < PN; ++i2) asm volatile("" : "+v"(pr[i2]));
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) asm volatile("" : "+v"(vr[i2]));
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) asm volatile("" : "+v"(kr[i2]));
+    };
+    auto step = [&](int i, u32x4 (&pr)[PN], u32x4 (&vr)[NV], u32x4 (&kr)[NV]) {
+        const int e = e_begin + i;
+        char* buf = smem + (NBUF == 2 ? (i & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();
+        wait_stage(i, pr, vr, kr);
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) *reinterpret_cast<u32x4*>(buf + r_dst + i2 * RSTEP * RP) = vr[i2];
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) *reinterpret_cast<u32x4*>(buf + t_dst + i2 * RSTEP * TP) = kr[i2];
+#pragma unroll
+        for (int i2 = 0; i2 < PN; ++i2) *reinterpret_cast<u32x4*>(ptile + pt_vec[i2]) = pr[i2];
+        if (i + NSTG < n_blk) issue(i + NSTG, pr, vr, kr);
         __syncthreads();
 
         // ---- (dP - D)^T / T tiles: keys x this wave's 16 queries -----------------------------
@@ -1011,9 +1048,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
         }
         if (store_ds) {
 #pragma unroll
-            for (int i = 0; i < PN; ++i)
-                *reinterpret_cast<u32x4*>(dS + (int64_t)e * (16 * WAVES * BW) + wave_off + i * 512) =
-                    *reinterpret_cast<const u32x4*>(ptile + pt_vec[i]);
+            for (int i2 = 0; i2 < PN; ++i2)
+                *reinterpret_cast<u32x4*>(dS + (int64_t)e * (16 * WAVES * BW) + wave_off + i2 * 512) =
+                    *reinterpret_cast<const u32x4*>(ptile + pt_vec[i2]);
         }
         // ---- dQ^T[e][query] += K^T dS^T ------------------------------------------------------
 #pragma unroll
@@ -1028,6 +1065,21 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_bwd_row_kerne
                 qacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), sf[kp], qacc[t]);
             }
         }
+    };
+    if constexpr (NSTG == 2) {
+        u32x4 p0[PN], v0[NV], k0[NV], p1[PN], v1[NV], k1[NV];
+        if (n_blk > 0) {
+            issue(0, p0, v0, k0);
+            issue(n_blk > 1 ? 1 : 0, p1, v1, k1);   // a row of one block requests it twice; the copy is not used
+        }
+        for (int i = 0; i < n_blk; i += 2) {
+            step(i, p0, v0, k0);
+            if (i + 1 < n_blk) step(i + 1, p1, v1, k1);
+        }
+    } else {
+        u32x4 p0[PN], v0[NV], k0[NV];
+        if (n_blk > 0) issue(0, p0, v0, k0);
+        for (int i = 0; i < n_blk; ++i) step(i, p0, v0, k0);
     }
     uint64_t pieces[ET];
 #pragma unroll

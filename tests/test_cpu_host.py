@@ -327,3 +327,39 @@ def test_packaged_config_tables_cover_the_sweep(op, kernels):
             for params in config.values():
                 assert params['_impl'] in ('sparta', 'openai')
                 assert all(isinstance(v, int) and v > 0 for k, v in params.items() if k != '_impl')
+
+
+def _listing(body):
+    return '_Z6kernelv:\n' + body + '\ts_endpgm\n'
+
+
+def _asm(*lines):
+    return '\t;;#ASMSTART\n' + ''.join(f'\t{line}\n' for line in lines) + '\t;;#ASMEND\n'
+
+
+def test_build_check_finds_registers_touched_while_loads_are_in_flight():
+    """The build scans the device assembly of kernels that prefetch through inline-assembly
+    loads: a compiler instruction that touches a destination register before the explicit
+    wait that covers it is reported, everything after the wait is not."""
+    from sparta_amd.build import check_inflight_registers
+    load_a = _asm('global_load_dwordx4 v[2:5], v[10:11], off nt')
+    load_b = _asm('global_load_dwordx4 v[6:9], v[12:13], off')
+    # a copy right after the load is issued (what the register allocator did once)
+    found = check_inflight_registers(_listing(load_a + '\tv_mov_b32_e32 v20, v3\n'))
+    assert [(k, t) for k, _, t in found] == [('_Z6kernelv', 'v_mov_b32_e32 v20, v3')]
+    # a spill of a pending register
+    assert check_inflight_registers(_listing(load_a + '\tscratch_store_dwordx4 off, v[2:5], off offset:16\n'))
+    # overwriting a pending register is just as wrong
+    assert check_inflight_registers(_listing(load_a + '\tv_accvgpr_read_b32 v4, a0\n'))
+    # the wait covers it
+    assert check_inflight_registers(_listing(load_a + _asm('s_waitcnt vmcnt(0)') + '\tds_write_b128 v30, v[2:5]\n')) == []
+    # vmcnt(1) leaves the newer load pending: the older registers are free, the newer are not
+    two = load_a + load_b + _asm('s_waitcnt vmcnt(1)')
+    assert check_inflight_registers(_listing(two + '\tds_write_b128 v30, v[2:5]\n')) == []
+    assert len(check_inflight_registers(_listing(two + '\tds_write_b128 v30, v[6:9]\n'))) == 1
+    # registers that are not pending, and the address registers of the load, may be used
+    assert check_inflight_registers(_listing(load_a + '\tv_add_u32_e32 v10, 4, v10\n\tv_mov_b32_e32 v21, v22\n')) == []
+    # text after an unconditional branch is another path
+    assert check_inflight_registers(_listing(load_a + '\ts_branch .LBB0_2\n.LBB0_1:\n\tv_mov_b32_e32 v2, 0\n')) == []
+    # a new kernel starts clean
+    assert check_inflight_registers(_listing(load_a) + '_Z6otherv:\n\tv_mov_b32_e32 v2, 0\n\ts_endpgm\n') == []
