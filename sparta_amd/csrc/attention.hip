@@ -247,11 +247,20 @@ __device__ __forceinline__ float lane_max(const f32x4 (&s)[KT]) {
     return fmaxf(m, s[KT - 1][3]);
 }
 
+// Wavefronts per SIMD a kernel's register budget is sized for: no more than its LDS footprint
+// lets a CU hold, and no more than eight wavefronts per SIMD-quarter of the workgroup
+// (two-wavefront workgroups with large tiles spilled under a budget of four).
+constexpr int waves_per_simd_for(int smem_bytes, int waves, int cap = 0) {
+    const int by_lds = (160 * 1024 / smem_bytes * waves + 3) / 4;
+    if (cap == 0) cap = 8 / waves;
+    return by_lds < 1 ? 1 : (by_lds < cap ? by_lds : cap);
+}
+
 // SEQ: no index and no mask bytes; entry b attends over its first L = seqlens[b / heads]
 // positions: the walk covers the key blocks below L, a key is live iff its position is, and
 // queries at or past L give zeros (block rows at or past L walk nothing).
 template <typename T, int BW, int E, int WAVES, bool HAS_MASK, bool SEQ = false>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(AttnParams p, int nbr, int batch) {
+__global__ __launch_bounds__(64 * WAVES, waves_per_simd_for((2 * BW * (E * 4 + 32) <= 64 * 1024 ? 2 : 1) * BW * (E * 4 + 32), WAVES)) void attention_kernel_v2(AttnParams p, int nbr, int batch) {
     static_assert(!SEQ || HAS_MASK, "the sequence-length mode masks by key position");
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
@@ -329,49 +338,70 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
         seq_len = seq_len < 0 ? 0 : (seq_len > p.Ns ? p.Ns : seq_len);
     }
     const int e_begin = SEQ ? 0 : p.row_ptr[br];
-    const int e_end = SEQ ? (br * (16 * WAVES) < seq_len ? (seq_len + BW - 1) / BW : 0) : p.row_ptr[br + 1];
-    auto column = [&](int e) { return SEQ ? e : (p.bcsr_idx[e] & 0xffff); };
-    u32x4 kr[NV], vr[NV];
-    // bc: block column of the tile in the staging registers; bc_next: the one after it, fetched
-    // a whole step before its address is needed (the wait for an index entry that is used at
-    // once would stall every step for an L2 round trip)
-    int bc = 0, bc_next = 0;
-    if (e_begin < e_end) {
-        bc = column(e_begin);
-        bc_next = column(e_begin + 1 < e_end ? e_begin + 1 : e_begin);
-        const int64_t off = (int64_t)bc * BW * E;
-#pragma unroll
-        for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
-#pragma unroll
-        for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+    const int n_blk = (SEQ ? (br * (16 * WAVES) < seq_len ? (seq_len + BW - 1) / BW : 0) : p.row_ptr[br + 1]) - e_begin;
+    // Block columns of the row: lane l holds entry l (broadcast with readlane, so no step
+    // waits for an index load); longer rows read the rest from the index.
+    int bc_vec = 0;
+    if constexpr (!SEQ) {
+        if (lane < n_blk) bc_vec = p.bcsr_idx[e_begin + lane] & 0xffff;
     }
-    for (int e = e_begin; e < e_end; ++e) {
-        char* buf = smem + (NBUF == 2 ? ((e - e_begin) & 1) * TILE : 0);
-        if constexpr (NBUF == 1) __syncthreads();  // the previous block's fragments are consumed
+    auto col_at = [&](int i) {
+        if constexpr (SEQ) return i;
+        else return i < 64 ? __builtin_amdgcn_readlane(bc_vec, i) : (p.bcsr_idx[e_begin + i] & 0xffff);
+    };
+    // Without mask bytes to fetch, two register stages: the K and V tiles of step i + 2 are
+    // requested while step i is staged and computed, through inline-assembly loads that are
+    // waited for with explicit counts (the compiler merges its own wait counts at the loop
+    // header and would drain both stages at every step).  With a mask, one stage of ordinary
+    // loads: the wait for the mask bytes would drain the second stage anyway.
+    constexpr int NSTG = (!HAS_MASK && !SEQ && NV <= 4) ? 2 : 1;
+    auto issue = [&](int i, u32x4 (&kr)[NV], u32x4 (&vr)[NV]) {
+        const int64_t off = (int64_t)col_at(i) * BW * E;
+        if constexpr (NSTG == 2) {
 #pragma unroll
-        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + k_dst + i * RSTEP * KP) = kr[i];
+            for (int i2 = 0; i2 < NV; ++i2)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kr[i2]) : "v"(Kg + off + i2 * NT * 8) : "memory");
 #pragma unroll
-        for (int i = 0; i < NV; ++i) *reinterpret_cast<u32x4*>(buf + v_dst + i * RSTEP * VP) = vr[i];
-        const int key0 = bc * BW;
-        // next live block (the last step re-reads its own block; the copy is not used)
-        bc = bc_next;
-        bc_next = column(e + 2 < e_end ? e + 2 : e_end - 1);
-        {
-            const int64_t off = (int64_t)bc * BW * E;
+            for (int i2 = 0; i2 < NV; ++i2)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(vr[i2]) : "v"(Vg + off + i2 * NT * 8) : "memory");
+        } else {
 #pragma unroll
-            for (int i = 0; i < NV; ++i) kr[i] = *reinterpret_cast<const u32x4*>(Kg + off + i * NT * 8);
+            for (int i2 = 0; i2 < NV; ++i2) kr[i2] = *reinterpret_cast<const u32x4*>(Kg + off + i2 * NT * 8);
 #pragma unroll
-            for (int i = 0; i < NV; ++i) vr[i] = *reinterpret_cast<const u32x4*>(Vg + off + i * NT * 8);
+            for (int i2 = 0; i2 < NV; ++i2) vr[i2] = *reinterpret_cast<const u32x4*>(Vg + off + i2 * NT * 8);
         }
+    };
+    // Wait until only the other stage is outstanding; the stage's registers pass through the
+    // statement so that no use is scheduled before it.
+    auto wait_stage = [&](int i, u32x4 (&kr)[NV], u32x4 (&vr)[NV]) {
+        if constexpr (NSTG == 1) return;   // plain loads: the compiler waits where the registers are used
+        if (i + 1 < n_blk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NV) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) asm volatile("" : "+v"(kr[i2]));
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) asm volatile("" : "+v"(vr[i2]));
+    };
+    auto step = [&](int i, u32x4 (&kr)[NV], u32x4 (&vr)[NV]) {
+        char* buf = smem + (NBUF == 2 ? (i & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();  // the previous block's fragments are consumed
+        wait_stage(i, kr, vr);
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) *reinterpret_cast<u32x4*>(buf + k_dst + i2 * RSTEP * KP) = kr[i2];
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) *reinterpret_cast<u32x4*>(buf + v_dst + i2 * RSTEP * VP) = vr[i2];
+        if (i + NSTG < n_blk) issue(i + NSTG, kr, vr);
         unsigned live[KT];
         if constexpr (SEQ) {
             // one byte per key of this lane, set while the key position is below the length
+            const int key0 = i * BW;
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
                 const int left = seq_len - (key0 + kt * 16 + g4 * 4);   // live keys among the lane's four
                 live[kt] = left >= 4 ? 0x01010101u : left <= 0 ? 0u : (0x01010101u >> (8 * (4 - left)));
             }
         } else if constexpr (HAS_MASK) {
+            const int key0 = col_at(i) * BW;
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
                 live[kt] = *reinterpret_cast<const uint32_t*>(p.mask + (int64_t)qrow * p.Ns + key0 + kt * 16 + g4 * 4);
@@ -431,6 +461,21 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void attention_kernel_v2(Att
                 oacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), pf[kp], oacc[t]);
             }
         }
+    };
+    if constexpr (NSTG == 2) {
+        u32x4 k0[NV], v0[NV], k1[NV], v1[NV];
+        if (n_blk > 0) {
+            issue(0, k0, v0);
+            issue(n_blk > 1 ? 1 : 0, k1, v1);   // a row of one block requests it twice; the copy is not used
+        }
+        for (int i = 0; i < n_blk; i += 2) {
+            step(i, k0, v0);
+            if (i + 1 < n_blk) step(i + 1, k1, v1);
+        }
+    } else {
+        u32x4 k0[NV], v0[NV];
+        if (n_blk > 0) issue(0, k0, v0);
+        for (int i = 0; i < n_blk; ++i) step(i, k0, v0);
     }
 
     // every accumulator row of lacc holds the row sum of query r16
@@ -538,7 +583,7 @@ static int launch_attention_v2(const AttnParams& p, int batch, int BW, int E, hi
 // P.V MFMAs, so the output needs no final division.  One launch replaces the scores,
 // softmax and P.V operators of the forward pipeline.
 template <typename T, int BW, int E, int WAVES, bool HAS_MASK>
-__global__ __launch_bounds__(64 * (WAVES + 1), 8 / WAVES) void attention_train_kernel(AttnParams p, int nbr, int batch) {
+__global__ __launch_bounds__(64 * (WAVES + 1), waves_per_simd_for((2 * BW * (E * 4 + 32) <= 64 * 1024 ? 2 : 1) * BW * (E * 4 + 32) + 2 * WAVES * 16 * (BW * 2), WAVES + 1, 8 / WAVES)) void attention_train_kernel(AttnParams p, int nbr, int batch) {
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
     constexpr int KP = E * 2;                 // K row pitch in bytes (16-byte chunks XOR-swizzled by row % 8)
@@ -854,19 +899,8 @@ static int launch_attention_train(const AttnParams& p, int batch, int BW, int E,
 // layout of P and fed to the dQ MFMAs.  Masked entries have P = 0 and so dS = 0: no mask is
 // needed.  dK and dV stay with the sparse-operand matmul kernels (dK = dS^T Q, dV = P^T dO).
 // Replaces three launches of the operator pipeline's backward (dP, softmax backward, dQ).
-// Wavefronts per SIMD the register budget is sized for: no more than the LDS footprint lets
-// a CU hold (two-wavefront workgroups with large tiles spilled under the budget of four).
-template <int BW, int E, int WAVES>
-constexpr int bwd_row_waves_per_simd() {
-    constexpr int TILE = BW * (E * 4 + 32);
-    constexpr int smem = (2 * TILE <= 64 * 1024 ? 2 * TILE : TILE) + WAVES * 16 * (BW * 2 + 16);
-    constexpr int by_lds = (160 * 1024 / smem * WAVES + 3) / 4;
-    constexpr int cap = 8 / WAVES;
-    return by_lds < 1 ? 1 : (by_lds < cap ? by_lds : cap);
-}
-
 template <typename T, int BW, int E, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, (bwd_row_waves_per_simd<BW, E, WAVES>())) void attention_bwd_row_kernel(AttnParams p, int nbr, int batch) {
+__global__ __launch_bounds__(64 * WAVES, waves_per_simd_for((2 * BW * (E * 4 + 32) <= 64 * 1024 ? 2 : 1) * BW * (E * 4 + 32) + WAVES * 16 * (BW * 2 + 16), WAVES)) void attention_bwd_row_kernel(AttnParams p, int nbr, int batch) {
     constexpr int NT = 64 * WAVES;
     constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
     constexpr int RP = E * 2;                 // pitch of the row-read tile (V): 16-byte chunks XOR-swizzled by row % 8
