@@ -40,9 +40,10 @@ def make_inputs(torch, device):
     return x, w, mask
 
 
-def time_graph(torch, fn, steps, warmup):
+def time_graph(torch, fn, steps, warmup, repeats=1):
     """Device time of `steps` calls of fn(), replayed from one captured graph and
-    bracketed by events on the replay stream.  Returns seconds for all steps."""
+    bracketed by events on the replay stream.  Returns seconds for all steps (the
+    shortest of `repeats` timed replays)."""
     for _ in range(max(warmup, 1)):
         fn()
     torch.cuda.synchronize()
@@ -56,13 +57,17 @@ def time_graph(torch, fn, steps, warmup):
                 fn()
         graph.replay()  # untimed replay: page in the graph
         stream.synchronize()
-        begin = torch.cuda.Event(enable_timing=True)
-        end = torch.cuda.Event(enable_timing=True)
-        begin.record(stream)
-        graph.replay()
-        end.record(stream)
-        stream.synchronize()
-    return begin.elapsed_time(end) / 1e3
+        best = None
+        for _ in range(max(repeats, 1)):
+            begin = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            begin.record(stream)
+            graph.replay()
+            end.record(stream)
+            stream.synchronize()
+            took = begin.elapsed_time(end) / 1e3
+            best = took if best is None else min(best, took)
+    return best
 
 
 def time_eager(torch, fn, steps, warmup):
@@ -120,8 +125,10 @@ def measured_traffic_bytes():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=200)
-    ap.add_argument('--warmup', type=int, default=20)
+    # a step takes under 30 us: 2000 + 2000 steps are 0.1 s of device time, enough for the clocks to
+    # settle (200 steps after 20 of warm-up measured 6 % slower than the steady state)
+    ap.add_argument('--steps', type=int, default=2000)
+    ap.add_argument('--warmup', type=int, default=2000)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run one plain 256 MiB device copy, so that a rocprofv3 --pmc run of this '
@@ -255,11 +262,12 @@ def main():
     if not args.no_secondary:
         import bench_configs
         try:
-            rows = bench_configs.run(['c1', 'c2', 'c3', 'c4', 'c5'], min(args.steps, 20), min(args.warmup, 5), time_graph,
+            rows = bench_configs.run(['c1', 'c2', 'c3', 'c4', 'c5'], min(args.steps, 50), min(args.warmup, 10), time_graph,
                                      time_eager, brief=True, verbose=False)
             out['secondary'] = {
                 'note': 'other benchmark configurations; each result was compared with the dense fp32 torch '
-                        'computation of the same inputs before it was timed',
+                        'computation of the same inputs before it was timed; times are the shortest of three '
+                        'graph replays of 50 steps (a single short replay right after the checks runs at ramping clocks)',
                 'results': [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in r.items()
                              if k != 'expert_counts'} for r in rows],
             }

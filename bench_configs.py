@@ -63,10 +63,11 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
     _emit.verbose = verbose
 
     def timed(fn):
+        # shortest of three replays: the first one after the correctness checks runs at ramping clocks
         try:
-            return time_graph(torch, fn, steps, warmup) / steps
+            return time_graph(torch, fn, steps, warmup, 3) / steps
         except Exception:
-            return time_eager(torch, fn, steps, warmup) / steps
+            return min(time_eager(torch, fn, steps, warmup) for _ in range(3)) / steps
 
     cfg32 = {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32}
     with torch.no_grad():
