@@ -236,17 +236,18 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
                 return torch.matmul(h.float(), (l2.weight.float() * m2.float()).t())
 
             for dynamic in ((True,) if brief else (True, False)):
-                op1 = sparta.nn.SparseLinear(l1, weight_mask=masks1[0], dynamic=dynamic)
+                # the activation between the layers runs in the first layer's epilogue
+                op1 = sparta.nn.SparseLinear(l1, weight_mask=masks1[0], dynamic=dynamic, activation='relu')
                 op2 = sparta.nn.SparseLinear(l2, weight_mask=masks2[0], dynamic=dynamic)
                 op1.build(cfg, sample_inputs=[x])
-                op2.build(cfg, sample_inputs=[torch.relu(op1(x))])
+                op2.build(cfg, sample_inputs=[op1(x)])
                 m1 = masks1[1].clone()
                 m2 = masks2[1].clone()
 
                 def step():
                     op1.update_mask(weight_mask=m1)
                     op2.update_mask(weight_mask=m2)
-                    return op2(torch.relu(op1(x)))
+                    return op2(op1(x))
 
                 _close(torch, step(), dense_ffn(m1, m2), f'c4 dynamic={dynamic}')
                 if dynamic:
@@ -262,8 +263,21 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
                 _emit(f'c4 dynamic-mask FFN 8192x768->3072->768 fp16, rebuild timed, dynamic={dynamic}', sec,
                       flops=2 * 2.0 * T * 116 * 32 * 64, extra={'timing': tag})
             if not brief:
-                fwd_only = timed(lambda: op2(torch.relu(op1(x))))
+                fwd_only = timed(lambda: op2(op1(x)))
                 _emit('c4 same FFN, masks fixed (no rebuild)', fwd_only, flops=2 * 2.0 * T * 116 * 32 * 64)
+                op1p = sparta.nn.SparseLinear(l1, weight_mask=m1, dynamic=True)
+                op2p = sparta.nn.SparseLinear(l2, weight_mask=m2, dynamic=True)
+                op1p.build(cfg, sample_inputs=[x])
+                op2p.build(cfg, sample_inputs=[torch.relu(op1p(x))])
+
+                def step_unfused():
+                    op1p.update_mask(weight_mask=m1)
+                    op2p.update_mask(weight_mask=m2)
+                    return op2p(torch.relu(op1p(x)))
+
+                _close(torch, step_unfused(), dense_ffn(m1, m2), 'c4 separate activation kernel')
+                _emit('c4 dynamic FFN with the activation as a separate torch kernel (as the reference would run it)',
+                      timed(step_unfused), flops=2 * 2.0 * T * 116 * 32 * 64)
                 sec = timed(lambda: l2(torch.relu(l1(x))))
                 _emit('c4 dense torch FFN fp16', sec, flops=2 * 2.0 * T * D * F)
 

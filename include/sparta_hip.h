@@ -172,8 +172,12 @@ int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
  * idx / idx_kind  see spx_idx_kind.  nnz_bound / nnz_dev as in spx_bcs_gather
  *                 (only DDS launches over blocks).
  * sched     optional output of spx_bcs_schedule for `ptr` (NULL = natural order).
- * tile_cfg  index into the tile-config table of the op (0 = default).
+ * tile_cfg  index into the tile-config table of the op (0 = default), optionally or-ed
+ *           with SPX_EPILOGUE_RELU (SDD and DSD): C = max(op(A) op(B) + bias, 0), NaN kept,
+ *           written by the same kernel.  No counterpart in the reference, whose
+ *           SparseLinear is followed by a separate activation kernel.
  * ------------------------------------------------------------------------ */
+#define SPX_EPILOGUE_RELU 0x10000
 int spx_matmul(int mode, int dtype, int transA, int transB, int compressed,
                const void* A, const void* B, const void* bias, void* C,
                const int32_t* ptr, const void* idx, int idx_kind, const int32_t* sched,

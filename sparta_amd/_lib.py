@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libsparta_hip.so')
 F32, F16, BF16 = 0, 1, 2
 SDD, DSD, DDS = 0, 1, 2
 IDX_BCSR_I32, IDX_BCSC_I32, IDX_BCSC_I64 = 0, 1, 2
+EPILOGUE_RELU = 0x10000   # or-ed into spx_matmul's tile_cfg
 E_NULL, E_SHAPE, E_DTYPE, E_ALIGN, E_WORKSPACE, E_CONFIG, E_NO_DEVICE = -1, -2, -3, -4, -5, -6, -7
 OP_SPMM, OP_DDS, OP_SOFTMAX, OP_ATTENTION, OP_MOE = 0, 1, 2, 3, 4
 

@@ -34,6 +34,8 @@ static int run_matmul(int mode, int transA, int transB, int compressed,
     }
 
     SpmmParams p;
+    p.relu = (tile_cfg & SPX_EPILOGUE_RELU) != 0;
+    tile_cfg &= ~SPX_EPILOGUE_RELU;
     p.bias = bias; p.out = C; p.ptr = ptr; p.idx = idx; p.idx_kind = idx_kind; p.sched = sched;
     p.K = K; p.BK = BK; p.log_bk = ilog2(BK);
     p.compressed = compressed;
@@ -100,6 +102,7 @@ extern "C" int spx_matmul(int mode, int dtype, int transA, int transB, int compr
     SPX_REQUIRE(idx_kind >= 0 && idx_kind <= 2, SPX_E_CONFIG, "unknown idx_kind %d", idx_kind);
     if (mode == SPX_DDS) {
         SPX_REQUIRE(idx_kind == SPX_IDX_BCSR_I32, SPX_E_CONFIG, "sparse-output matmul reads a BCSR index");
+        SPX_REQUIRE(!(tile_cfg & SPX_EPILOGUE_RELU), SPX_E_CONFIG, "the fused activation covers sdd and dsd only");
     } else {
         SPX_REQUIRE(ptr, SPX_E_NULL, "row_ptr / col_ptr is required for sdd and dsd");
         const bool wants_bcsr = (mode == SPX_DSD) ? (transB != 0) : (transA == 0);

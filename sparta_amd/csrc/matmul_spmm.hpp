@@ -36,7 +36,11 @@ struct SpmmParams {
     int64_t o_ld;
     int bias_on_m;       // bias indexed by canonical m instead of n
     int64_t d_batch, s_batch, o_batch, bias_batch;
+    int relu;           // epilogue: negative results (after the bias) become zero
 };
+
+// Optional activation of the epilogue; NaN stays NaN (as torch.relu keeps it).
+__device__ __forceinline__ float epilogue_act(float v, int relu) { return (relu && v < 0.f) ? 0.f : v; }
 
 template <typename T, int BN, int WM>
 __global__ __launch_bounds__(256) void spmm_kernel(SpmmParams p) {
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(SpmmParams p) {
                         const int bi = p.bias_on_m ? (m0 + m < p.Mc ? m0 + m : 0) : j * BN + n;
                         v += Elem<T>::to_float(biasT[bi]);
                     }
-                    Es[m * LDE + n] = Elem<T>::from_float(v);
+                    Es[m * LDE + n] = Elem<T>::from_float(epilogue_act(v, p.relu));
                 }
         __syncthreads();
         constexpr int VPR = BN / VE;
@@ -170,7 +174,7 @@ __global__ __launch_bounds__(256) void spmm_kernel(SpmmParams p) {
                         const int bi = p.bias_on_m ? (m0 + m < p.Mc ? m0 + m : 0) : j * BN + n;
                         v += Elem<T>::to_float(biasT[bi]);
                     }
-                    Es[n * LDE + m] = Elem<T>::from_float(v);
+                    Es[n * LDE + m] = Elem<T>::from_float(epilogue_act(v, p.relu));
                 }
         __syncthreads();
         constexpr int VPR = TM / VE;

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void spmm_direct_kernel(SpmmParams p, int n_mt
             for (int q = 0; q < 4; ++q) {
                 float v = acc[i][t][q];
                 if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (SWAP ? m : m + q) : (SWAP ? n + q : n)]);
-                vals[q] = Elem<T>::from_float(v);
+                vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
             }
             T* dst = SWAP ? out + (int64_t)m * p.o_ld + n : out + (int64_t)n * p.o_ld + m;
             if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);

@@ -209,7 +209,7 @@ __global__ __launch_bounds__(256) void spmm_ksplit_kernel(SpmmParams p, int n_mt
             for (int e = 0; e < EPL; ++e) {
                 float x = v[e];
                 if (biasT) x += Elem<T>::to_float(biasT[p.bias_on_m ? m : j * BN + col + e]);
-                vals[e] = Elem<T>::from_float(x);
+                vals[e] = Elem<T>::from_float(epilogue_act(x, p.relu));
             }
             T* dst = out + (int64_t)m * p.o_ld + (int64_t)j * BN + col;
 #pragma unroll
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) void spmm_ksplit_kernel(SpmmParams p, int n_mt
                 for (int w = 0; w < 4; ++w) x += P[(w * 64 + row + q) * PB + n];
                 const int m = m0 + row + q;
                 if (biasT) x += Elem<T>::to_float(biasT[p.bias_on_m ? (m < p.Mc ? m : 0) : j * BN + n]);
-                vals[q] = Elem<T>::from_float(x);
+                vals[q] = Elem<T>::from_float(epilogue_act(x, p.relu));
             }
             T* dst = out + ((int64_t)j * BN + n) * p.o_ld + m0 + row;
             if (m0 + row + 4 <= p.Mc) {

@@ -311,7 +311,7 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
                     float v = acc[i][t][q];
                     const int n = j * BN + t * 16 + g4 * 4 + q;
                     if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m0 + i * 16 + r16 < p.Mc ? m0 + i * 16 + r16 : 0) : n]);
-                    vals[q] = Elem<T>::from_float(v);
+                    vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
                 }
                 T* dst = eT + r16 * LDE + t * 16 + g4 * 4;
                 if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256, (BN <= 32 && NST == 2) ? 4 : 2) void spmm_pane
                     float v = acc[i][t][q];
                     const int m = m0 + i * 16 + g4 * 4 + q;
                     if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m < p.Mc ? m : 0) : j * BN + t * 16 + r16]);
-                    vals[q] = Elem<T>::from_float(v);
+                    vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
                 }
                 T* dst = eT + r16 * LDE + i * 16 + g4 * 4;
                 if constexpr (sizeof(T) == 2) *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(vals);

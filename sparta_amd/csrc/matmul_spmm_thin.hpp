@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256) void spmm_thin_kernel(SpmmParams p, int nb, in
         for (int q = 0; q < 4; ++q) {
             float v = acc[t][q];
             if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? t * 16 + g4 * 4 + q : n]);
-            vals[q] = Elem<T>::from_float(v);
+            vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
         }
         *reinterpret_cast<uint64_t*>(out + (int64_t)n * p.o_ld + t * 16 + g4 * 4) = *reinterpret_cast<const uint64_t*>(vals);
     }

@@ -42,6 +42,7 @@ class SparseBatchMatMulCtx(SparseCtxBase):
         self._transpose_B = transpose_B
         self._biased = biased
         self._compressed = compressed
+        self._activation: Optional[str] = None
         sparse_tensor = 'ABC'[mode.index('s')]
         self._tesa_shapes: Dict[str, Tuple[str, str]] = {}
         for name, (bias, order, tA, tB) in _derive_kernels(mode, transpose_A, transpose_B, biased).items():
@@ -65,10 +66,23 @@ class SparseBatchMatMulCtx(SparseCtxBase):
         self._kernels['backward:B'].set_shape(*((batch_size, N, M, K) if self._transpose_B
                                                 else (batch_size, K, M, N)))
 
+    def set_activation(self, activation: Optional[str]):
+        """Fuse an activation (None or 'relu') into the forward kernel's epilogue; the
+        autograd function then masks the incoming gradient with the sign of the output."""
+        if activation not in (None, 'relu'):
+            raise ValueError(f'unsupported fused activation: {activation!r}')
+        if activation is not None and self._mode == 'dds':
+            raise ValueError('the fused activation covers the sdd and dsd kernels only')
+        self._activation = activation
+        fwd = self._kernels['forward:C'].active_kernel()
+        if fwd is not None:
+            fwd.set_epilogue(activation)
+
     def build(self, config: Dict[str, Dict[str, Any]]):
         super().build(config)
         fwd = self._kernels['forward:C'].active_kernel()
         if fwd is not None:
+            fwd.set_epilogue(self._activation)
             self.forward_C = (lambda A, B, bias: fwd(A, B, bias)) if self._biased else (lambda A, B: fwd(A, B))
             if self._mode == 'dds' and self._compressed:
                 kernel = fwd
@@ -119,16 +133,21 @@ class SparseBatchMatMulFunc(torch.autograd.Function):
     def forward(ctx, sparta_ctx: SparseBatchMatMulCtx, input: torch.Tensor, weight: torch.Tensor,
                 bias: Optional[torch.Tensor] = None):
         input, weight = input.detach(), weight.detach()
-        ctx.save_for_backward(input, weight, bias)
         ctx.sparta_ctx = sparta_ctx
         if bias is None:
-            return sparta_ctx.forward_C(input, weight)
-        return sparta_ctx.forward_C(input, weight, bias.detach())
+            output = sparta_ctx.forward_C(input, weight)
+        else:
+            output = sparta_ctx.forward_C(input, weight, bias.detach())
+        # a fused relu: the gradient passes where the output is positive
+        ctx.save_for_backward(input, weight, bias, output if sparta_ctx._activation == 'relu' else None)
+        return output
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor):
-        input, weight, bias = ctx.saved_tensors
+        input, weight, bias, gate = ctx.saved_tensors
         grad_output = grad_output.detach().contiguous()
+        if gate is not None:
+            grad_output = grad_output * (gate > 0)
         grad_input = grad_weight = grad_bias = None
         if ctx.needs_input_grad[1]:
             grad_input = ctx.sparta_ctx.backward_A(grad_output, weight)

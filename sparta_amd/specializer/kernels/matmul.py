@@ -8,7 +8,7 @@ The two implementation names of the reference are kept as configuration slots:
 point; both run the same gfx950 MFMA kernels.  The thread-tile look-up table of
 the reference has no counterpart: THREAD_SIZE_* values are accepted and ignored.
 """
-from typing import Any, Dict, List
+from typing import Any, Dict, List, Optional
 
 import torch
 
@@ -52,7 +52,19 @@ class SparseMatMulKernel(KernelBase):
             self._tesa_vars = ['col_ptr', 'BCSC_idx', 'nnz']
         if mode == 'dds':
             self._tesa_vars = self._tesa_vars[1:]
+        self._epilogue = 0
         super().__init__()
+
+    def set_epilogue(self, activation: Optional[str]):
+        """Activation applied by the kernel's own epilogue (an extension: the reference runs a
+        separate elementwise kernel after the operator): None or 'relu', sdd / dsd only."""
+        if activation not in (None, 'relu'):
+            raise ValueError(f'unsupported fused activation: {activation!r}')
+        if activation is not None and self._mode == 'dds':
+            raise ValueError('the fused activation covers the sdd and dsd kernels only')
+        self._epilogue = _lib.EPILOGUE_RELU if activation == 'relu' else 0
+        if self.ready:
+            self.update_func()
 
     # ---- ports / parameters -------------------------------------------------------
     def _set_ports(self):
@@ -134,7 +146,7 @@ class SparseMatMulKernel(KernelBase):
         tA, tB = int(self._transpose_A), int(self._transpose_B)
         compressed = int(self._compressed)
         biased = self._biased
-        tile_cfg = int(self.get_parameter('TILE_CFG') or 0)
+        tile_cfg = int(self.get_parameter('TILE_CFG') or 0) | self._epilogue
         tile_elems = self.get_parameter(self._sparse_block_H) * self.get_parameter(self._sparse_block_W)
         lib = _lib.load()
 
@@ -213,6 +225,8 @@ class SparseMatMulKernel(KernelBase):
         C = torch.matmul(lhs, rhs)
         if self._biased:
             C = C + args[2].unsqueeze(1)
+        if self._epilogue:
+            C = torch.relu(C)
         if self._mode == 'dds':
             port = self.ports['C']
             C = C * (port.indexes.get_mask() if self.ready else port.mask)

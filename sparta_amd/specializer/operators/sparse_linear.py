@@ -21,6 +21,9 @@ class SparseLinear(OperatorBase):
             once per rebuild); with a weight mask the weight stays dense and the kernels
             read its live blocks through the index (no re-compression), with an input
             mask the compressed operand is kept at full capacity.
+        activation: None or 'relu' (an extension; the reference's operator has none): the
+            activation that follows the layer, applied by the matmul kernel's own epilogue
+            instead of a separate elementwise kernel.  Input and weight masks only.
 
     Shape: input (B, in_features) -> output (B, out_features).
 
@@ -39,8 +42,11 @@ class SparseLinear(OperatorBase):
 
     def __init__(self, raw_module: torch.nn.Linear, input_mask: Optional[torch.Tensor] = None,
                  weight_mask: Optional[torch.Tensor] = None, output_mask: Optional[torch.Tensor] = None,
-                 dynamic: bool = False):
+                 dynamic: bool = False, activation: Optional[str] = None):
         super().__init__(raw_module)
+        if activation not in (None, 'relu'):
+            raise ValueError(f'unsupported fused activation: {activation!r}')
+        self._activation = activation
         N, K = raw_module.weight.shape
         biased = raw_module.bias is not None
         self._raw_weight = torch.clone(raw_module.weight)
@@ -59,6 +65,7 @@ class SparseLinear(OperatorBase):
             M = output_mask.shape[0]
         else:
             raise ValueError('expected a sparse mask on input / weight / output')
+        self._sparse_ctx.set_activation(activation)
         self._shape = {'batch_size': 1, 'M': M, 'K': K, 'N': N}
         self._dynamic = dynamic
         self._set_dynamic(dynamic)
@@ -107,6 +114,10 @@ class SparseLinear(OperatorBase):
     def _compile(self, config: Optional[Dict[str, Dict[str, Any]]] = None):
         super()._compile(config)
         self._update_parameters()
+
+    def _dense_forward(self, *args):
+        out = super()._dense_forward(*args)
+        return torch.relu(out) if self._activation == 'relu' else out
 
     def _sparse_forward(self, input_tensor: torch.Tensor):
         args = [self._sparse_ctx, input_tensor, self.weight]

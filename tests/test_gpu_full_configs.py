@@ -87,7 +87,10 @@ def topk_block_mask(shape, seed, block=(32, 64), keep_frac=0.1):
     return np.kron(grid, np.ones(block, dtype=np.uint8)), int(grid.sum())
 
 
-def test_c4_dynamic_ffn_three_mask_updates(gpu):
+@pytest.mark.parametrize('fused', [True, False])
+def test_c4_dynamic_ffn_three_mask_updates(fused, gpu):
+    # fused: the activation between the layers runs in the first layer's epilogue (what bench.py times)
+    act = (lambda h: h) if fused else torch.relu
     T, D, F = 8192, 768, 3072
     rng = np.random.default_rng(2022)
     x = torch.from_numpy(rng.standard_normal((T, D)).astype(np.float32)).half()
@@ -103,11 +106,12 @@ def test_c4_dynamic_ffn_three_mask_updates(gpu):
     masks2 = [topk_block_mask((D, F), 100 + s) for s in range(4)]
     assert all(n == 116 for _, n in masks1 + masks2)  # ceil(0.1 * 1152)
     cfg = {'forward:C': {'_impl': 'openai', 'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 64, 'BLOCK_SIZE_N_VALUE': 32}}
-    op1 = sparta.nn.SparseLinear(l1, weight_mask=torch.from_numpy(masks1[0][0]).to(gpu), dynamic=True)
+    op1 = sparta.nn.SparseLinear(l1, weight_mask=torch.from_numpy(masks1[0][0]).to(gpu), dynamic=True,
+                                 activation='relu' if fused else None)
     op2 = sparta.nn.SparseLinear(l2, weight_mask=torch.from_numpy(masks2[0][0]).to(gpu), dynamic=True)
     with torch.no_grad():
         op1.build(cfg, sample_inputs=[xg])
-        op2.build(cfg, sample_inputs=[torch.relu(op1(xg))])
+        op2.build(cfg, sample_inputs=[act(op1(xg))])
 
     xn, w1n, w2n = (t.to(torch.float64).numpy() for t in (x, w1, w2))
 
@@ -124,7 +128,7 @@ def test_c4_dynamic_ffn_three_mask_updates(gpu):
         with torch.no_grad():
             op1.update_mask(weight_mask=torch.from_numpy(m1).to(gpu))
             op2.update_mask(weight_mask=torch.from_numpy(m2).to(gpu))
-            y = op2(torch.relu(op1(xg)))
+            y = op2(act(op1(xg)))
         for op, m in ((op1, m1), (op2, m2)):
             idx = op.get_sparse_indexes('B')
             row_ptr, bcsr, nnz = bcs.build_bcsr(m, 32, 64)
@@ -140,7 +144,7 @@ def test_c4_dynamic_ffn_three_mask_updates(gpu):
     def graph_step():
         op1.update_mask(weight_mask=m1g)
         op2.update_mask(weight_mask=m2g)
-        return op2(torch.relu(op1(xg)))
+        return op2(act(op1(xg)))
 
     with torch.no_grad():
         graph_step()

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 
 def run_case(gpu, mode, tA, tB, biased, compressed, dtype, blocks, impl='sparta',
-             batch=4, M=128, K=256, N=192, gran=(8, 8), sparsity=0.9, seed=2022, tile_cfg=0):
+             batch=4, M=128, K=256, N=192, gran=(8, 8), sparsity=0.9, seed=2022, tile_cfg=0, activation=None):
     BM, BK, BN = blocks
     A_shape = (K, M) if tA else (M, K)
     B_shape = (N, K) if tB else (K, N)
@@ -34,12 +34,16 @@ def run_case(gpu, mode, tA, tB, biased, compressed, dtype, blocks, impl='sparta'
     kernel.set_shape(batch, M, K, N)
     kernel.compile({'BLOCK_SIZE_M_VALUE': BM, 'BLOCK_SIZE_K_VALUE': BK, 'BLOCK_SIZE_N_VALUE': BN,
                     'TILE_CFG': tile_cfg})
+    if activation is not None:
+        kernel.set_epilogue(activation)
     indexes = kernel.ports[port].indexes
     tile = {'sdd': (BK, BM) if tA else (BM, BK), 'dsd': (BN, BK) if tB else (BK, BN), 'dds': (BM, BN)}[mode]
     assert (indexes.block_H, indexes.block_W) == tile
 
     want = ops.matmul_reference(a_np, b_np, bias_np if biased else None, mode=mode, transpose_A=tA,
                                 transpose_B=tB, mask=mask_np, block=tile, dtype=np.float64)
+    if activation == 'relu':
+        want = np.maximum(want, 0.0)
     A = a_t.to(gpu)
     B = b_t.to(gpu)
     # masked operands go in masked (the kernel reads every element of a live block)
@@ -112,6 +116,29 @@ def test_matmul_tile_configs(tile_cfg, mode, compressed, dtype, blocks, gpu):
     run_case(gpu, mode, False, True, True, compressed, dtype, blocks, batch=2,
              M=320 if mode == 'dsd' else 192, K=256, N=192 if mode == 'dsd' else 328, gran=(16, 16),
              sparsity=0.7, seed=11, tile_cfg=tile_cfg)
+
+
+@pytest.mark.parametrize('tile_cfg', [0, 1, 2, 3, 4, 5, 6, 7, 8, 10])
+@pytest.mark.parametrize('mode', ['sdd', 'dsd'])
+@pytest.mark.parametrize('biased', [False, True])
+@pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (32, 64, 32)),
+                                          (torch.float32, (16, 16, 16))])
+def test_matmul_fused_relu(tile_cfg, mode, biased, dtype, blocks, gpu):
+    """SPX_EPILOGUE_RELU or-ed into the tile config: every kernel family of the sparse-operand
+    product clamps its result (after the bias) at zero in its own epilogue."""
+    run_case(gpu, mode, False, True, biased, True, dtype, blocks, batch=2,
+             M=320 if mode == 'dsd' else 192, K=256, N=192 if mode == 'dsd' else 328, gran=(16, 16),
+             sparsity=0.7, seed=29, tile_cfg=tile_cfg, activation='relu')
+
+
+def test_matmul_fused_relu_thin_operand_and_rejections(gpu):
+    run_case(gpu, 'sdd', False, False, True, True, torch.float16, (64, 32, 32), batch=5, M=448, K=320, N=64,
+             gran=(32, 32), sparsity=0.8, seed=31, tile_cfg=9, activation='relu')
+    kernel = SparTASparseMatMulKernel(mode='dds', biased=False, transpose_A=False, transpose_B=True, compressed=True)
+    with pytest.raises(ValueError):
+        kernel.set_epilogue('relu')
+    with pytest.raises(ValueError):
+        SparTASparseMatMulKernel(mode='dsd').set_epilogue('gelu')
 
 
 @pytest.mark.parametrize('mode', ['sdd', 'dsd'])

@@ -46,6 +46,51 @@ def test_readme_flow_fp32(gpu):
     assert np.all(np.abs(g - wnt) <= 1e-4 + 1e-4 * np.abs(wnt)), np.abs(g - wnt).max()
 
 
+@pytest.mark.parametrize('kind', ['input', 'weight'])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+@pytest.mark.parametrize('dynamic', [False, True])
+def test_sparse_linear_fused_relu(kind, dtype, dynamic, gpu, M=128, K=256, N=192):
+    """SparseLinear(activation='relu'): relu(x W^T + b) from the matmul kernel's epilogue, with
+    the gradients of relu(linear) (the incoming gradient is gated by the sign of the output)."""
+    x_np, x = randn((M, K), 14, dtype)
+    w_np, w = randn((N, K), 15, dtype, scale=0.5)
+    b_np, b = randn((N,), 16, dtype)
+    gy_np, gy = randn((M, N), 17, dtype)
+    shape = {'input': (M, K), 'weight': (N, K)}[kind]
+    mask_np = ops.block_mask(shape, (8, 8), 0.9, seed=3)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    w_in = w * torch.from_numpy(mask_np).to(dtype) if kind == 'weight' else w
+    op = sparta.nn.SparseLinear(dense_linear(K, N, w_in, b, gpu, dtype), dynamic=dynamic, activation='relu',
+                                **{f'{kind}_mask': mask})
+    cfg = {k: dict(CFG32) for k in ('forward:C', 'backward:A', 'backward:B')}
+    op.build(cfg, sample_inputs=[x.to(gpu)])
+    xr = (x.to(gpu).float() * (mask if kind == 'input' else 1)).requires_grad_(True)
+    wr = (w.to(gpu).float() * (mask if kind == 'weight' else 1)).requires_grad_(True)
+    br = b.to(gpu).float().requires_grad_(True)
+    pre = torch.nn.functional.linear(xr, wr, br)
+    xs = (x.to(gpu) * (mask.to(dtype) if kind == 'input' else 1)).requires_grad_(True)
+    y = op(xs)
+    assert float(y.detach().min()) >= 0.0
+    assert_close(y, torch.relu(pre).detach().double().cpu().numpy(), dtype, f'{kind} relu forward')
+    y.backward(gy.to(gpu))
+    # the reference gradient is gated by the operator's own output: an entry within rounding
+    # of zero may fall on either side, and either gate is a correct derivative there
+    pre.backward(gy.to(gpu).float() * (y.detach() > 0))
+    block_mask = op.get_sparse_indexes({'input': 'A', 'weight': 'B'}[kind]).get_mask()
+    gx_want = xr.grad * (block_mask if kind == 'input' else 1)
+    assert_close(xs.grad, gx_want.double().cpu().numpy(), dtype, f'{kind} relu grad_x')
+    gw = op.weight.grad
+    if kind == 'weight' and not dynamic:
+        gw = op.get_sparse_indexes('B').inverse(gw)
+    gw_want = wr.grad * (block_mask if kind == 'weight' else 1)
+    assert_close(gw if kind == 'input' else gw * block_mask.to(gw.dtype), gw_want.double().cpu().numpy(), dtype, f'{kind} relu grad_w')
+    assert_close(op.bias.grad, br.grad.double().cpu().numpy(), dtype, f'{kind} relu grad_b')
+    with pytest.raises(ValueError):
+        sparta.nn.SparseLinear(dense_linear(K, N, w, b, gpu, dtype), output_mask=torch.ones((M, N), device=gpu), activation='relu')
+    with pytest.raises(ValueError):
+        sparta.nn.SparseLinear(dense_linear(K, N, w_in, b, gpu, dtype), weight_mask=mask, activation='gelu')
+
+
 @pytest.mark.parametrize('kind', ['input', 'weight', 'output'])
 @pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
 def test_sparse_linear_forward_backward_and_mask_updates(kind, dtype, gpu, M=128, K=256, N=192):
