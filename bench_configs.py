@@ -201,10 +201,13 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
                     fn(*leaves).backward(grad)
 
                 n_step = min(steps, 20)
-                for fused, name in ((True, 'c3 training step, fused forward, row-side and column-side backward kernels'),
-                                    (False, 'c3 training step, three operators forward and six kernels backward')):
+                for fused, recompute, name in (
+                        (True, True, 'c3 training step, no stored probabilities (forward with row statistics, recomputing row-side and column-side backward kernels)'),
+                        (True, False, 'c3 training step, stored probabilities (fused forward, row-side and column-side backward kernels)'),
+                        (False, False, 'c3 training step, three operators forward and six kernels backward')):
                     att_t._fused = fused
-                    sec = time_eager(torch, lambda: step(att_t), n_step, 3) / n_step
+                    att_t._recompute = recompute
+                    sec = min(time_eager(torch, lambda: step(att_t), n_step, 3) for _ in range(3)) / n_step
                     _emit(name, sec, flops=3 * flops)
                 dense = lambda a, b, c: torch.nn.functional.scaled_dot_product_attention(
                     a.view(8, 12, N, E), b.view(8, 12, N, E), c.view(8, 12, N, E)).view(BH, N, E)

@@ -274,6 +274,35 @@ int spx_attention_backward_kv(int dtype, const void* grad_out, const void* q, co
                               const int32_t* col_ptr, const void* bcsc_idx, int idx_kind, float inv_temperature,
                               int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
 
+/* Training path that keeps no probabilities.  spx_attention_forward_lse is
+ * spx_attention_forward (pipelined kernel) that also records, per query, the log2-domain
+ * log-sum-exp of its score row (row_lse, float [batch, Nt]; +inf for a row without a live
+ * entry): probs = exp2(score * inv_temperature * log2(e) - row_lse).  The two backward entry
+ * points recompute the probabilities of every live block from q, k and row_lse instead of
+ * reading them: spx_attention_backward_q gives grad_q and row_dot (as
+ * spx_attention_backward_scores does, which it replaces together with the probability buffer),
+ * spx_attention_backward_kv_recompute gives grad_k and grad_v (as spx_attention_backward_kv).
+ * Against the reference's backward chain (sparse_attention.py:76-80 run in reverse: five
+ * launches, probabilities and score gradients written and re-read) the whole step reads and
+ * writes only q, k, v, out, grad_out and the three gradients.  Block-level masks only (every
+ * element of a live block attends): element masks go through spx_attention_forward_train.
+ * 16-bit types; block shapes as spx_attention_forward_train, the column side also BH <= 2 * BW. */
+int spx_attention_forward_lse(int dtype, const void* q, const void* k, const void* v, void* out,
+                              float* row_lse, const int32_t* row_ptr, const int32_t* bcsr_idx,
+                              const uint8_t* mask, float inv_temperature,
+                              int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
+int spx_attention_backward_q(int dtype, const void* grad_out, const void* out, const void* q,
+                             const void* k, const void* v, const float* row_lse,
+                             void* grad_q, float* row_dot,
+                             const int32_t* row_ptr, const int32_t* bcsr_idx, float inv_temperature,
+                             int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
+int spx_attention_backward_kv_recompute(int dtype, const void* grad_out, const void* q, const void* k,
+                                        const void* v, const float* row_lse, const float* row_dot,
+                                        void* grad_k, void* grad_v,
+                                        const int32_t* col_ptr, const void* bcsc_idx, int idx_kind,
+                                        float inv_temperature,
+                                        int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream);
+
 /* ------------------------------------------------------------------------ *
  * Sequence-length attention: q, k, v, out are [batch, heads, N, E]; batch b
  * attends over its first seqlens[b] positions only (int32 [batch], on the

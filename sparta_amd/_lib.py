@@ -56,6 +56,9 @@ _SIGNATURES = {
     'spx_attention_forward_train': (_I, [_I, _P, _P, _P, _P, _P, _L, _P, _P, _P, _F, _I, _I, _I, _I, _I, _I, _P]),
     'spx_attention_backward_scores': (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _F, _I, _I, _I, _I, _I, _I, _P]),
     'spx_attention_backward_kv': (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P]),
+    'spx_attention_forward_lse': (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _I, _P]),
+    'spx_attention_backward_q': (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _I, _P]),
+    'spx_attention_backward_kv_recompute': (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P]),
     'spx_attention_seqlen_forward': (_I, [_I, _P, _P, _P, _P, _P, _F, _I, _I, _I, _I, _I, _P]),
     'spx_moe_index_workspace_bytes': (_Z, [_I, _I]),
     'spx_moe_index': (_I, [_P, _I, _I, _P, _P, _P, _P, _Z, _P]),

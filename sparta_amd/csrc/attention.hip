@@ -44,6 +44,7 @@ struct AttnParams {
     void* grad_v;
     const int32_t* seqlens;   // sequence-length mode of the pipelined kernel: one length per `heads` entries
     int heads;
+    float* row_lse;       // log2-domain log-sum-exp per query: written by the forward kernel, read by the recomputing backward kernels
 };
 
 template <typename T> struct AttnMma;
@@ -481,6 +482,10 @@ __global__ __launch_bounds__(64 * WAVES, waves_per_simd_for((2 * BW * (E * 4 + 3
     // every accumulator row of lacc holds the row sum of query r16
     const float l_run = lacc[0];
     const float inv_l = (l_run > 0.f && (!SEQ || qrow < seq_len)) ? 1.f / l_run : 0.f;
+    // log2-domain log-sum-exp of the row: P = exp2(score - row_lse) reproduces the normalised
+    // probabilities in a backward pass that keeps no copy of them (+inf: no live entry, P = 0)
+    if (p.row_lse && g4 == 0)
+        p.row_lse[b * p.Nt + qrow] = l_run > 0.f ? __builtin_amdgcn_logf(l_run) - negm[0] : __builtin_inff();
     uint64_t pieces[ET];
 #pragma unroll
     for (int t = 0; t < ET; ++t) {
@@ -1163,6 +1168,239 @@ static int launch_attention_bwd_row(const AttnParams& p, int batch, int BW, int 
     return fail(SPX_E_CONFIG, "the attention backward kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
 }
 
+// ---- backward pass without stored probabilities, row side ---------------------------------
+// The forward kernel records one number per query, the log2-domain log-sum-exp L of its row;
+// P = exp2(S - L) then reproduces the normalised probabilities wherever they are needed, and
+// neither P nor dS ever goes to memory.  Per live block a wavefront computes, for its 16
+// queries,  (S - L)^T = K Q^T  (accumulators started at -L, Q scaled by log2(e) / T),
+// (dP - D)^T / T = V dO^T  (accumulators started at -D / T, dO scaled by 1 / T),
+// dS^T = exp2(S - L) o (dP - D) / T  as the B operand of  dQ^T += K^T dS^T.
+// V is staged for row reads; K in rows padded for the transpose reads of the last product,
+// which the row reads of the first product share (rows r and r + 8 fall on the same banks:
+// eight two-way conflicts per block against sixteen transpose reads).  Block-level masks only
+// (an element mask would have to be re-applied here); the K / V tiles of step i + 2 are
+// requested while step i runs, as in attention_bwd_row_kernel.
+template <typename T, int BW, int E, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, waves_per_simd_for((2 * BW * (E * 4 + 32) <= 64 * 1024 ? 2 : 1) * BW * (E * 4 + 32), WAVES))
+void attention_bwd_row_rc_kernel(AttnParams p, int nbr, int batch) {
+    constexpr int NT = 64 * WAVES;
+    constexpr int KT = BW / 16, ET = E / 16, EC = E / 32;
+    constexpr int RP = E * 2;                 // pitch of the row-read tile (V): 16-byte chunks XOR-swizzled by row % 8
+    constexpr int TP = E * 2 + 32;            // pitch of the K tile (transpose reads and row reads)
+    constexpr int TILE = BW * (RP + TP);
+    constexpr int NBUF = 2 * TILE <= 64 * 1024 ? 2 : 1;
+    constexpr int VPR = E / 8;
+    constexpr int NV = BW * VPR / NT;
+    constexpr int RSTEP = NT / VPR;
+    constexpr int NSTG = 2 * NV * 4 <= 48 ? 2 : 1;   // register stages of the prefetch
+    static_assert(BW * VPR % NT == 0 && NT % VPR == 0 && KT % 2 == 0, "tile does not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    const int L = blockIdx.x;
+    const int slot = L >> 3;
+    const int64_t b = (slot / nbr) * 8 + (L & 7);
+    const int br = slot % nbr;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* dO = reinterpret_cast<const T*>(p.grad_out) + b * (int64_t)p.Nt * E;
+    const T* O = reinterpret_cast<const T*>(p.out) + b * (int64_t)p.Nt * E;
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.Nt * E;
+    const T* Kg = reinterpret_cast<const T*>(p.k) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    const T* Vg = reinterpret_cast<const T*>(p.v) + b * (int64_t)p.Ns * E + threadIdx.x * 8;
+    T* dQ = reinterpret_cast<T*>(p.grad_q) + b * (int64_t)p.Nt * E;
+
+    const int qrow = br * (16 * WAVES) + wave * 16 + r16;
+    const float c2 = p.inv_t * 1.4426950408889634f;
+    Frag gf[EC], qf[EC];   // dO / T and Q * log2(e) / T of this lane's query
+    float d_part = 0.f;
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        const Frag g_raw = Mma32<T>::load(dO + (int64_t)qrow * E + c * 32 + g4 * 8);
+        const Frag o_raw = Mma32<T>::load(O + (int64_t)qrow * E + c * 32 + g4 * 8);
+        const Frag q_raw = Mma32<T>::load(Q + (int64_t)qrow * E + c * 32 + g4 * 8);
+        f32x8 gs, qs;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            gs[j] = (float)g_raw[j] * p.inv_t;
+            qs[j] = (float)q_raw[j] * c2;
+            d_part += gs[j] * (float)o_raw[j];
+        }
+        gf[c] = AttnPack<T>::pack(gs);
+        qf[c] = AttnPack<T>::pack(qs);
+    }
+    const float d_row = xor32_sum(xor16_sum(d_part));
+    if (p.row_dot && g4 == 0) p.row_dot[b * p.Nt + qrow] = d_row;
+    const float lse = p.row_lse[b * p.Nt + qrow];
+    const f32x4 negd = f32x4{-d_row, -d_row, -d_row, -d_row};
+    const f32x4 negl = f32x4{-lse, -lse, -lse, -lse};
+
+    f32x4 qacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) qacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int st_row = threadIdx.x / VPR, st_chunk = threadIdx.x % VPR;
+    const int r_dst = st_row * RP + (st_chunk ^ (st_row & 7)) * 16;     // V tile
+    const int t_dst = BW * RP + st_row * TP + st_chunk * 16;            // K tile
+    const int r_src = r16 * RP;
+    const int r_sw = r16 & 7;
+    const int k_src = BW * RP + r16 * TP + g4 * 16;                     // K rows as A operand of the scores
+    const int t_src = BW * RP + (g4 * 4 + (r16 >> 2)) * TP + (r16 & 3) * 8;
+
+    const int e_begin = p.row_ptr[br];
+    const int n_blk = p.row_ptr[br + 1] - e_begin;
+    // block columns of the row: lane l holds entry l; longer rows read the rest from the index
+    int bc_vec = 0;
+    if (lane < n_blk) bc_vec = p.bcsr_idx[e_begin + lane] & 0xffff;
+    auto col_at = [&](int i) {
+        return i < 64 ? __builtin_amdgcn_readlane(bc_vec, i) : (p.bcsr_idx[e_begin + i] & 0xffff);
+    };
+    auto issue = [&](int i, u32x4 (&vr)[NV], u32x4 (&kr)[NV]) {
+        const int64_t off = (int64_t)col_at(i) * BW * E;
+        if constexpr (NSTG == 2) {
+#pragma unroll
+            for (int i2 = 0; i2 < NV; ++i2)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(vr[i2]) : "v"(Vg + off + i2 * NT * 8) : "memory");
+#pragma unroll
+            for (int i2 = 0; i2 < NV; ++i2)
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kr[i2]) : "v"(Kg + off + i2 * NT * 8) : "memory");
+        } else {
+#pragma unroll
+            for (int i2 = 0; i2 < NV; ++i2) vr[i2] = *reinterpret_cast<const u32x4*>(Vg + off + i2 * NT * 8);
+#pragma unroll
+            for (int i2 = 0; i2 < NV; ++i2) kr[i2] = *reinterpret_cast<const u32x4*>(Kg + off + i2 * NT * 8);
+        }
+    };
+    auto wait_stage = [&](int i, u32x4 (&vr)[NV], u32x4 (&kr)[NV]) {
+        if constexpr (NSTG == 1) return;   // plain loads: the compiler waits where the registers are used
+        if (i + 1 < n_blk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NV) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) asm volatile("" : "+v"(vr[i2]));
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) asm volatile("" : "+v"(kr[i2]));
+    };
+    auto step = [&](int i, u32x4 (&vr)[NV], u32x4 (&kr)[NV]) {
+        char* buf = smem + (NBUF == 2 ? (i & 1) * TILE : 0);
+        if constexpr (NBUF == 1) __syncthreads();
+        wait_stage(i, vr, kr);
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) *reinterpret_cast<u32x4*>(buf + r_dst + i2 * RSTEP * RP) = vr[i2];
+#pragma unroll
+        for (int i2 = 0; i2 < NV; ++i2) *reinterpret_cast<u32x4*>(buf + t_dst + i2 * RSTEP * TP) = kr[i2];
+        if (i + NSTG < n_blk) issue(i + NSTG, vr, kr);
+        __syncthreads();
+
+        // ---- (S - L)^T and (dP - D)^T / T tiles: keys x this wave's 16 queries -----------------
+        f32x4 s[KT], dp[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            s[kt] = negl;
+            dp[kt] = negd;
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag kf = *reinterpret_cast<const Frag*>(buf + k_src + kt * 16 * TP + c * 64);
+                s[kt] = Mma32<T>::mma(kf, qf[c], s[kt]);
+                const Frag vf = *reinterpret_cast<const Frag*>(buf + r_src + kt * 16 * RP + (((c * 4 + g4) ^ r_sw) * 16));
+                dp[kt] = Mma32<T>::mma(vf, gf[c], dp[kt]);
+            }
+        }
+        Frag sf[KT / 2];
+#pragma unroll
+        for (int kp = 0; kp < KT / 2; ++kp) {
+            f32x8 ds;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int kt = 2 * kp + (j >> 2), q = j & 3;
+                ds[j] = __builtin_amdgcn_exp2f(s[kt][q]) * dp[kt][q];
+            }
+            sf[kp] = AttnPack<T>::pack(ds);
+        }
+        // ---- dQ^T[e][query] += K^T dS^T ------------------------------------------------------
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int kp = 0; kp < KT / 2; ++kp) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + t_src + (kp * 32) * TP + t * 32));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (lds_s16x4*)(buf + t_src + (kp * 32 + 16) * TP + t * 32));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                qacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, both), sf[kp], qacc[t]);
+            }
+        }
+    };
+    if constexpr (NSTG == 2) {
+        u32x4 v0[NV], k0[NV], v1[NV], k1[NV];
+        if (n_blk > 0) {
+            issue(0, v0, k0);
+            issue(n_blk > 1 ? 1 : 0, v1, k1);   // a row of one block requests it twice; the copy is not used
+        }
+        for (int i = 0; i < n_blk; i += 2) {
+            step(i, v0, k0);
+            if (i + 1 < n_blk) step(i + 1, v1, k1);
+        }
+    } else {
+        u32x4 v0[NV], k0[NV];
+        if (n_blk > 0) issue(0, v0, k0);
+        for (int i = 0; i < n_blk; ++i) step(i, v0, k0);
+    }
+    uint64_t pieces[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T vals[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vals[q] = Elem<T>::from_float(qacc[t][q]);
+        pieces[t] = *reinterpret_cast<const uint64_t*>(vals);
+    }
+    if constexpr (WAVES * 16 * (E * 2 + 16) <= NBUF * TILE) {
+        __syncthreads();   // the K / V tiles are dead: their space carries the output tiles
+        wave_rows_store<E>(smem + wave * (16 * (E * 2 + 16)), dQ + (int64_t)(qrow - r16) * E, pieces);
+    } else {
+#pragma unroll
+        for (int t = 0; t < ET; ++t) *reinterpret_cast<uint64_t*>(dQ + (int64_t)qrow * E + t * 16 + g4 * 4) = pieces[t];
+    }
+}
+
+template <typename T, int BW, int E, int WAVES>
+static int launch_attention_bwd_row_rc_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr int TILE = BW * (E * 4 + 32);
+    constexpr size_t smem = 2 * TILE <= 64 * 1024 ? 2 * TILE : TILE;
+    const int nbr = p.Nt / p.BH;
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbr;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_row_rc_kernel<T, BW, E, WAVES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_bwd_row_rc_kernel)");
+    }
+    hipLaunchKernelGGL((attention_bwd_row_rc_kernel<T, BW, E, WAVES>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbr, batch);
+    SPX_LAUNCH_CHECK("attention_bwd_row_rc_kernel");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_bwd_row_rc(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTNR_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_bwd_row_rc_inst<T, bw, e, bh / 16>(p, batch, st);
+    SPX_ATTNR_CASE(32, 32, 64) SPX_ATTNR_CASE(32, 64, 64) SPX_ATTNR_CASE(32, 128, 64)
+    SPX_ATTNR_CASE(32, 32, 128) SPX_ATTNR_CASE(32, 64, 128) SPX_ATTNR_CASE(32, 128, 128)
+    SPX_ATTNR_CASE(64, 32, 64) SPX_ATTNR_CASE(64, 64, 64) SPX_ATTNR_CASE(64, 128, 64)
+    SPX_ATTNR_CASE(64, 32, 128) SPX_ATTNR_CASE(64, 64, 128) SPX_ATTNR_CASE(64, 128, 128)
+    SPX_ATTNR_CASE(128, 64, 64) SPX_ATTNR_CASE(128, 128, 64)
+    SPX_ATTNR_CASE(128, 32, 128) SPX_ATTNR_CASE(128, 64, 128) SPX_ATTNR_CASE(128, 128, 128)
+#undef SPX_ATTNR_CASE
+    return fail(SPX_E_CONFIG, "the attention backward kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
 // ---- backward pass, column side: gradients of the keys and of the values -------------------
 //   dV = P^T dO,   dK = dS^T Q,   dS = P o (dO V^T - D) / T  (recomputed here from P)
 // One workgroup per block column (BW keys) and batch entry, one wavefront per 16 keys, walking
@@ -1358,6 +1596,189 @@ __global__ __launch_bounds__(64 * WAVES, (BH * E <= 64 * 64 || BH == 32) ? 3 : (
     }
 }
 
+// ---- backward pass without stored probabilities, column side -------------------------------
+// As attention_bwd_col_kernel, with the probabilities recomputed instead of read: per live
+// block of the column, from the dO and Q tiles of the query block (rows padded for transpose
+// reads, read as rows for the first two products) and the K and V rows of this wavefront's 16
+// keys in registers,
+//   S - L = Q K^T   (K scaled by log2(e) / T, accumulators started at -L, the log2-domain
+//                    log-sum-exp of the query row recorded by the forward kernel),
+//   (dP - D) / T = dO V^T   (V scaled by 1 / T, accumulators started at -D / T),
+//   P = exp2(S - L),  dS = P o (dP - D) / T,  both already in the B-operand layout of
+//   dK^T += Q^T dS  and  dV^T += dO^T P.
+// L and D of the block's queries pass through LDS (one float per thread).  Block-level masks
+// only.
+template <typename T, int BH, int E, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, (BH * E <= 64 * 64 || BH == 32) ? 3 : (BH * E <= 128 * 64 ? 2 : 1))
+void attention_bwd_col_rc_kernel(AttnParams p, int nbc, int batch) {
+    constexpr int BW = 16 * WAVES;
+    constexpr int NT = 64 * WAVES;
+    constexpr int QT = BH / 16, ET = E / 16, EC = E / 32;
+    constexpr int DP = E * 2 + 32;            // row pitch of the dO and Q tiles
+    constexpr int Q_OFF = BH * DP, S_OFF = 2 * BH * DP;   // S_OFF: BH values of L, then BH of D / T
+    constexpr int VPR = E / 8;                // 16-byte vectors per row
+    constexpr int NVD = BH * VPR / NT;        // vectors per thread: dO / Q tile
+    static_assert(BH * VPR % NT == 0 && QT % 2 == 0 && 2 * BH <= NT, "tiles do not split over the workgroup");
+    typedef typename Mma32<T>::frag Frag;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    typedef float f32x8 __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    extern __shared__ __align__(16) char smem[];
+
+    const int L = blockIdx.x;
+    const int slot_l = L >> 3;
+    const int64_t b = (slot_l / nbc) * 8 + (L & 7);
+    const int j = slot_l % nbc;
+    if (b >= batch) return;
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g4 = lane >> 4;
+
+    const T* dO = reinterpret_cast<const T*>(p.grad_out) + b * (int64_t)p.Nt * E + threadIdx.x * 8;
+    const T* Q = reinterpret_cast<const T*>(p.q) + b * (int64_t)p.Nt * E + threadIdx.x * 8;
+    // thread t < BH fetches L of query t of the block, thread BH + t its D / T
+    const float* stat = (threadIdx.x < BH ? p.row_lse : p.row_dot) + b * (int64_t)p.Nt + (threadIdx.x % BH);
+    T* dK = reinterpret_cast<T*>(p.grad_k) + b * (int64_t)p.Ns * E;
+    T* dV = reinterpret_cast<T*>(p.grad_v) + b * (int64_t)p.Ns * E;
+
+    const int krow = j * BW + wave * 16 + r16;
+    const float c2 = p.inv_t * 1.4426950408889634f;
+    Frag vf[EC], kf[EC];     // V / T and K * log2(e) / T of this lane's key
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+        const Frag v_raw = Mma32<T>::load(reinterpret_cast<const T*>(p.v) + (b * (int64_t)p.Ns + krow) * E + c * 32 + g4 * 8);
+        const Frag k_raw = Mma32<T>::load(reinterpret_cast<const T*>(p.k) + (b * (int64_t)p.Ns + krow) * E + c * 32 + g4 * 8);
+        f32x8 vs, ks;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            vs[x] = (float)v_raw[x] * p.inv_t;
+            ks[x] = (float)k_raw[x] * c2;
+        }
+        vf[c] = AttnPack<T>::pack(vs);
+        kf[c] = AttnPack<T>::pack(ks);
+    }
+
+    f32x4 kacc[ET], vacc[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) kacc[t] = vacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // staging map (a tile is contiguous in memory: vector v = tid + i * NT is row v / VPR)
+    const int d_dst = (threadIdx.x / VPR) * DP + (threadIdx.x % VPR) * 16;
+    constexpr int D_RSTEP = NT / VPR;
+    static_assert(NT % VPR == 0, "rows per pass");
+    const int a_src = r16 * DP + g4 * 16;                                    // dO / Q rows as A operands
+    const int t_src = (g4 * 4 + (r16 >> 2)) * DP + (r16 & 3) * 8;            // transpose reads of dO / Q
+    const bool has_stat = threadIdx.x < 2 * BH;
+
+    const int e_begin = p.col_ptr[j];
+    const int e_end = p.col_ptr[j + 1];
+    auto query_block = [&](int e) {
+        return p.bcsc_wide ? (int)(reinterpret_cast<const long long*>(p.bcsc_idx)[e] & 0xffff)
+                           : (reinterpret_cast<const int32_t*>(p.bcsc_idx)[e] & 0xffff);
+    };
+    u32x4 do_r[NVD], q_r[NVD];
+    float st_r = 0.f;
+    auto issue = [&](int qb) {
+        const int64_t off = (int64_t)qb * BH * E;
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) do_r[i] = *reinterpret_cast<const u32x4*>(dO + off + i * NT * 8);
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) q_r[i] = *reinterpret_cast<const u32x4*>(Q + off + i * NT * 8);
+        if (has_stat) st_r = stat[qb * BH];
+    };
+    int qb = 0, qb_next = 0;
+    if (e_begin < e_end) {
+        qb = query_block(e_begin);
+        qb_next = query_block(e_begin + 1 < e_end ? e_begin + 1 : e_begin);
+        issue(qb);
+    }
+    for (int e = e_begin; e < e_end; ++e) {
+        __syncthreads();   // everyone is done with the previous tiles
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) *reinterpret_cast<u32x4*>(smem + d_dst + i * D_RSTEP * DP) = do_r[i];
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) *reinterpret_cast<u32x4*>(smem + Q_OFF + d_dst + i * D_RSTEP * DP) = q_r[i];
+        if (has_stat) *reinterpret_cast<float*>(smem + S_OFF + threadIdx.x * 4) = st_r;
+        // next live block of the column (the last step re-reads its own block; the copy is not used)
+        qb = qb_next;
+        qb_next = query_block(e + 2 < e_end ? e + 2 : e_end - 1);
+        issue(qb);
+        __syncthreads();
+
+        // ---- S - L and (dP - D) / T: 16 queries x this wave's 16 keys per tile -----------------
+        f32x4 s[QT], dp[QT];
+#pragma unroll
+        for (int t = 0; t < QT; ++t) {
+            s[t] = -*reinterpret_cast<const f32x4*>(smem + S_OFF + (t * 16 + g4 * 4) * 4);
+            dp[t] = -*reinterpret_cast<const f32x4*>(smem + S_OFF + (BH + t * 16 + g4 * 4) * 4);
+#pragma unroll
+            for (int c = 0; c < EC; ++c) {
+                const Frag qa = *reinterpret_cast<const Frag*>(smem + Q_OFF + a_src + t * 16 * DP + c * 64);
+                s[t] = Mma32<T>::mma(qa, kf[c], s[t]);
+                const Frag ga = *reinterpret_cast<const Frag*>(smem + a_src + t * 16 * DP + c * 64);
+                dp[t] = Mma32<T>::mma(ga, vf[c], dp[t]);
+            }
+        }
+        // ---- P = exp2(S - L), dS = P o (dP - D) / T: both as B operands ------------------------
+        Frag pf[QT / 2], sf[QT / 2];
+#pragma unroll
+        for (int kp = 0; kp < QT / 2; ++kp) {
+            f32x8 pv, ds;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                pv[x] = __builtin_amdgcn_exp2f(s[2 * kp + (x >> 2)][x & 3]);
+                ds[x] = pv[x] * dp[2 * kp + (x >> 2)][x & 3];
+            }
+            pf[kp] = AttnPack<T>::pack(pv);
+            sf[kp] = AttnPack<T>::pack(ds);
+        }
+        // ---- dK^T[e][key] += Q^T dS,  dV^T[e][key] += dO^T P ----------------------------------
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+#pragma unroll
+            for (int kp = 0; kp < QT / 2; ++kp) {
+                const s16x4 qlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + Q_OFF + t_src + (kp * 32) * DP + t * 32));
+                const s16x4 qhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + Q_OFF + t_src + (kp * 32 + 16) * DP + t * 32));
+                const s16x8 qa = __builtin_shufflevector(qlo, qhi, 0, 1, 2, 3, 4, 5, 6, 7);
+                kacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, qa), sf[kp], kacc[t]);
+                const s16x4 glo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + t_src + (kp * 32) * DP + t * 32));
+                const s16x4 ghi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(smem + t_src + (kp * 32 + 16) * DP + t * 32));
+                const s16x8 ga = __builtin_shufflevector(glo, ghi, 0, 1, 2, 3, 4, 5, 6, 7);
+                vacc[t] = Mma32<T>::mma(__builtin_bit_cast(Frag, ga), pf[kp], vacc[t]);
+            }
+        }
+    }
+
+    // lane holds dK^T[e = 16 t + 4 g4 + q][key r16] (and dV^T): rows of 16 keys per wave
+    uint64_t kp_[ET], vp_[ET];
+#pragma unroll
+    for (int t = 0; t < ET; ++t) {
+        T kv[4], vv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            kv[q] = Elem<T>::from_float(kacc[t][q]);
+            vv[q] = Elem<T>::from_float(vacc[t][q]);
+        }
+        kp_[t] = *reinterpret_cast<const uint64_t*>(kv);
+        vp_[t] = *reinterpret_cast<const uint64_t*>(vv);
+    }
+    const int64_t row0 = (int64_t)(krow - r16) * E;
+    if constexpr (WAVES * 16 * (E * 2 + 16) <= 2 * BH * DP) {
+        __syncthreads();   // the tiles are dead: their space carries the output tiles
+        char* tile = smem + wave * (16 * (E * 2 + 16));
+        wave_rows_store<E>(tile, dK + row0, kp_);
+        wave_rows_store<E>(tile, dV + row0, vp_);
+    } else {
+#pragma unroll
+        for (int t = 0; t < ET; ++t) {
+            *reinterpret_cast<uint64_t*>(dK + row0 + (int64_t)r16 * E + t * 16 + g4 * 4) = kp_[t];
+            *reinterpret_cast<uint64_t*>(dV + row0 + (int64_t)r16 * E + t * 16 + g4 * 4) = vp_[t];
+        }
+    }
+}
+
 // Query blocks of 32 / 64 / 128, key blocks of 32 / 64 / 128, head dims 64 / 128, with at
 // least one vector of the dO tile per thread.
 static bool attention_bwd_col_supported(int BH, int BW, int E) {
@@ -1392,6 +1813,41 @@ static int launch_attention_bwd_col(const AttnParams& p, int batch, int BW, int 
     SPX_ATTNC_CASE(128, 32, 64) SPX_ATTNC_CASE(128, 64, 64) SPX_ATTNC_CASE(128, 128, 64)
     SPX_ATTNC_CASE(128, 32, 128) SPX_ATTNC_CASE(128, 64, 128) SPX_ATTNC_CASE(128, 128, 128)
 #undef SPX_ATTNC_CASE
+    return fail(SPX_E_CONFIG, "the key / value gradient kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
+}
+
+// The recomputing column-side kernel also needs a thread per row statistic: BH <= 2 * BW.
+static bool attention_bwd_col_rc_supported(int BH, int BW, int E) {
+    return attention_bwd_col_supported(BH, BW, E) && BH <= 2 * BW;
+}
+
+template <typename T, int BH, int E, int WAVES>
+static int launch_attention_bwd_col_rc_inst(const AttnParams& p, int batch, hipStream_t st) {
+    constexpr size_t smem = 2 * BH * (E * 2 + 32) + 2 * BH * 4;
+    const int nbc = p.Ns / (16 * WAVES);
+    const int64_t groups = ((int64_t)batch + 7) / 8 * 8 * nbc;
+    if (groups > 0x7fffffff) return fail(SPX_E_SHAPE, "too many workgroups (%lld)", (long long)groups);
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_bwd_col_rc_kernel<T, BH, E, WAVES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(attention_bwd_col_rc_kernel)");
+    }
+    hipLaunchKernelGGL((attention_bwd_col_rc_kernel<T, BH, E, WAVES>), dim3((unsigned)groups), dim3(64 * WAVES), smem, st, p, nbc, batch);
+    SPX_LAUNCH_CHECK("attention_bwd_col_rc_kernel");
+    return 0;
+}
+
+template <typename T>
+static int launch_attention_bwd_col_rc(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
+#define SPX_ATTNCR_CASE(bh, bw, e) \
+    if (p.BH == bh && BW == bw && E == e) return launch_attention_bwd_col_rc_inst<T, bh, e, bw / 16>(p, batch, st);
+    SPX_ATTNCR_CASE(32, 32, 64) SPX_ATTNCR_CASE(32, 64, 64)
+    SPX_ATTNCR_CASE(32, 32, 128) SPX_ATTNCR_CASE(32, 64, 128) SPX_ATTNCR_CASE(32, 128, 128)
+    SPX_ATTNCR_CASE(64, 32, 64) SPX_ATTNCR_CASE(64, 64, 64) SPX_ATTNCR_CASE(64, 128, 64)
+    SPX_ATTNCR_CASE(64, 32, 128) SPX_ATTNCR_CASE(64, 64, 128) SPX_ATTNCR_CASE(64, 128, 128)
+    SPX_ATTNCR_CASE(128, 64, 64) SPX_ATTNCR_CASE(128, 128, 64)
+    SPX_ATTNCR_CASE(128, 64, 128) SPX_ATTNCR_CASE(128, 128, 128)
+#undef SPX_ATTNCR_CASE
     return fail(SPX_E_CONFIG, "the key / value gradient kernel does not cover blocks (%d,%d) with head dim %d", p.BH, BW, E);
 }
 
@@ -1830,12 +2286,12 @@ static int launch_attention_seqlen(const SeqlenParams& p, int batch_heads, int E
 
 }  // namespace spx
 
-extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, const void* v, void* out,
-                                     const int32_t* row_ptr, const int32_t* bcsr_idx,
-                                     const uint8_t* mask, float inv_temperature,
-                                     int batch, int Nt, int Ns, int E, int BH, int BW,
-                                     int tile_cfg, spx_stream_t stream) {
-    using namespace spx;
+namespace spx {
+static int attention_forward_impl(int dtype, const void* q, const void* k, const void* v, void* out, float* row_lse,
+                                  const int32_t* row_ptr, const int32_t* bcsr_idx,
+                                  const uint8_t* mask, float inv_temperature,
+                                  int batch, int Nt, int Ns, int E, int BH, int BW,
+                                  int tile_cfg, spx_stream_t stream) {
     SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
                 "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
@@ -1848,7 +2304,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
                 "q, k, v, out must be 16-byte aligned");
     SPX_REQUIRE(!mask || (Ns % 4 == 0 && aligned(mask, 4)), SPX_E_ALIGN, "mask rows must be 4-byte aligned");
     if (batch == 0) return 0;
-    AttnParams p;
+    AttnParams p = {};
     p.q = q; p.k = k; p.v = v; p.out = out;
     p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx; p.mask = mask;
     p.inv_t = inv_temperature;
@@ -1856,7 +2312,7 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     p.probs = nullptr; p.probs_batch = 0;
     p.grad_out = nullptr; p.grad_scores = nullptr; p.grad_q = nullptr; p.row_dot = nullptr;
     p.col_ptr = nullptr; p.bcsc_idx = nullptr; p.bcsc_wide = 0; p.grad_k = nullptr; p.grad_v = nullptr;
-    p.seqlens = nullptr; p.heads = 1;
+    p.seqlens = nullptr; p.heads = 1; p.row_lse = row_lse;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     // tile_cfg 0: the pipelined kernel where it applies; 1: one-buffer kernel; 2: pipelined kernel;
     // 3: pipelined kernel on 32x32x16 MFMAs (one wavefront per 32 queries; measured within a few
@@ -1872,6 +2328,28 @@ extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, co
     }
     if (dtype == SPX_F16) return launch_attention<_Float16>(p, batch, BW, E, st);
     return launch_attention<bf16_t>(p, batch, BW, E, st);
+}
+}  // namespace spx
+
+extern "C" int spx_attention_forward(int dtype, const void* q, const void* k, const void* v, void* out,
+                                     const int32_t* row_ptr, const int32_t* bcsr_idx,
+                                     const uint8_t* mask, float inv_temperature,
+                                     int batch, int Nt, int Ns, int E, int BH, int BW,
+                                     int tile_cfg, spx_stream_t stream) {
+    return spx::attention_forward_impl(dtype, q, k, v, out, nullptr, row_ptr, bcsr_idx, mask, inv_temperature,
+                                       batch, Nt, Ns, E, BH, BW, tile_cfg, stream);
+}
+
+extern "C" int spx_attention_forward_lse(int dtype, const void* q, const void* k, const void* v, void* out,
+                                         float* row_lse, const int32_t* row_ptr, const int32_t* bcsr_idx,
+                                         const uint8_t* mask, float inv_temperature,
+                                         int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(row_lse && aligned(row_lse, 4), SPX_E_NULL, "row_lse is required");
+    SPX_REQUIRE(attention_v2_supported(BH, BW, E), SPX_E_CONFIG,
+                "the forward kernel that records the row statistic covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 (got %d, %d, %d)", BH, BW, E);
+    return attention_forward_impl(dtype, q, k, v, out, row_lse, row_ptr, bcsr_idx, mask, inv_temperature,
+                                  batch, Nt, Ns, E, BH, BW, 2, stream);
 }
 
 extern "C" int spx_attention_forward_train(int dtype, const void* q, const void* k, const void* v, void* out,
@@ -1894,7 +2372,7 @@ extern "C" int spx_attention_forward_train(int dtype, const void* q, const void*
     SPX_REQUIRE(probs_batch_stride % 8 == 0, SPX_E_ALIGN, "probs_batch_stride must be a multiple of 8 elements");
     SPX_REQUIRE(!mask || (Ns % 4 == 0 && aligned(mask, 4)), SPX_E_ALIGN, "mask rows must be 4-byte aligned");
     if (batch == 0) return 0;
-    AttnParams p;
+    AttnParams p = {};
     p.q = q; p.k = k; p.v = v; p.out = out;
     p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx; p.mask = mask;
     p.inv_t = inv_temperature;
@@ -1972,6 +2450,69 @@ extern "C" int spx_attention_backward_kv(int dtype, const void* grad_out, const 
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     if (dtype == SPX_F16) return launch_attention_bwd_col<_Float16>(p, batch, BW, E, st);
     return launch_attention_bwd_col<bf16_t>(p, batch, BW, E, st);
+}
+
+extern "C" int spx_attention_backward_q(int dtype, const void* grad_out, const void* out, const void* q,
+                                        const void* k, const void* v, const float* row_lse,
+                                        void* grad_q, float* row_dot,
+                                        const int32_t* row_ptr, const int32_t* bcsr_idx, float inv_temperature,
+                                        int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
+                "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
+    SPX_REQUIRE(grad_out && out && q && k && v && row_lse && grad_q && row_ptr && bcsr_idx, SPX_E_NULL,
+                "a required buffer is NULL");
+    SPX_REQUIRE(Nt > 0 && Ns > 0 && BH > 0 && BW > 0 && Nt % BH == 0 && Ns % BW == 0, SPX_E_SHAPE,
+                "mask shape (%d,%d) is not a multiple of the block (%d,%d)", Nt, Ns, BH, BW);
+    SPX_REQUIRE(attention_v2_supported(BH, BW, E), SPX_E_CONFIG,
+                "the attention backward kernel covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 (got %d, %d, %d)", BH, BW, E);
+    SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
+    SPX_REQUIRE(aligned(grad_out, 16) && aligned(out, 16) && aligned(q, 16) && aligned(k, 16) && aligned(v, 16) &&
+                aligned(grad_q, 16) && aligned(row_lse, 4) && aligned(row_dot, 4), SPX_E_ALIGN,
+                "buffers must be 16-byte aligned");
+    if (batch == 0) return 0;
+    AttnParams p = {};
+    p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out);
+    p.row_ptr = row_ptr; p.bcsr_idx = bcsr_idx;
+    p.inv_t = inv_temperature;
+    p.Nt = Nt; p.Ns = Ns; p.BH = BH;
+    p.grad_out = grad_out; p.grad_q = grad_q; p.row_dot = row_dot; p.row_lse = const_cast<float*>(row_lse);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (dtype == SPX_F16) return launch_attention_bwd_row_rc<_Float16>(p, batch, BW, E, st);
+    return launch_attention_bwd_row_rc<bf16_t>(p, batch, BW, E, st);
+}
+
+extern "C" int spx_attention_backward_kv_recompute(int dtype, const void* grad_out, const void* q, const void* k,
+                                                   const void* v, const float* row_lse, const float* row_dot,
+                                                   void* grad_k, void* grad_v,
+                                                   const int32_t* col_ptr, const void* bcsc_idx, int idx_kind,
+                                                   float inv_temperature,
+                                                   int batch, int Nt, int Ns, int E, int BH, int BW, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE,
+                "fused attention runs in float16 / bfloat16 (fp32 accumulate); got dtype %d", dtype);
+    SPX_REQUIRE(grad_out && q && k && v && row_lse && row_dot && grad_k && grad_v && col_ptr && bcsc_idx, SPX_E_NULL,
+                "a required buffer is NULL");
+    SPX_REQUIRE(idx_kind == SPX_IDX_BCSC_I32 || idx_kind == SPX_IDX_BCSC_I64, SPX_E_CONFIG,
+                "the key / value gradient kernel walks a BCSC index (got index kind %d)", idx_kind);
+    SPX_REQUIRE(Nt > 0 && Ns > 0 && BH > 0 && BW > 0 && Nt % BH == 0 && Ns % BW == 0, SPX_E_SHAPE,
+                "mask shape (%d,%d) is not a multiple of the block (%d,%d)", Nt, Ns, BH, BW);
+    SPX_REQUIRE(attention_bwd_col_rc_supported(BH, BW, E), SPX_E_CONFIG,
+                "the recomputing key / value gradient kernel covers query blocks 32/64/128, key blocks 32/64/128 and head dims 64/128 with BH * E >= 32 * BW and BH <= 2 * BW (got %d, %d, %d)", BH, BW, E);
+    SPX_REQUIRE(batch >= 0 && batch <= 65535, SPX_E_SHAPE, "batch %d out of range", batch);
+    SPX_REQUIRE(aligned(grad_out, 16) && aligned(q, 16) && aligned(k, 16) && aligned(v, 16) && aligned(row_lse, 4) &&
+                aligned(row_dot, 4) && aligned(grad_k, 16) && aligned(grad_v, 16), SPX_E_ALIGN, "buffers must be 16-byte aligned");
+    if (batch == 0) return 0;
+    AttnParams p = {};
+    p.q = q; p.k = k; p.v = v;
+    p.inv_t = inv_temperature;
+    p.Nt = Nt; p.Ns = Ns; p.BH = BH;
+    p.grad_out = grad_out; p.row_dot = const_cast<float*>(row_dot); p.row_lse = const_cast<float*>(row_lse);
+    p.col_ptr = col_ptr; p.bcsc_idx = bcsc_idx; p.bcsc_wide = idx_kind == SPX_IDX_BCSC_I64;
+    p.grad_k = grad_k; p.grad_v = grad_v;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (dtype == SPX_F16) return launch_attention_bwd_col_rc<_Float16>(p, batch, BW, E, st);
+    return launch_attention_bwd_col_rc<bf16_t>(p, batch, BW, E, st);
 }
 
 extern "C" int spx_attention_seqlen_forward(int dtype, const void* q, const void* k, const void* v, void* out,

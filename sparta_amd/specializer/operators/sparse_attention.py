@@ -60,20 +60,51 @@ class _FusedAttentionFunc(torch.autograd.Function):
         return None, grad_q if need_q else None, grad_k if need_k else None, grad_v if need_v else None
 
 
+class _RecomputeAttentionFunc(torch.autograd.Function):
+    """Training path that keeps no probabilities: the forward kernel records one number per
+    query (the log-sum-exp of its score row), and the row-side and column-side backward
+    kernels recompute the probabilities of every live block from q, k and that number."""
+
+    @staticmethod
+    def forward(ctx, op: 'SparseAttention', query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
+        q, k, v = query.detach().contiguous(), key.detach().contiguous(), value.detach().contiguous()
+        out, row_lse = op._fused_forward_lse(q, k, v)
+        ctx.save_for_backward(q, k, v, out, row_lse)
+        ctx.op = op
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        q, k, v, out, row_lse = ctx.saved_tensors
+        op = ctx.op
+        grad_out = grad_out.detach().contiguous()
+        need_q, need_k, need_v = ctx.needs_input_grad[1:4]
+        grad_q, row_dot = op._recompute_backward_q(grad_out, out, q, k, v, row_lse)
+        grad_k = grad_v = None
+        if need_k or need_v:
+            grad_k, grad_v = op._recompute_backward_kv(grad_out, q, k, v, row_lse, row_dot)
+        return None, grad_q if need_q else None, grad_k if need_k else None, grad_v if need_v else None
+
+
 class SparseAttention(OperatorBase):
     r"""Args:
         mask: (N_target, N_source) mask of the score entries that take part.
         fused: run the single fused forward kernel when autograd is not recording
             (default True).  The three-operator pipeline is always built as well and
             is used whenever gradients are needed.
+        recompute: with a mask that is uniform inside its blocks, train without storing
+            the probabilities (default True): the backward kernels recompute them from
+            q, k and one number per query.  Masks with partly live blocks, and
+            `recompute=False`, keep the probabilities of the live blocks for the backward pass.
         fused_tile_cfg: tile configuration of the fused kernel (0 = the library's choice;
             see spx_tile_cfg_info for the others).
 
     Shape: query (B*H, N_target, E), key / value (B*H, N_source, E) -> (B*H, N_target, E).
     """
 
-    def __init__(self, mask: torch.Tensor, fused: bool = True, fused_tile_cfg: int = 0):
+    def __init__(self, mask: torch.Tensor, fused: bool = True, fused_tile_cfg: int = 0, recompute: bool = True):
         super().__init__()
+        self._recompute = recompute
         self.mask = mask
         self._Nt, self._Ns = mask.shape
         self._matmul_qk = SparseBatchMatMul(C_mask=mask, transpose_A=False, transpose_B=True, compressed=True)
@@ -96,6 +127,8 @@ class SparseAttention(OperatorBase):
             recording = torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)
             if not recording:
                 return self._fused_forward(query, key, value)
+            if self._recompute and self._recompute_supported(query):
+                return _RecomputeAttentionFunc.apply(self, query, key, value)
             if self._fused_train_supported(query):
                 return _FusedAttentionFunc.apply(self, query, key, value)
         scores = self._matmul_qk.forward(query, key)
@@ -111,6 +144,60 @@ class SparseAttention(OperatorBase):
             return False
         ctxs = (self._matmul_qk._sparse_ctx, self._matmul_out._sparse_ctx)
         return all(hasattr(c, 'backward_B') for c in ctxs)
+
+    def _recompute_supported(self, query: torch.Tensor) -> bool:
+        """The kernels that recompute the probabilities cover block-level masks, 3-D 16-bit
+        inputs and the block shapes of both backward kernels, and walk both indexes."""
+        indexes = self._sparse_port.indexes
+        BH, BW, E = indexes.block_H, indexes.block_W, query.shape[-1]
+        return (query.dim() == 3 and BH in (32, 64, 128) and BW in (32, 64, 128) and E in (64, 128)
+                and BW * E // 8 >= BH * 4 and BH * E >= 32 * BW and BH <= 2 * BW
+                and getattr(indexes, 'col_ptr', None) is not None and getattr(indexes, 'row_ptr', None) is not None
+                and self._element_mask() is None)
+
+    def _fused_forward_lse(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+        """(output, log-sum-exp per query) from spx_attention_forward_lse."""
+        indexes = self._sparse_port.indexes
+        batch, _, E = q.shape
+        out = torch.empty_like(q)
+        row_lse = torch.empty((batch, self._Nt), dtype=torch.float32, device=q.device)
+        rc = _lib.load().spx_attention_forward_lse(
+            _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
+            _lib.dev_ptr(row_lse), _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), None,
+            float(self._inv_temperature), batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W,
+            _lib.current_stream(q.device))
+        _lib.check(rc, 'spx_attention_forward_lse')
+        return out, row_lse
+
+    def _recompute_backward_q(self, grad_out, out, q, k, v, row_lse):
+        """(query gradient, row constants) from spx_attention_backward_q."""
+        indexes = self._sparse_port.indexes
+        batch, _, E = grad_out.shape
+        grad_q = torch.empty_like(q)
+        row_dot = torch.empty((batch, self._Nt), dtype=torch.float32, device=q.device)
+        rc = _lib.load().spx_attention_backward_q(
+            _lib.dtype_code(q.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(out), _lib.dev_ptr(q), _lib.dev_ptr(k),
+            _lib.dev_ptr(v), _lib.dev_ptr(row_lse), _lib.dev_ptr(grad_q), _lib.dev_ptr(row_dot),
+            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), float(self._inv_temperature),
+            batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W, _lib.current_stream(q.device))
+        _lib.check(rc, 'spx_attention_backward_q')
+        return grad_q, row_dot
+
+    def _recompute_backward_kv(self, grad_out, q, k, v, row_lse, row_dot):
+        """(key gradient, value gradient) from spx_attention_backward_kv_recompute."""
+        indexes = self._sparse_port.indexes
+        batch, _, E = grad_out.shape
+        grad_k = torch.empty_like(k)
+        grad_v = torch.empty_like(v)
+        idx = indexes._bcsc_buf
+        kind = _lib.IDX_BCSC_I64 if idx.dtype == torch.int64 else _lib.IDX_BCSC_I32
+        rc = _lib.load().spx_attention_backward_kv_recompute(
+            _lib.dtype_code(q.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),
+            _lib.dev_ptr(row_lse), _lib.dev_ptr(row_dot), _lib.dev_ptr(grad_k), _lib.dev_ptr(grad_v),
+            _lib.dev_ptr(indexes.col_ptr), _lib.dev_ptr(idx), kind, float(self._inv_temperature),
+            batch, self._Nt, self._Ns, E, indexes.block_H, indexes.block_W, _lib.current_stream(q.device))
+        _lib.check(rc, 'spx_attention_backward_kv_recompute')
+        return grad_k, grad_v
 
     def _element_mask(self):
         indexes = self._sparse_port.indexes

@@ -175,31 +175,45 @@ def train_config(bh, bw):
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('bh,bw,E', [(64, 64, 64), (32, 64, 64), (64, 32, 128), (64, 64, 128)])
-@pytest.mark.parametrize('gran', [(1, 1), None])
-def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, gpu, H=3, Nt=256, Ns=384):
+@pytest.mark.parametrize('gran,recompute', [((1, 1), True), (None, False), (None, True)])
+def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, recompute, gpu, H=3, Nt=256, Ns=384):
     """With gradients recorded and the backward kernels built, the forward pass is one
-    launch that also writes the probabilities: output and the three gradients agree with
-    the three-operator pipeline and with dense fp32 autograd; empty block rows and (with an
-    element-granular mask) partly masked blocks and fully masked queries included."""
+    launch that also writes the probabilities - or, for a block-level mask with
+    recompute=True, one number per query from which the two backward launches recompute
+    them: output and the three gradients agree with the three-operator pipeline and with
+    dense fp32 autograd; empty block rows and (with an element-granular mask) partly masked
+    blocks and fully masked queries included."""
     _, q = randn((H, Nt, E), 31, dtype)
     _, k = randn((H, Ns, E), 32, dtype)
     _, v = randn((H, Ns, E), 33, dtype)
     _, g = randn((H, Nt, E), 34, dtype)
     mask_np = ops.block_mask((Nt, Ns), gran or (bh, bw), 0.8 if gran else 0.6, seed=35)
     mask_np[:bh] = 0            # an empty block row
-    mask_np[bh + 3] = 0         # a fully masked query inside a live block row
+    block_level = recompute and gran is None
+    if not block_level:
+        mask_np[bh + 3] = 0     # a fully masked query inside a live block row (the mask is then not block-level)
     mask = torch.from_numpy(mask_np).to(gpu)
-    att = SparseAttention(mask=mask)
+    att = SparseAttention(mask=mask, recompute=recompute)
     leaves = [t.to(gpu).requires_grad_(True) for t in (q, k, v)]
     att.build(train_config(bh, bw), sample_inputs=[t.detach() for t in leaves])
     calls = []
-    inner = att._fused_forward_train
-    att._fused_forward_train = lambda *a: (calls.append(1), inner(*a))[1]
     bwd_calls = []
-    inner_bwd = att._fused_backward_scores
-    att._fused_backward_scores = lambda *a, **kw: (bwd_calls.append(1), inner_bwd(*a, **kw))[1]
-    inner_kv = att._fused_backward_kv
-    att._fused_backward_kv = lambda *a: (bwd_calls.append(2), inner_kv(*a))[1]
+    if block_level:   # no probabilities are stored
+        inner = att._fused_forward_lse
+        att._fused_forward_lse = lambda *a: (calls.append(1), inner(*a))[1]
+        inner_bwd = att._recompute_backward_q
+        att._recompute_backward_q = lambda *a: (bwd_calls.append(1), inner_bwd(*a))[1]
+        inner_kv = att._recompute_backward_kv
+        att._recompute_backward_kv = lambda *a: (bwd_calls.append(2), inner_kv(*a))[1]
+        att._fused_forward_train = None
+    else:
+        inner = att._fused_forward_train
+        att._fused_forward_train = lambda *a: (calls.append(1), inner(*a))[1]
+        inner_bwd = att._fused_backward_scores
+        att._fused_backward_scores = lambda *a, **kw: (bwd_calls.append(1), inner_bwd(*a, **kw))[1]
+        inner_kv = att._fused_backward_kv
+        att._fused_backward_kv = lambda *a: (bwd_calls.append(2), inner_kv(*a))[1]
+        att._fused_forward_lse = None
 
     def run(fused):
         att._fused = fused
@@ -224,7 +238,7 @@ def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, gpu, H=3, Nt=
     for name, a, b, c in zip(('out', 'grad_q', 'grad_k', 'grad_v'), got, piped, want):
         torch.testing.assert_close(a, c, rtol=2e-2, atol=2e-2, msg=lambda m: f'{name} vs dense autograd: {m}')
         torch.testing.assert_close(a, b, rtol=2e-2, atol=2e-2, msg=lambda m: f'{name} vs pipeline: {m}')
-    assert float(got[0][:, :bh].abs().max()) == 0.0 and float(got[0][:, bh + 3].abs().max()) == 0.0
+    assert float(got[0][:, :bh].abs().max()) == 0.0 and (block_level or float(got[0][:, bh + 3].abs().max()) == 0.0)
 
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
@@ -298,6 +312,80 @@ def test_attention_backward_scores_kernel(dtype, BH, BW, E, element_mask, gpu, b
     torch.testing.assert_close(indexes.inverse(grad_scores).float(), scores.grad, **tol)
     torch.testing.assert_close(grad_q.float(), qf.grad, **tol)
     assert float(grad_q[:, :BH].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('BH,BW,E', [(32, 32, 64), (32, 128, 64), (64, 64, 64), (64, 128, 128), (128, 64, 64),
+                                     (128, 128, 128), (32, 64, 128), (64, 128, 64), (32, 128, 128),
+                                     (64, 32, 64), (128, 128, 64), (64, 32, 128)])
+def test_attention_recompute_kernels(dtype, BH, BW, E, gpu, batch=3, Nt=256, Ns=384):
+    """spx_attention_forward_lse, spx_attention_backward_q and spx_attention_backward_kv_recompute
+    through the C-ABI: output, the recorded log-sum-exp, the row constants and the three
+    gradients agree with dense fp32 autograd over every block shape the kernels cover - no
+    probabilities are stored anywhere; an empty block row, a block row with one live block
+    and batch sizes that do not fill the eight-way workgroup numbering included."""
+    from sparta_amd import _lib
+    from sparta_amd.tesa import get_bcs_function
+    _, q = randn((batch, Nt, E), 51, dtype)
+    _, k = randn((batch, Ns, E), 52, dtype)
+    _, v = randn((batch, Ns, E), 53, dtype)
+    _, g = randn((batch, Nt, E), 54, dtype)
+    mask_np = ops.block_mask((Nt, Ns), (BH, BW), 0.6, seed=55)
+    mask_np[:BH] = 0
+    if Nt >= 2 * BH:
+        mask_np[BH:2 * BH] = 0
+        mask_np[BH:2 * BH, :BW] = 1
+    mask = torch.from_numpy(mask_np).to(gpu)
+    indexes = get_bcs_function(BH, BW, True, True).build_indexes(mask)
+    q, k, v, g = q.to(gpu), k.to(gpu), v.to(gpu), g.to(gpu)
+    inv_t = 1.0 / float(np.sqrt(E))
+    lib = _lib.load()
+    st = _lib.current_stream(gpu)
+    out = torch.full_like(q, float('nan'))
+    lse = torch.full((batch, Nt), float('nan'), dtype=torch.float32, device=gpu)
+    rc = lib.spx_attention_forward_lse(
+        _lib.dtype_code(dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out), _lib.dev_ptr(lse),
+        _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), None, inv_t, batch, Nt, Ns, E, BH, BW, st)
+    _lib.check(rc, 'spx_attention_forward_lse')
+    grad_q = torch.full_like(q, float('nan'))
+    row_dot = torch.full((batch, Nt), float('nan'), dtype=torch.float32, device=gpu)
+    rc = lib.spx_attention_backward_q(
+        _lib.dtype_code(dtype), _lib.dev_ptr(g), _lib.dev_ptr(out), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),
+        _lib.dev_ptr(lse), _lib.dev_ptr(grad_q), _lib.dev_ptr(row_dot), _lib.dev_ptr(indexes.row_ptr),
+        _lib.dev_ptr(indexes._bcsr_buf), inv_t, batch, Nt, Ns, E, BH, BW, st)
+    _lib.check(rc, 'spx_attention_backward_q')
+
+    qf, kf, vf = (t.float().requires_grad_(True) for t in (q, k, v))
+    masked = (qf @ kf.transpose(1, 2) * inv_t).masked_fill(mask == 0, float('-inf'))
+    p_ref = torch.softmax(masked, -1).nan_to_num(0.0)
+    o_ref = p_ref @ vf
+    o_ref.backward(g.float())
+    tol = dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(out.float(), o_ref.detach(), **tol)
+    # natural-log log-sum-exp of the live scores = row_lse * ln 2; +inf where nothing is live
+    lse_ref = torch.logsumexp(masked.detach(), -1)
+    live = torch.isfinite(lse_ref)
+    torch.testing.assert_close((lse * float(np.log(2.0)))[live], lse_ref[live], rtol=2e-3, atol=2e-3)
+    assert bool(torch.isinf(lse[~live]).all()) and bool((lse[~live] > 0).all())
+    torch.testing.assert_close(row_dot, (g.float() * out.float()).sum(-1) * inv_t, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(grad_q.float(), qf.grad, **tol)
+    assert float(grad_q[:, :BH].abs().max()) == 0.0
+    if BH * E >= 32 * BW and BH <= 2 * BW:
+        grad_k = torch.full_like(k, float('nan'))
+        grad_v = torch.full_like(v, float('nan'))
+        rc = lib.spx_attention_backward_kv_recompute(
+            _lib.dtype_code(dtype), _lib.dev_ptr(g), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(lse),
+            _lib.dev_ptr(row_dot), _lib.dev_ptr(grad_k), _lib.dev_ptr(grad_v), _lib.dev_ptr(indexes.col_ptr),
+            _lib.dev_ptr(indexes._bcsc_buf), _lib.IDX_BCSC_I64, inv_t, batch, Nt, Ns, E, BH, BW, st)
+        _lib.check(rc, 'spx_attention_backward_kv_recompute')
+        torch.testing.assert_close(grad_v.float(), vf.grad, **tol)
+        torch.testing.assert_close(grad_k.float(), kf.grad, **tol)
+    else:
+        rc = lib.spx_attention_backward_kv_recompute(
+            _lib.dtype_code(dtype), _lib.dev_ptr(g), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(lse),
+            _lib.dev_ptr(row_dot), _lib.dev_ptr(q), _lib.dev_ptr(q), _lib.dev_ptr(indexes.col_ptr),
+            _lib.dev_ptr(indexes._bcsc_buf), _lib.IDX_BCSC_I64, inv_t, batch, Nt, Ns, E, BH, BW, st)
+        assert rc != 0 and 'BH <= 2 * BW' in _lib.last_error()
 
 
 @pytest.mark.parametrize('needs', [(True, False, False), (False, True, False), (False, False, True), (True, False, True)])
