@@ -38,18 +38,21 @@ def _hipcc() -> str:
 # the register allocator inserts, or a spill, would read them before the data has arrived.
 # Translation units with such loads are therefore compiled with their device assembly kept,
 # and the assembly is checked.
-_ASM_LOAD_MARK = 'global_load_dwordx4 %0'
+_ASM_LOAD_MARKS = ('global_load_dwordx4 %0', 'buffer_load_dwordx4 %0')
 
 
-def _has_register_prefetch(src: str) -> bool:
+def _has_register_prefetch(src: str, _seen=None) -> bool:
+    """True if the file, or a header of this directory that it includes (at any depth),
+    issues loads into registers through inline assembly."""
+    seen = set() if _seen is None else _seen
+    if src in seen or not os.path.exists(src):
+        return False
+    seen.add(src)
     text = open(src).read()
-    if _ASM_LOAD_MARK in text:
+    if any(mark in text for mark in _ASM_LOAD_MARKS):
         return True
-    for name in re.findall(r'#include "([^"]+)"', text):
-        header = os.path.join(CSRC, name)
-        if os.path.exists(header) and _ASM_LOAD_MARK in open(header).read():
-            return True
-    return False
+    return any(_has_register_prefetch(os.path.join(CSRC, name), seen)
+               for name in re.findall(r'#include "([^"]+)"', text))
 
 
 def _registers(token: str) -> set:
@@ -64,11 +67,12 @@ def check_inflight_registers(asm: str) -> list:
     """Scan device assembly for compiler-generated instructions that touch a VGPR between the
     inline-assembly load that targets it and the inline-assembly wait that covers it.
 
-    The text of each kernel is walked in order.  An inline ``global_load_dwordx4`` makes its
-    destination registers pending; an inline ``s_waitcnt vmcnt(N)`` leaves the N newest loads
-    pending (loads complete in order); a compiler ``s_waitcnt vmcnt(0)``, an unconditional
-    branch or the end of the kernel clears the state (what follows in the text is not what
-    runs next).  Returns a list of (kernel, line number, instruction).
+    The text of each kernel is walked in order.  An inline ``global_load_*`` / ``buffer_load_*``
+    makes its destination registers pending; a memory instruction of the compiler's own takes
+    a place in the same queue; ``s_waitcnt vmcnt(N)``, inline or not, leaves the N newest
+    entries pending (vector memory operations retire in order); an unconditional branch or the
+    end of the kernel clears the state (what follows in the text is not what runs next).
+    Returns a list of (kernel, line number, instruction).
     """
     findings = []
     kernel, pending, in_asm = None, [], False
@@ -87,7 +91,7 @@ def check_inflight_registers(asm: str) -> list:
             in_asm = False
             continue
         if in_asm:
-            if text.startswith('global_load_dwordx4'):
+            if text.startswith(('global_load_', 'buffer_load_')) and 'lds' not in text.split()[0]:
                 pending.append(_registers(text.split()[1].rstrip(',')))
             elif text.startswith('s_waitcnt') and 'vmcnt' in text:
                 n = int(re.search(r'vmcnt\((\d+)\)', text).group(1))
@@ -96,11 +100,18 @@ def check_inflight_registers(asm: str) -> list:
         if text.startswith('s_endpgm'):
             kernel = None
             continue
-        if text.startswith(('s_branch', 's_setpc')) or (text.startswith('s_waitcnt') and 'vmcnt(0)' in text):
+        if text.startswith(('s_branch', 's_setpc')):
             pending = []
+            continue
+        if text.startswith('s_waitcnt') and 'vmcnt(' in text:
+            n = int(re.search(r'vmcnt\((\d+)\)', text).group(1))
+            pending = pending[len(pending) - n:] if n else []
             continue
         if not pending:
             continue
+        if text.startswith(('global_', 'buffer_', 'scratch_', 'flat_')):
+            # a memory instruction of the compiler's own takes a place in the same queue
+            pending.append(set())
         used = set()
         for token in re.findall(r'v\[\d+:\d+\]|v\d+', text):
             used |= _registers(token)

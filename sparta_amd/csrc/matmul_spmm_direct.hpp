@@ -121,6 +121,35 @@ __global__ __launch_bounds__(256) void spmm_direct_kernel(SpmmParams p, int n_mt
     // ---- epilogue: each lane holds 4 memory-contiguous outputs per tile ------------
     const T* biasT = p.bias ? reinterpret_cast<const T*>(p.bias) + b * p.bias_batch : nullptr;
     T* out = reinterpret_cast<T*>(p.out) + b * p.o_batch;
+    // The lane's bias values are fetched together, ahead of the stores: loaded where they are
+    // used, every tile's values wait for their own round trip (the compiler cannot move a
+    // load across the stores of the tile before).  bias_m[i][q] / bias_n[t][q]: q is the
+    // position inside the lane's four contiguous outputs when the bias runs along them.
+    float bias_m[WM][4], bias_n[NT][4];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bias_m[i][q] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bias_n[t][q] = 0.f;
+    if (biasT) {
+        if (p.bias_on_m) {
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int m = m0 + i * 16 + (SWAP ? r16 : g4 * 4 + q);
+                    bias_m[i][q] = Elem<T>::to_float(biasT[m < p.Mc ? m : 0]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) bias_n[t][q] = Elem<T>::to_float(biasT[j * BN + t * 16 + (SWAP ? g4 * 4 + q : r16)]);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < WM; ++i)
 #pragma unroll
@@ -133,8 +162,7 @@ __global__ __launch_bounds__(256) void spmm_direct_kernel(SpmmParams p, int n_mt
             T vals[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                float v = acc[i][t][q];
-                if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (SWAP ? m : m + q) : (SWAP ? n + q : n)]);
+                const float v = acc[i][t][q] + bias_m[i][q] + bias_n[t][q];
                 vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
             }
             T* dst = SWAP ? out + (int64_t)m * p.o_ld + n : out + (int64_t)n * p.o_ld + m;

@@ -243,6 +243,27 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
             // out[m][n], n contiguous.  One 16-row slab per pass: LDS [16][BN + pad].
             constexpr int LDE = BN + E16;
             constexpr int CPR = BN / E16;  // 16-byte chunks per row
+            // The lane's bias values are fetched together, ahead of the LDS traffic below: loaded
+            // where they are used, each one waits for its own round trip (the compiler cannot move
+            // a load across the stores to the staging tile).
+            float bias_n[NT][4], bias_m[4];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) bias_n[t][q] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) bias_m[i] = 0.f;
+            if (biasT) {
+                if (p.bias_on_m) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) bias_m[i] = Elem<T>::to_float(biasT[m0 + i * 16 + r16 < p.Mc ? m0 + i * 16 + r16 : 0]);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) bias_n[t][q] = Elem<T>::to_float(biasT[j * BN + t * 16 + g4 * 4 + q]);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -250,9 +271,7 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
                     T vals[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        float v = acc[i][t][q];
-                        const int n = j * BN + t * 16 + g4 * 4 + q;
-                        if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m0 + i * 16 + r16 < p.Mc ? m0 + i * 16 + r16 : 0) : n]);
+                        const float v = acc[i][t][q] + bias_n[t][q] + bias_m[i];
                         vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
                     }
                     T* dst = eT + r16 * LDE + t * 16 + g4 * 4;
@@ -274,6 +293,27 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
             // out[n][m], m contiguous.  One 16-column slab per pass: LDS [16 n][64 m + pad].
             constexpr int LDE = 64 + E16;
             constexpr int CPR = 64 / E16;
+            float bias_m[4][4], bias_n[NT];   // fetched together, as above
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) bias_m[i][q] = 0.f;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) bias_n[t] = 0.f;
+            if (biasT) {
+                if (p.bias_on_m) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int m = m0 + i * 16 + g4 * 4 + q;
+                            bias_m[i][q] = Elem<T>::to_float(biasT[m < p.Mc ? m : 0]);
+                        }
+                } else {
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) bias_n[t] = Elem<T>::to_float(biasT[j * BN + t * 16 + r16]);
+                }
+            }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
 #pragma unroll
@@ -281,9 +321,7 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
                     T vals[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        float v = acc[i][t][q];
-                        const int m = m0 + i * 16 + g4 * 4 + q;
-                        if (biasT) v += Elem<T>::to_float(biasT[p.bias_on_m ? (m < p.Mc ? m : 0) : j * BN + t * 16 + r16]);
+                        const float v = acc[i][t][q] + bias_m[i][q] + bias_n[t];
                         vals[q] = Elem<T>::from_float(epilogue_act(v, p.relu));
                     }
                     T* dst = eT + r16 * LDE + i * 16 + g4 * 4;
