@@ -468,22 +468,31 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
         // LDS operations of one wavefront complete in order: no barrier needed
         const int c = lane & 7;
         const int n = n0 + wn * 64 + c * 8;
+        // the tokens of the lane's rows, fetched together ahead of the stores (a load between
+        // two stores waits for the store before it as well)
+        int toks[8];
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass) {
+            const int r = wm * 64 + pass * 8 + (lane >> 3);
+            toks[pass] = r < rows ? p.token_perm[row0 + r] : -1;
+        }
 #pragma unroll
         for (int pass = 0; pass < 8; ++pass) {
             const int row = pass * 8 + (lane >> 3);
-            const int r = wm * 64 + row;
             const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * 128 + ((c ^ (row & 7)) << 4));
-            if (r < rows && n < p.N) {
-                const int tok = p.token_perm[row0 + r];
-                *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
-            }
+            if (toks[pass] >= 0 && n < p.N) *reinterpret_cast<u32x4*>(out + (int64_t)toks[pass] * p.N + n) = v;
         }
     } else {
+    int toks[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int r = wm * 64 + i * 16 + r16;
-        if (r >= rows) continue;
-        const int tok = p.token_perm[row0 + r];
+        toks[i] = r < rows ? p.token_perm[row0 + r] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (toks[i] < 0) continue;
+        const int tok = toks[i];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int n = n0 + wn * 64 + t * 16 + g4 * 4;
@@ -736,22 +745,32 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                 }
         const int c = lane & 7;
         const int n = n0 + wcol + c * 8;
+        // The token of every row this lane stores, fetched together ahead of the stores: a
+        // load placed between the stores waits for the store before it as well (one counter,
+        // in order), i.e. for a write to memory and a read from it per pass.
+        int toks[WR / 8];
+#pragma unroll
+        for (int pass = 0; pass < WR / 8; ++pass) {
+            const int r = wrow + pass * 8 + (lane >> 3);
+            toks[pass] = r < rows ? p.token_perm[row0 + r] : -1;
+        }
 #pragma unroll
         for (int pass = 0; pass < WR / 8; ++pass) {
             const int row = pass * 8 + (lane >> 3);
-            const int r = wrow + row;
             const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * 128 + ((c ^ (row & 7)) << 4));
-            if (r < rows && n < p.N) {
-                const int tok = p.token_perm[row0 + r];
-                *reinterpret_cast<u32x4*>(out + (int64_t)tok * p.N + n) = v;
-            }
+            if (toks[pass] >= 0 && n < p.N) *reinterpret_cast<u32x4*>(out + (int64_t)toks[pass] * p.N + n) = v;
         }
     } else {
+    int toks[MT];   // fetched together ahead of the stores, as above
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int r = wrow + i * 16 + r16;
-        if (r >= rows) continue;
-        const int tok = p.token_perm[row0 + r];
+        toks[i] = r < rows ? p.token_perm[row0 + r] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        if (toks[i] < 0) continue;
+        const int tok = toks[i];
 #pragma unroll
         for (int t = 0; t < NTT; ++t) {
             const int n = n0 + wcol + t * 16 + g4 * 4;
