@@ -248,8 +248,8 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
                 m2 = masks2[1].clone()
 
                 def step():
-                    op1.update_mask(weight_mask=m1)
-                    op2.update_mask(weight_mask=m2)
+                    # the two rebuilds are independent: one library call, one pair of launches
+                    sparta.nn.update_masks([(op1, {'weight_mask': m1}), (op2, {'weight_mask': m2})])
                     return op2(op1(x))
 
                 _close(torch, step(), dense_ffn(m1, m2), f'c4 dynamic={dynamic}')

@@ -122,6 +122,30 @@ int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
                             int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
                             void* workspace, size_t workspace_bytes, spx_stream_t stream);
 
+/* Several independent index builds in one call: every job has the arguments of
+ * spx_bcs_index_scheduled.  Jobs that take the bit-word path (16-byte aligned masks with
+ * W % 16 == 0 and at most 2048 words of 64 blocks per side) share one pair of launches, up to
+ * four at a time - a model that rebuilds the masks of several layers per step otherwise pays
+ * one pair of small dependent launches per layer; the other jobs are built one after the
+ * other.  Results are those of separate calls.  No counterpart in the reference, which builds
+ * one index per call (block_compressed.py:242-265). */
+typedef struct spx_bcs_index_job {
+    const uint8_t* mask;
+    int H, W, BH, BW;
+    int32_t* row_ptr;
+    int32_t* bcsr_idx;
+    int32_t* col_ptr;
+    void* bcsc_idx;
+    int bcsc_i64;
+    int32_t* nnz_dev;
+    int cap;
+    int32_t* row_order;
+    int32_t* col_order;
+    void* workspace;
+    size_t workspace_bytes;
+} spx_bcs_index_job;
+int spx_bcs_index_batch(const spx_bcs_index_job* jobs, int n_jobs, spx_stream_t stream);
+
 /* spx_bcs_index for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): no workspace argument.
  * No counterpart in the reference.  The scratch of the two kernels lives in a device

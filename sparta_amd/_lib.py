@@ -35,6 +35,17 @@ class TileCfg(ctypes.Structure):
 _c = ctypes
 _P, _I, _L, _F, _Z = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float, _c.c_size_t
 
+
+class BcsIndexJob(ctypes.Structure):
+    """spx_bcs_index_job: the arguments of spx_bcs_index_scheduled for one mask."""
+    _fields_ = [
+        ('mask', _P), ('H', _I), ('W', _I), ('BH', _I), ('BW', _I),
+        ('row_ptr', _P), ('bcsr_idx', _P), ('col_ptr', _P), ('bcsc_idx', _P), ('bcsc_i64', _I),
+        ('nnz_dev', _P), ('cap', _I), ('row_order', _P), ('col_order', _P),
+        ('workspace', _P), ('workspace_bytes', _Z),
+    ]
+
+
 _SIGNATURES = {
     'spx_last_error': (_c.c_char_p, []),
     'spx_version': (_I, []),
@@ -42,6 +53,7 @@ _SIGNATURES = {
     'spx_bcs_index_workspace_bytes': (_Z, [_I, _I, _I, _I]),
     'spx_bcs_index': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P, _Z, _P]),
     'spx_bcs_index_scheduled': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _Z, _P]),
+    'spx_bcs_index_batch': (_I, [_c.POINTER(BcsIndexJob), _I, _P]),
     'spx_bcs_index_static_max_bytes': (_Z, []),
     'spx_bcs_index_static': (_I, [_P, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _I, _P]),
     'spx_bcs_gather': (_I, [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _L, _P]),

@@ -262,12 +262,12 @@ struct BitsParams {
     int rows_per_part;          // mask rows of a block-row that one workgroup covers (BH / Q)
 };
 
-__global__ __launch_bounds__(256) void live_bits_kernel(BitsParams p) {
+// word wi of block-row r, row group `part`
+__device__ __forceinline__ void live_bits_body(const BitsParams& p, int wi, int r, int part) {
     __shared__ uint32_t flags[64];
     const int tid = threadIdx.x;
     if (tid < 64) flags[tid] = 0;
     __syncthreads();
-    const int wi = blockIdx.x, r = blockIdx.y, part = blockIdx.z;
     const int64_t col0 = (int64_t)wi * 64 * p.BW;            // first mask column of the word
     const int64_t left = p.W - col0;
     const int nch = (int)((left < 64 * p.BW ? left : 64 * p.BW) >> 4);  // 16-byte chunks per mask row
@@ -319,6 +319,10 @@ __global__ __launch_bounds__(256) void live_bits_kernel(BitsParams p) {
         const unsigned long long word = __ballot(flags[tid] != 0);
         if (tid == 0) p.pbits[(int64_t)part * p.NW + (int64_t)r * p.WPR + wi] = word;
     }
+}
+
+__global__ __launch_bounds__(256) void live_bits_kernel(BitsParams p) {
+    live_bits_body(p, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 __device__ __forceinline__ int block_exclusive_scan_1024(int v, int* lds, int* total) {
@@ -387,7 +391,8 @@ __device__ __forceinline__ unsigned long long transpose_bits_64x64(unsigned long
     return x;
 }
 
-__global__ __launch_bounds__(1024) void emit_words_kernel(EmitParams p, int nslice, int sides, int nparts) {
+// workgroup bx of the nslice * (1 or 2) of one index
+__device__ __forceinline__ void emit_words_body(const EmitParams& p, int nslice, int sides, int nparts, int bx) {
     __shared__ unsigned long long s_bits[EMIT_FAST_WORDS];   // row words
     __shared__ int s_base[EMIT_FAST_WORDS];                  // exclusive prefix of their popcounts
     __shared__ unsigned long long s_cbits[EMIT_FAST_WORDS];  // column words
@@ -398,8 +403,8 @@ __global__ __launch_bounds__(1024) void emit_words_kernel(EmitParams p, int nsli
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    const int side = sides == 3 ? (int)blockIdx.x / nslice : (sides == 2 ? 1 : 0);  // 0 BCSR, 1 BCSC
-    const int slice = (int)blockIdx.x % nslice;
+    const int side = sides == 3 ? bx / nslice : (sides == 2 ? 1 : 0);  // 0 BCSR, 1 BCSC
+    const int slice = bx % nslice;
 
     // ---- row words: word g = r * WPR + wi covers columns wi*64 .. wi*64+63 of row r ----
     const int NW = p.R * p.WPR;
@@ -495,6 +500,43 @@ __global__ __launch_bounds__(1024) void emit_words_kernel(EmitParams p, int nsli
     if (slice == nslice - 1 && p.col_order) schedule_from_lds(s_cbase, p.WPC, p.Cn, nnz2, p.col_order, s_bins);
 }
 
+__global__ __launch_bounds__(1024) void emit_words_kernel(EmitParams p, int nslice, int sides, int nparts) {
+    emit_words_body(p, nslice, sides, nparts, (int)blockIdx.x);
+}
+
+// ---- several independent masks in one pair of launches ---------------------------------
+// A model that rebuilds the indexes of several layers per step issues as many pairs of small
+// dependent launches, each a few workgroups wide and each waiting for the one before it.
+// Here the workgroups of up to INDEX_BATCH_MAX builds share the two launches: the x range of
+// the grid is cut into one piece per build (x_end), the other grid dimensions are those of the
+// largest build and the workgroups outside a build's own range leave at once.
+constexpr int INDEX_BATCH_MAX = 4;
+struct BitsBatch {
+    BitsParams job[INDEX_BATCH_MAX];
+    int x_end[INDEX_BATCH_MAX], R[INDEX_BATCH_MAX], nparts[INDEX_BATCH_MAX];
+    int n;
+};
+struct EmitBatch {
+    EmitParams job[INDEX_BATCH_MAX];
+    int x_end[INDEX_BATCH_MAX], nslice[INDEX_BATCH_MAX], sides[INDEX_BATCH_MAX], nparts[INDEX_BATCH_MAX];
+    int n;
+};
+
+__global__ __launch_bounds__(256) void live_bits_batch_kernel(BitsBatch b) {
+    const int bx = blockIdx.x;
+    int j = 0;
+    while (j + 1 < b.n && bx >= b.x_end[j]) ++j;
+    if ((int)blockIdx.y >= b.R[j] || (int)blockIdx.z >= b.nparts[j]) return;
+    live_bits_body(b.job[j], bx - (j ? b.x_end[j - 1] : 0), blockIdx.y, blockIdx.z);
+}
+
+__global__ __launch_bounds__(1024) void emit_words_batch_kernel(EmitBatch b) {
+    const int bx = blockIdx.x;
+    int j = 0;
+    while (j + 1 < b.n && bx >= b.x_end[j]) ++j;
+    emit_words_body(b.job[j], b.nslice[j], b.sides[j], b.nparts[j], bx - (j ? b.x_end[j - 1] : 0));
+}
+
 __global__ __launch_bounds__(1024) void schedule_kernel(const int32_t* ptr, int n, int32_t* order) {
     __shared__ int bins[256];
     schedule_segments(ptr, n, order, bins);
@@ -541,11 +583,21 @@ extern "C" size_t spx_bcs_index_workspace_bytes(int H, int W, int BH, int BW) {
 }
 
 namespace spx {
+// what bcs_index_impl would have launched on the bit-word path, handed back instead
+struct FastIndexJob {
+    BitsParams bits;
+    EmitParams emit;
+    int WPR, R, nparts, nslice, sides;
+    int ready;   // 0: this build takes the general path and was not prepared
+};
+// fast != NULL: validate and, where the bit-word path applies, fill *fast without launching
+// (fast->ready = 1); where it does not, leave fast->ready = 0 and launch nothing either.
 static int bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW,
                           int32_t* row_ptr, int32_t* bcsr_idx,
                           int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
                           int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
-                          void* workspace, size_t workspace_bytes, spx_stream_t stream);
+                          void* workspace, size_t workspace_bytes, spx_stream_t stream,
+                          FastIndexJob* fast = nullptr);
 }
 
 extern "C" int spx_bcs_index(const uint8_t* mask, int H, int W, int BH, int BW,
@@ -573,8 +625,10 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
                                int32_t* row_ptr, int32_t* bcsr_idx,
                                int32_t* col_ptr, void* bcsc_idx, int bcsc_i64,
                                int32_t* nnz_dev, int cap, int32_t* row_order, int32_t* col_order,
-                               void* workspace, size_t workspace_bytes, spx_stream_t stream) {
+                               void* workspace, size_t workspace_bytes, spx_stream_t stream,
+                               FastIndexJob* fast) {
     using namespace spx;
+    if (fast) fast->ready = 0;
     int rc = check_index_shape(H, W, BH, BW);
     if (rc) return rc;
     SPX_REQUIRE(mask && nnz_dev && workspace, SPX_E_NULL, "mask, nnz_dev and workspace are required");
@@ -623,16 +677,24 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
         bp.log_bw = ilog2(BW);
         bp.rows_per_part = BH / nparts;
         ep.wbits = bp.pbits;
-        hipLaunchKernelGGL(live_bits_kernel, dim3(ws.WPR, ws.R, nparts), dim3(256), 0, st, bp);
-        SPX_LAUNCH_CHECK("live_bits_kernel");
         const int sides = (row_ptr ? 1 : 0) | (col_ptr ? 2 : 0);
         // enough slices that a slice writes at most ~2048 index entries
         int nslice = (ws.R * ws.Cn + 2047) / 2048;
         nslice = nslice < 1 ? 1 : (nslice > 8 ? 8 : nslice);
+        if (fast) {   // the caller launches (several builds in one pair of launches)
+            fast->bits = bp; fast->emit = ep;
+            fast->WPR = ws.WPR; fast->R = ws.R; fast->nparts = nparts; fast->nslice = nslice; fast->sides = sides;
+            fast->ready = 1;
+            return 0;
+        }
+        hipLaunchKernelGGL(live_bits_kernel, dim3(ws.WPR, ws.R, nparts), dim3(256), 0, st, bp);
+        SPX_LAUNCH_CHECK("live_bits_kernel");
         hipLaunchKernelGGL(emit_words_kernel, dim3(nslice * (sides == 3 ? 2 : 1)), dim3(1024), 0, st, ep, nslice, sides, nparts);
         SPX_LAUNCH_CHECK("emit_words_kernel");
         return 0;
     }
+
+    if (fast) return 0;   // general path: the caller builds this one on its own
 
     // Segment width: at most 256 threads * vec bytes, at least one block wide;
     // narrowed while that buys more workgroups (the launch wants >> 256 of them).
@@ -659,6 +721,59 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
     SPX_LAUNCH_CHECK("liveness_kernel");
     hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
     SPX_LAUNCH_CHECK("emit_kernel");
+    return 0;
+}
+
+extern "C" int spx_bcs_index_batch(const spx_bcs_index_job* jobs, int n_jobs, spx_stream_t stream) {
+    using namespace spx;
+    SPX_REQUIRE(n_jobs >= 0, SPX_E_SHAPE, "negative job count");
+    SPX_REQUIRE(jobs || n_jobs == 0, SPX_E_NULL, "jobs is required");
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    for (int first = 0; first < n_jobs;) {
+        // validate and prepare up to INDEX_BATCH_MAX builds; those on the bit-word path share
+        // one pair of launches, the others are built one by one
+        const int last = first + INDEX_BATCH_MAX < n_jobs ? first + INDEX_BATCH_MAX : n_jobs;
+        FastIndexJob prep[INDEX_BATCH_MAX];
+        for (int i = first; i < last; ++i) {
+            const spx_bcs_index_job& j = jobs[i];
+            SPX_REQUIRE(!j.row_order || j.row_ptr, SPX_E_NULL, "row_order needs the BCSR index");
+            SPX_REQUIRE(!j.col_order || j.col_ptr, SPX_E_NULL, "col_order needs the BCSC index");
+            const int rc = bcs_index_impl(j.mask, j.H, j.W, j.BH, j.BW, j.row_ptr, j.bcsr_idx, j.col_ptr, j.bcsc_idx,
+                                          j.bcsc_i64, j.nnz_dev, j.cap, j.row_order, j.col_order, j.workspace,
+                                          j.workspace_bytes, stream, &prep[i - first]);
+            if (rc) return rc;
+        }
+        BitsBatch bb;
+        EmitBatch eb;
+        int n = 0, bx = 0, ex = 0, max_r = 1, max_parts = 1;
+        for (int i = first; i < last; ++i) {
+            const FastIndexJob& f = prep[i - first];
+            if (!f.ready) continue;
+            bb.job[n] = f.bits; bb.R[n] = f.R; bb.nparts[n] = f.nparts;
+            bx += f.WPR; bb.x_end[n] = bx;
+            eb.job[n] = f.emit; eb.nslice[n] = f.nslice; eb.sides[n] = f.sides; eb.nparts[n] = f.nparts;
+            ex += f.nslice * (f.sides == 3 ? 2 : 1); eb.x_end[n] = ex;
+            max_r = f.R > max_r ? f.R : max_r;
+            max_parts = f.nparts > max_parts ? f.nparts : max_parts;
+            ++n;
+        }
+        if (n > 0) {
+            bb.n = eb.n = n;
+            hipLaunchKernelGGL(live_bits_batch_kernel, dim3(bx, max_r, max_parts), dim3(256), 0, st, bb);
+            SPX_LAUNCH_CHECK("live_bits_batch_kernel");
+            hipLaunchKernelGGL(emit_words_batch_kernel, dim3(ex), dim3(1024), 0, st, eb);
+            SPX_LAUNCH_CHECK("emit_words_batch_kernel");
+        }
+        for (int i = first; i < last; ++i) {
+            if (prep[i - first].ready) continue;
+            const spx_bcs_index_job& j = jobs[i];
+            const int rc = bcs_index_impl(j.mask, j.H, j.W, j.BH, j.BW, j.row_ptr, j.bcsr_idx, j.col_ptr, j.bcsc_idx,
+                                          j.bcsc_i64, j.nnz_dev, j.cap, j.row_order, j.col_order, j.workspace,
+                                          j.workspace_bytes, stream);
+            if (rc) return rc;
+        }
+        first = last;
+    }
     return 0;
 }
 

@@ -70,10 +70,18 @@ class PortConfig:
             self.mask = mask
             self._update_indexes()
 
+    def index_builder(self):
+        """The function context that builds this port's indexes (None before block sizes are set)."""
+        if not self.is_sparse or not self._block_H or not self._block_W or self._block_H <= 0 or self._block_W <= 0:
+            return None
+        return get_bcs_function(self._block_H, self._block_W, self.BCSR, self.BCSC)
+
     def _update_indexes(self):
-        if self.mask is None or self._block_H <= 0 or self._block_W <= 0:
+        if self.mask is None:
             return
-        builder = get_bcs_function(self._block_H, self._block_W, self.BCSR, self.BCSC)
+        builder = self.index_builder()
+        if builder is None:
+            return
         self.indexes = builder.build_indexes(self.mask)
 
     def connect(self, kernel: 'KernelBase', port_name: str):

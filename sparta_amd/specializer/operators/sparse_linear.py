@@ -74,6 +74,17 @@ class SparseLinear(OperatorBase):
     def update_mask(self, input_mask: Optional[torch.Tensor] = None,
                     weight_mask: Optional[torch.Tensor] = None,
                     output_mask: Optional[torch.Tensor] = None):
+        self._set_mask(self._mask_arguments(input_mask, weight_mask, output_mask))
+        self._after_mask_update()
+
+    def _after_mask_update(self):
+        if self.ready:
+            self._update_parameters()
+
+    def _mask_arguments(self, input_mask: Optional[torch.Tensor] = None,
+                        weight_mask: Optional[torch.Tensor] = None,
+                        output_mask: Optional[torch.Tensor] = None) -> Dict[str, torch.Tensor]:
+        """Check the arguments of `update_mask`; returns {sparse port: mask}."""
         given = {k: v for k, v in (('input', input_mask), ('weight', weight_mask), ('output', output_mask))
                  if v is not None}
         if len(given) > 1:
@@ -86,9 +97,7 @@ class SparseLinear(OperatorBase):
         ok = all(w is None or w == got for w, got in zip(want, mask.shape))
         shown = tuple('?' if w is None else w for w in want)
         assert ok and mask.dim() == 2, f'expected {kind} mask shape {shown}, got {tuple(mask.shape)}'
-        self._set_mask({self._PORT_OF[kind]: mask})
-        if self.ready:
-            self._update_parameters()
+        return {self._PORT_OF[kind]: mask}
 
     def _read_sample_inputs(self, A: torch.Tensor):
         M, K = self._shape['M'], self._shape['K']

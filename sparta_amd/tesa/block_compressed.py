@@ -14,7 +14,7 @@ sparta/tesa/block_compressed.py:23-413 with two deliberate differences:
 """
 from __future__ import annotations
 
-from typing import Dict, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import numpy as np
 import torch
@@ -214,9 +214,9 @@ class BCSFunctionContext(TeSAFunctionContext):
             self._workspaces[key] = nbytes
         return torch.empty((nbytes,), dtype=torch.uint8, device=device)
 
-    def build_indexes(self, mask: torch.Tensor, capacity: Optional[int] = None) -> BCSIndexes:
-        """mask: uint8 (or any 1-byte dtype) [H, W] on the GPU.  `capacity` bounds the
-        number of index entries kept (default: every block)."""
+    def _prepare(self, mask: torch.Tensor, capacity: Optional[int] = None) -> dict:
+        """Output buffers and workspace of one index build (everything
+        spx_bcs_index_scheduled takes), allocated but not yet filled."""
         assert mask.dim() == 2, 'only 2D mask is supported'
         if mask.dtype != torch.uint8:
             mask = (mask != 0).to(torch.uint8)
@@ -228,34 +228,47 @@ class BCSFunctionContext(TeSAFunctionContext):
         cap = R * Cn if capacity is None else int(capacity)
         dev = mask.device
         i32 = dict(dtype=torch.int32, device=dev)
-        nnz_dev = torch.empty((1,), **i32)
-        row_ptr = bcsr = col_ptr = bcsc = None
+        job = dict(mask=mask, H=H, W=W, cap=cap, nnz_dev=torch.empty((1,), **i32),
+                   row_ptr=None, bcsr=None, col_ptr=None, bcsc=None, row_order=None, col_order=None)
         if self._BCSR:
-            row_ptr = torch.empty((R + 1,), **i32)
-            bcsr = torch.empty((cap,), **i32)
+            job['row_ptr'] = torch.empty((R + 1,), **i32)
+            job['bcsr'] = torch.empty((cap,), **i32)
+            job['row_order'] = torch.empty((R,), **i32)   # the launch orders of the matmul kernels
         both = self._BCSR and self._BCSC
         if self._BCSC:
-            col_ptr = torch.empty((Cn + 1,), **i32)
-            bcsc = torch.empty((cap,), dtype=torch.int64 if both else torch.int32, device=dev)
-        # the launch orders of the matmul kernels come out of the same launch
-        row_order = torch.empty((R,), **i32) if self._BCSR else None
-        col_order = torch.empty((Cn,), **i32) if self._BCSC else None
-        ws = self._workspace(H, W, dev)
+            job['col_ptr'] = torch.empty((Cn + 1,), **i32)
+            job['bcsc'] = torch.empty((cap,), dtype=torch.int64 if both else torch.int32, device=dev)
+            job['col_order'] = torch.empty((Cn,), **i32)  # come out of the same launch
+        job['ws'] = self._workspace(H, W, dev)
+        return job
+
+    def _wrap(self, job: dict) -> BCSIndexes:
+        BH, BW = self._block_H, self._block_W
+        if self._BCSR and self._BCSC:
+            indexes = BCSRCIndexes(self, job['mask'], job['row_ptr'], job['col_ptr'], job['bcsr'], job['bcsc'],
+                                   job['nnz_dev'], BH, BW)
+        elif self._BCSR:
+            indexes = BCSRIndexes(self, job['mask'], job['row_ptr'], job['bcsr'], job['nnz_dev'], BH, BW)
+        else:
+            indexes = BCSCIndexes(self, job['mask'], job['col_ptr'], job['bcsc'], job['nnz_dev'], BH, BW)
+        indexes.__dict__['_launch_order'] = {k: v for k, v in (('row', job['row_order']), ('col', job['col_order']))
+                                             if v is not None}
+        return indexes
+
+    def build_indexes(self, mask: torch.Tensor, capacity: Optional[int] = None) -> BCSIndexes:
+        """mask: uint8 (or any 1-byte dtype) [H, W] on the GPU.  `capacity` bounds the
+        number of index entries kept (default: every block)."""
+        job = self._prepare(mask, capacity)
+        dev = job['mask'].device
         with torch.cuda.device(dev):
             rc = _lib.load().spx_bcs_index_scheduled(
-                _lib.dev_ptr(mask), H, W, BH, BW,
-                _lib.dev_ptr(row_ptr), _lib.dev_ptr(bcsr), _lib.dev_ptr(col_ptr), _lib.dev_ptr(bcsc),
-                1 if both else 0, _lib.dev_ptr(nnz_dev), cap, _lib.dev_ptr(row_order), _lib.dev_ptr(col_order),
-                _lib.dev_ptr(ws), ws.numel(), _lib.current_stream(dev))
+                _lib.dev_ptr(job['mask']), job['H'], job['W'], self._block_H, self._block_W,
+                _lib.dev_ptr(job['row_ptr']), _lib.dev_ptr(job['bcsr']), _lib.dev_ptr(job['col_ptr']),
+                _lib.dev_ptr(job['bcsc']), 1 if (self._BCSR and self._BCSC) else 0, _lib.dev_ptr(job['nnz_dev']),
+                job['cap'], _lib.dev_ptr(job['row_order']), _lib.dev_ptr(job['col_order']),
+                _lib.dev_ptr(job['ws']), job['ws'].numel(), _lib.current_stream(dev))
         _lib.check(rc, 'spx_bcs_index_scheduled')
-        if both:
-            indexes = BCSRCIndexes(self, mask, row_ptr, col_ptr, bcsr, bcsc, nnz_dev, BH, BW)
-        elif self._BCSR:
-            indexes = BCSRIndexes(self, mask, row_ptr, bcsr, nnz_dev, BH, BW)
-        else:
-            indexes = BCSCIndexes(self, mask, col_ptr, bcsc, nnz_dev, BH, BW)
-        indexes.__dict__['_launch_order'] = {k: v for k, v in (('row', row_order), ('col', col_order)) if v is not None}
-        return indexes
+        return self._wrap(job)
 
     # ---- values ------------------------------------------------------------------
     def convert(self, dense: torch.Tensor, index: torch.Tensor, block_nnz: int, H: int, W: int,
@@ -308,6 +321,34 @@ class BCSFunctionContext(TeSAFunctionContext):
 
 
 _bcs_function_cache: Dict[Tuple[int, int, bool, bool], BCSFunctionContext] = {}
+
+
+def build_indexes_batch(requests) -> List[BCSIndexes]:
+    """Indexes of several masks in one library call (spx_bcs_index_batch: the builds that
+    qualify share one pair of launches).  `requests` is a sequence of
+    (BCSFunctionContext, mask) or (BCSFunctionContext, mask, capacity); all masks on one GPU.
+    The results equal those of `context.build_indexes(mask, capacity)` one by one."""
+    requests = [tuple(r) + (None,) * (3 - len(r)) for r in requests]
+    if not requests:
+        return []
+    jobs = [ctx._prepare(mask, cap) for ctx, mask, cap in requests]
+    dev = jobs[0]['mask'].device
+    assert all(j['mask'].device == dev for j in jobs), 'the masks of one batch must be on one device'
+    array = (_lib.BcsIndexJob * len(jobs))()
+    addr = lambda t: None if t is None else t.data_ptr()
+    for slot, (ctx, _, _), job in zip(array, requests, jobs):
+        slot.mask = addr(job['mask'])
+        slot.H, slot.W, slot.BH, slot.BW = job['H'], job['W'], ctx._block_H, ctx._block_W
+        slot.row_ptr, slot.bcsr_idx = addr(job['row_ptr']), addr(job['bcsr'])
+        slot.col_ptr, slot.bcsc_idx = addr(job['col_ptr']), addr(job['bcsc'])
+        slot.bcsc_i64 = 1 if (ctx._BCSR and ctx._BCSC) else 0
+        slot.nnz_dev, slot.cap = addr(job['nnz_dev']), job['cap']
+        slot.row_order, slot.col_order = addr(job['row_order']), addr(job['col_order'])
+        slot.workspace, slot.workspace_bytes = addr(job['ws']), job['ws'].numel()
+    with torch.cuda.device(dev):
+        rc = _lib.load().spx_bcs_index_batch(array, len(jobs), _lib.current_stream(dev))
+    _lib.check(rc, 'spx_bcs_index_batch')
+    return [ctx._wrap(job) for (ctx, _, _), job in zip(requests, jobs)]
 
 
 def get_bcs_function(block_H: int, block_W: int, BCSR: bool, BCSC: bool) -> BCSFunctionContext:

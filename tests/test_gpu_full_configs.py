@@ -87,8 +87,9 @@ def topk_block_mask(shape, seed, block=(32, 64), keep_frac=0.1):
     return np.kron(grid, np.ones(block, dtype=np.uint8)), int(grid.sum())
 
 
-@pytest.mark.parametrize('fused', [True, False])
-def test_c4_dynamic_ffn_three_mask_updates(fused, gpu):
+@pytest.mark.parametrize('fused,batched', [(True, True), (True, False), (False, False)])
+def test_c4_dynamic_ffn_three_mask_updates(fused, batched, gpu):
+    # batched: both index rebuilds through sparta.nn.update_masks (one pair of launches), as bench.py issues them
     # fused: the activation between the layers runs in the first layer's epilogue (what bench.py times)
     act = (lambda h: h) if fused else torch.relu
     T, D, F = 8192, 768, 3072
@@ -126,8 +127,12 @@ def test_c4_dynamic_ffn_three_mask_updates(fused, gpu):
     for step in range(1, 4):  # three mask updates after the build
         m1, m2 = masks1[step][0], masks2[step][0]
         with torch.no_grad():
-            op1.update_mask(weight_mask=torch.from_numpy(m1).to(gpu))
-            op2.update_mask(weight_mask=torch.from_numpy(m2).to(gpu))
+            if batched:
+                sparta.nn.update_masks([(op1, {'weight_mask': torch.from_numpy(m1).to(gpu)}),
+                                        (op2, {'weight_mask': torch.from_numpy(m2).to(gpu)})])
+            else:
+                op1.update_mask(weight_mask=torch.from_numpy(m1).to(gpu))
+                op2.update_mask(weight_mask=torch.from_numpy(m2).to(gpu))
             y = op2(act(op1(xg)))
         for op, m in ((op1, m1), (op2, m2)):
             idx = op.get_sparse_indexes('B')
@@ -142,8 +147,11 @@ def test_c4_dynamic_ffn_three_mask_updates(fused, gpu):
     m2g = torch.from_numpy(masks2[0][0]).to(gpu).clone()
 
     def graph_step():
-        op1.update_mask(weight_mask=m1g)
-        op2.update_mask(weight_mask=m2g)
+        if batched:
+            sparta.nn.update_masks([(op1, {'weight_mask': m1g}), (op2, {'weight_mask': m2g})])
+        else:
+            op1.update_mask(weight_mask=m1g)
+            op2.update_mask(weight_mask=m2g)
         return op2(act(op1(xg)))
 
     with torch.no_grad():

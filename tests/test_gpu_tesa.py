@@ -80,6 +80,44 @@ def _check_indexes(mask_np, BH, BW, gpu):
     return r, c, rc
 
 
+def test_index_batch_equals_single_builds(gpu):
+    """spx_bcs_index_batch: several masks in one call - different shapes, block sizes and
+    formats, more jobs than share one pair of launches, a mask whose width rules out the
+    bit-word path (built on its own inside the call), an empty mask and a full one - give
+    exactly the indexes of one build_indexes call each, against the oracle as well."""
+    from sparta_amd.tesa import build_indexes_batch
+    cases = [((3072, 768), (32, 64), True, False, 0.9), ((768, 3072), (32, 64), True, False, 0.9),
+             ((1024, 768), (8, 8), True, True, 0.8), ((256, 4096), (64, 16), False, True, 0.5),
+             ((512, 520), (8, 8), True, True, 0.7),          # 520 % 16 != 0: general path
+             ((4096, 4096), (32, 32), True, True, 0.95), ((64, 64), (32, 32), True, False, 0.0)]
+    requests, masks = [], []
+    for i, (shape, blk, r, c, sparsity) in enumerate(cases):
+        mask_np = ops.block_mask(shape, blk, sparsity, seed=70 + i)
+        if i == 2:
+            mask_np[:] = 0
+        masks.append(mask_np)
+        requests.append((get_bcs_function(blk[0], blk[1], r, c), torch.from_numpy(mask_np).to(gpu)))
+    batch = build_indexes_batch(requests)
+    assert len(batch) == len(cases)
+    for (ctx, mask), got, mask_np, (shape, blk, r, c, _) in zip(requests, batch, masks, cases):
+        want = ctx.build_indexes(mask)
+        assert type(got) is type(want) and got.block_nnz == want.block_nnz
+        row_ptr, bcsr, col_ptr, bcsc64, nnz = bcs.build_bcsrc(mask_np, blk[0], blk[1])
+        assert got.block_nnz == nnz
+        if r:
+            assert np.array_equal(got.row_ptr.cpu().numpy(), row_ptr)
+            assert np.array_equal(got.BCSR_idx.cpu().numpy()[:nnz], bcsr)
+            assert torch.equal(got.BCSR_idx[:nnz], want.BCSR_idx[:nnz])
+            _check_launch_order(got.launch_order('row'), row_ptr)
+        if c:
+            assert np.array_equal(got.col_ptr.cpu().numpy(), col_ptr)
+            assert torch.equal(got.BCSC_idx[:nnz], want.BCSC_idx[:nnz])
+            _check_launch_order(got.launch_order('col'), col_ptr)
+        if r and c:
+            assert np.array_equal(got.BCSC_idx.cpu().numpy()[:nnz], bcsc64)
+    assert build_indexes_batch([]) == []
+
+
 @pytest.mark.parametrize('BH', EDGES)
 @pytest.mark.parametrize('BW', EDGES)
 def test_index_reference_shapes(BH, BW, gpu):
