@@ -63,9 +63,10 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
     _emit.verbose = verbose
 
     def timed(fn):
-        # shortest of three replays: the first one after the correctness checks runs at ramping clocks
+        # shortest replay out of at least three and at least 50 ms of them: the first ones after
+        # the correctness checks run at ramping clocks
         try:
-            return time_graph(torch, fn, steps, warmup, 3) / steps
+            return time_graph(torch, fn, steps, warmup, 3, 0.05) / steps
         except Exception:
             return min(time_eager(torch, fn, steps, warmup) for _ in range(3)) / steps
 
