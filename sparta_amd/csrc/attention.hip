@@ -2073,13 +2073,7 @@ static int launch_attention_v3_inst(const AttnParams& p, int batch, hipStream_t 
 
 // The wide-MFMA kernel covers query blocks of 32 / 64 / 128 (one wavefront per 32 queries),
 // key blocks of 32 / 64 / 128 and head dimensions 64 / 128, as long as a thread stages one
-// to eight 16-byte vectors of each tile.
-static bool attention_v3_supported(int BH, int BW, int E) {
-    if (!((BH == 32 || BH == 64 || BH == 128) && (BW == 32 || BW == 64 || BW == 128) && (E == 64 || E == 128))) return false;
-    const int nt = BH * 2, vecs = BW * E / 8;
-    return vecs % nt == 0 && vecs / nt >= 1 && vecs / nt <= 8;
-}
-
+// to eight 16-byte vectors of each tile: the combinations listed here.
 template <typename T>
 static int launch_attention_v3(const AttnParams& p, int batch, int BW, int E, hipStream_t st) {
 #define SPX_ATTN3_CASE(bh, bw, e) \
