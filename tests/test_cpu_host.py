@@ -93,6 +93,61 @@ def test_host_validation_without_gpu():
         _lib.check(700, 'x')
 
 
+def test_host_validation_of_recompute_batch_and_moe_entry_points():
+    """Argument checks that come before any launch or device query: they run without a GPU."""
+    lib = _lib.load()
+    one = ctypes.c_void_p(256)  # never dereferenced
+    f16, i64 = _lib.F16, _lib.IDX_BCSC_I64
+    lse = lambda dtype=f16, row_lse=one, Nt=256, E=64: lib.spx_attention_forward_lse(
+        dtype, one, one, one, one, row_lse, one, one, None, 0.125, 1, Nt, 256, E, 64, 64, None)
+    assert lse(dtype=0) == _lib.E_DTYPE
+    assert lse(row_lse=None) == _lib.E_NULL and 'row_lse' in _lib.last_error()
+    assert lse(Nt=250) == _lib.E_SHAPE
+    assert lse(E=48) == _lib.E_CONFIG
+    bq = lambda dtype=f16, row_lse=one, BH=64: lib.spx_attention_backward_q(
+        dtype, one, one, one, one, one, row_lse, one, one, one, one, 0.125, 1, 256, 256, 64, BH, 64, None)
+    assert bq(dtype=0) == _lib.E_DTYPE
+    assert bq(row_lse=None) == _lib.E_NULL
+    assert bq(BH=16) == _lib.E_CONFIG
+    kv = lambda dtype=f16, row_lse=one, kind=i64, BH=64, BW=64: lib.spx_attention_backward_kv_recompute(
+        dtype, one, one, one, one, row_lse, one, one, one, one, one, kind, 0.125, 1, 256, 256, 64, BH, BW, None)
+    assert kv(dtype=0) == _lib.E_DTYPE
+    assert kv(row_lse=None) == _lib.E_NULL
+    assert kv(kind=_lib.IDX_BCSR_I32) == _lib.E_CONFIG and 'BCSC' in _lib.last_error()
+    assert kv(BH=128, BW=32) == _lib.E_CONFIG and 'BH <= 2 * BW' in _lib.last_error()
+    # batched index build: nothing to do, no job array, a job with a bad shape
+    assert lib.spx_bcs_index_batch(None, 0, None) == 0
+    assert lib.spx_bcs_index_batch(None, 2, None) == _lib.E_NULL
+    jobs = (_lib.BcsIndexJob * 2)()
+    assert lib.spx_bcs_index_batch(jobs, 2, None) == _lib.E_CONFIG
+    jobs[0].H, jobs[0].W, jobs[0].BH, jobs[0].BW = 64, 60, 32, 32
+    assert lib.spx_bcs_index_batch(jobs, 1, None) == _lib.E_SHAPE
+    # index build on the library's own scratch: limits are checked before the array is looked up
+    assert lib.spx_bcs_index_static_max_bytes() == 1 << 20
+    rc = lib.spx_bcs_index_static(None, 64, 64, 3, 32, None, None, None, None, 0, None, 0, None)
+    assert rc == _lib.E_CONFIG
+    rc = lib.spx_bcs_index_static(one, 65536, 65536, 4, 4, one, one, None, None, 0, one, 1 << 28, None)
+    assert rc == _lib.E_WORKSPACE and 'spx_bcs_index' in _lib.last_error()
+    # fused activation: sparse-output products have none
+    rc = lib.spx_matmul(_lib.DDS, 1, 0, 1, 1, one, one, None, one, one, one, 0, None, 1, None, 0, 1, 64, 64, 64, 32, 32, 32,
+                        _lib.EPILOGUE_RELU, None)
+    assert rc == _lib.E_CONFIG and 'sdd and dsd' in _lib.last_error()
+    # MoE
+    moe = lambda dtype=f16, tokens=one, weight=one, layout=1, n_tok=16, in_dim=64, cfg=0: lib.spx_moe_forward(
+        dtype, tokens, weight, layout, one, one, one, n_tok, in_dim, 64, 2, cfg, None)
+    assert moe(cfg=9) == _lib.E_CONFIG
+    assert moe(dtype=7) == _lib.E_DTYPE
+    assert moe(in_dim=72) == _lib.E_SHAPE
+    assert moe(layout=3) == _lib.E_CONFIG
+    assert moe(n_tok=0, tokens=None, weight=None) == 0
+    assert moe(weight=None) == _lib.E_NULL
+    assert moe(tokens=ctypes.c_void_p(264)) == _lib.E_ALIGN
+    assert lib.spx_moe_index_workspace_bytes(1000, 8) >= 9 * 4 and lib.spx_moe_index_workspace_bytes(1000, 0) == 0
+    assert lib.spx_moe_index(one, 16, 0, one, one, one, one, 1024, None) == _lib.E_SHAPE
+    assert lib.spx_moe_index(one, 1000, 8, one, one, one, one, 16, None) == _lib.E_WORKSPACE
+    assert lib.spx_moe_index(one, 1000, 8, None, one, one, one, 1 << 20, None) == _lib.E_NULL
+
+
 def test_cpu_tensors_are_rejected_loudly():
     with pytest.raises(RuntimeError, match='GPU only'):
         _lib.dev_ptr(torch.zeros(4))
