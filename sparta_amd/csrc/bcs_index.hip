@@ -815,6 +815,7 @@ extern "C" int spx_bcs_index_static(const uint8_t* mask, int H, int W, int BH, i
     using namespace spx;
     int rc = check_index_shape(H, W, BH, BW);
     if (rc) return rc;
+    SPX_REQUIRE(mask && nnz_dev, SPX_E_NULL, "mask and nnz_dev are required");
     const size_t need = index_workspace(H, W, BH, BW).total;
     SPX_REQUIRE(need <= BCS_SCRATCH_BYTES, SPX_E_WORKSPACE,
                 "a (%d,%d) mask in (%d,%d) blocks needs %zu bytes of scratch, the static buffer holds %zu: "

@@ -126,6 +126,8 @@ def test_host_validation_of_recompute_batch_and_moe_entry_points():
     assert lib.spx_bcs_index_static_max_bytes() == 1 << 20
     rc = lib.spx_bcs_index_static(None, 64, 64, 3, 32, None, None, None, None, 0, None, 0, None)
     assert rc == _lib.E_CONFIG
+    rc = lib.spx_bcs_index_static(None, 64, 64, 32, 32, one, one, None, None, 0, one, 4, None)
+    assert rc == _lib.E_NULL
     rc = lib.spx_bcs_index_static(one, 65536, 65536, 4, 4, one, one, None, None, 0, one, 1 << 28, None)
     assert rc == _lib.E_WORKSPACE and 'spx_bcs_index' in _lib.last_error()
     # fused activation: sparse-output products have none
