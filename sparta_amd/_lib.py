@@ -138,7 +138,14 @@ def dev_ptr(t: Optional[torch.Tensor]):
     return _c.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def current_stream(device=None):
+    """The current stream of `device` as a C pointer.  A torch.device with an index takes the
+    short way (no Stream object is built: this runs once per kernel launch)."""
+    if _raw_stream is not None and isinstance(device, torch.device) and device.index is not None:
+        return _c.c_void_p(_raw_stream(device.index))
     return _c.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
