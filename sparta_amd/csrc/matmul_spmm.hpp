@@ -266,7 +266,10 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
             tile_cfg = 10;
         else if (panel_ok && p.Mc >= 512 && fill) tile_cfg = p.Mc >= 1024 ? 7 : 5;
         else if (ksplit_ok && !fill && p.K / p.BK >= 8) tile_cfg = 8;  // few tiles, long block-columns
-        else if (panel7_ok && p.Mc >= 512 && fill) tile_cfg = 7;
+        // operands that are not both k-contiguous (input gradients, transposed layouts) have only
+        // the LDS-staged kernel besides 7, which 7 beats two- to threefold at every size measured
+        // (64 to 8192 rows, 10 to 99 % sparsity)
+        else if (panel7_ok && (!kcontig || (p.Mc >= 512 && fill))) tile_cfg = 7;
         else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
         else tile_cfg = p.Mc >= 1024 && fill ? 2 : 1;
     }
