@@ -270,6 +270,9 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
         // the LDS-staged kernel besides 7, which 7 beats two- to threefold at every size measured
         // (64 to 8192 rows, 10 to 99 % sparsity)
         else if (panel7_ok && (!kcontig || (p.Mc >= 512 && fill))) tile_cfg = 7;
+        // sparse blocks wider than the K-split kernel takes: the register-direct kernel only while
+        // the problem is small and its block-columns short (measured 2 - 3x behind 5 otherwise)
+        else if (panel_ok && !ksplit_ok && (big_tiles >= 128 || (big_tiles >= 64 && p.K / p.BK >= 64))) tile_cfg = 5;
         else if (kcontig) tile_cfg = p.Mc >= 1024 && fill ? 4 : 3;
         else tile_cfg = p.Mc >= 1024 && fill ? 2 : 1;
     }
