@@ -375,21 +375,26 @@ static int launch_dds_pipe_inst(const DdsParams& p, int nnz_bound, int batch, hi
 // k-contiguous MFMA fragments come from the LDS transpose read of gfx950 for the 16-bit
 // types (lane i of a 16-lane group addresses 4 entries of k-row i/4, lane j receives
 // column j of the four rows) or from four 4-byte reads for fp32.
-template <typename T, int BM, int BN, int NST>
+// AT / BT say which of the two is stored that way; an operand with the flag off is
+// k-contiguous ([M, K] / [N, K]), kept as [m][k] rows in its part of the stage and read
+// with plain 16-byte fragment loads as in dds_pipe_kernel - the mixed layouts of a plain
+// C = A B (A [M, K], B [K, N]) and of C = A^T B^T.
+template <typename T, int BM, int BN, int NST, bool AT = true, bool BT = true>
 __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
     constexpr int MT = BM / 16, NT = BN / 16;
     typedef DdsWaveGrid<MT, NT> G;
     constexpr int ES = (int)sizeof(T);
     constexpr int VE = 16 / ES;
-    constexpr int KT = DdsPipeCfg<BM, BN>::STAGE_BYTES / ES;   // k-rows per stage
+    constexpr int KT = DdsPipeCfg<BM, BN>::STAGE_BYTES / ES;   // k per stage
     constexpr int KW = KT / G::KS;
-    constexpr int LDA = BM + VE, LDB = BN + VE;                // row pitches (elements)
-    constexpr int A_BYTES = KT * LDA * ES;
-    constexpr int BUF = KT * (LDA + LDB) * ES;
-    constexpr int CA = BM / VE, CB = BN / VE;                  // 16-byte chunks per k-row
-    constexpr int NA = KT * CA;                                // chunks of the A part
-    constexpr int NV = KT * (CA + CB) / 256;
-    static_assert(KT * (CA + CB) % 256 == 0, "stage does not split over the workgroup");
+    constexpr int LDA = (AT ? BM : KT) + VE, LDB = (BT ? BN : KT) + VE;   // row pitches (elements)
+    constexpr int A_ROWS = AT ? KT : BM, B_ROWS = BT ? KT : BN;           // LDS rows of the two parts
+    constexpr int A_BYTES = A_ROWS * LDA * ES;
+    constexpr int BUF = A_BYTES + B_ROWS * LDB * ES;
+    constexpr int CA = (AT ? BM : KT) / VE, CB = (BT ? BN : KT) / VE;     // 16-byte chunks per row
+    constexpr int NA = A_ROWS * CA;                            // chunks of the A part
+    constexpr int NV = (NA + B_ROWS * CB) / 256;
+    static_assert((NA + B_ROWS * CB) % 256 == 0, "stage does not split over the workgroup");
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -410,10 +415,11 @@ __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
     const int wgm = wt / G::WGN;
     const int wgn = wt % G::WGN;
 
-    const T* A = reinterpret_cast<const T*>(p.A) + b * p.a_batch + (int64_t)bi * BM;
-    const T* B = reinterpret_cast<const T*>(p.B) + b * p.b_batch + (int64_t)bj * BN;
+    const T* A = reinterpret_cast<const T*>(p.A) + b * p.a_batch + (int64_t)bi * BM * (AT ? 1 : p.a_ld);
+    const T* B = reinterpret_cast<const T*>(p.B) + b * p.b_batch + (int64_t)bj * BN * (BT ? 1 : p.b_ld);
 
-    // staging map: chunk v = tid + 256 u; the first NA chunks are (k-row, piece) of A, the rest of B
+    // staging map: chunk v = tid + 256 u; the first NA chunks are (row, piece) of the A part
+    // (k-rows, or rows of the block with the stage's k range), the rest of the B part
     const T* src[NV];
     int64_t sstep[NV];
     int dst[NV];
@@ -421,16 +427,16 @@ __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
     for (int u = 0; u < NV; ++u) {
         const int v = threadIdx.x + 256 * u;
         if (v < NA) {
-            const int k = v / CA, c = v % CA;
-            src[u] = A + (int64_t)k * p.a_ld + c * VE;
-            sstep[u] = (int64_t)KT * p.a_ld;
-            dst[u] = (k * LDA + c * VE) * ES;
+            const int r = v / CA, c = v % CA;
+            src[u] = A + (int64_t)r * p.a_ld + c * VE;
+            sstep[u] = AT ? (int64_t)KT * p.a_ld : (int64_t)KT;
+            dst[u] = (r * LDA + c * VE) * ES;
         } else {
             const int w = v - NA;
-            const int k = w / CB, c = w % CB;
-            src[u] = B + (int64_t)k * p.b_ld + c * VE;
-            sstep[u] = (int64_t)KT * p.b_ld;
-            dst[u] = A_BYTES + (k * LDB + c * VE) * ES;
+            const int r = w / CB, c = w % CB;
+            src[u] = B + (int64_t)r * p.b_ld + c * VE;
+            sstep[u] = BT ? (int64_t)KT * p.b_ld : (int64_t)KT;
+            dst[u] = A_BYTES + (r * LDB + c * VE) * ES;
         }
     }
 
@@ -455,6 +461,9 @@ __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
     const int b_tr = A_BYTES + ((g4 * 8 + (r16 >> 2)) * LDB + (wgn * G::WTN * 16 + (r16 & 3) * 4)) * ES;
     const int a_f32 = ((g4 * 4) * LDA + wgm * G::WTM * 16 + r16) * ES;
     const int b_f32 = A_BYTES + ((g4 * 4) * LDB + wgn * G::WTN * 16 + r16) * ES;
+    // k-contiguous parts: row r16 of the wavefront's first tile, element 0 of the row
+    const int a_row = ((wgm * G::WTM * 16 + r16) * LDA) * ES;
+    const int b_row = A_BYTES + ((wgn * G::WTN * 16 + r16) * LDB) * ES;
     for (int it = 0; it < n_st; it += NST) {
 #pragma unroll
         for (int r = 0; r < NST; ++r) {
@@ -480,15 +489,23 @@ __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
                         Frag af[G::WTM], bf[G::WTN];
 #pragma unroll
                         for (int x = 0; x < G::WTM; ++x) {
-                            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + a_tr + (kb * LDA + x * 16) * ES));
-                            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + a_tr + ((kb + 4) * LDA + x * 16) * ES));
-                            af[x] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                            if constexpr (AT) {
+                                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + a_tr + (kb * LDA + x * 16) * ES));
+                                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + a_tr + ((kb + 4) * LDA + x * 16) * ES));
+                                af[x] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                            } else {
+                                af[x] = Mma32<T>::load(reinterpret_cast<const T*>(buf + a_row) + x * 16 * LDA + kb + g4 * 8);
+                            }
                         }
 #pragma unroll
                         for (int y = 0; y < G::WTN; ++y) {
-                            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + b_tr + (kb * LDB + y * 16) * ES));
-                            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + b_tr + ((kb + 4) * LDB + y * 16) * ES));
-                            bf[y] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                            if constexpr (BT) {
+                                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + b_tr + (kb * LDB + y * 16) * ES));
+                                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(buf + b_tr + ((kb + 4) * LDB + y * 16) * ES));
+                                bf[y] = __builtin_bit_cast(Frag, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                            } else {
+                                bf[y] = Mma32<T>::load(reinterpret_cast<const T*>(buf + b_row) + y * 16 * LDB + kb + g4 * 8);
+                            }
                         }
 #pragma unroll
                         for (int x = 0; x < G::WTM; ++x)
@@ -501,15 +518,25 @@ __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
                         const int kb = kpart * KW + kc;
                         typename Mma16<T>::frag af[G::WTM], bf[G::WTN];
 #pragma unroll
-                        for (int x = 0; x < G::WTM; ++x)
+                        for (int x = 0; x < G::WTM; ++x) {
+                            if constexpr (AT) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                af[x][j] = *reinterpret_cast<const float*>(buf + a_f32 + ((kb + j) * LDA + x * 16) * ES);
+                                for (int j = 0; j < 4; ++j)
+                                    af[x][j] = *reinterpret_cast<const float*>(buf + a_f32 + ((kb + j) * LDA + x * 16) * ES);
+                            } else {
+                                af[x] = Mma16<T>::load(reinterpret_cast<const T*>(buf + a_row) + x * 16 * LDA + kb + g4 * 4);
+                            }
+                        }
 #pragma unroll
-                        for (int y = 0; y < G::WTN; ++y)
+                        for (int y = 0; y < G::WTN; ++y) {
+                            if constexpr (BT) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                bf[y][j] = *reinterpret_cast<const float*>(buf + b_f32 + ((kb + j) * LDB + y * 16) * ES);
+                                for (int j = 0; j < 4; ++j)
+                                    bf[y][j] = *reinterpret_cast<const float*>(buf + b_f32 + ((kb + j) * LDB + y * 16) * ES);
+                            } else {
+                                bf[y] = Mma16<T>::load(reinterpret_cast<const T*>(buf + b_row) + y * 16 * LDB + kb + g4 * 4);
+                            }
+                        }
 #pragma unroll
                         for (int x = 0; x < G::WTM; ++x)
 #pragma unroll
@@ -523,21 +550,23 @@ __global__ __launch_bounds__(256) void dds_pipe_t_kernel(DdsParams p) {
     dds_epilogue<T, BM, BN>(p, acc, reinterpret_cast<float*>(smem), i, bi, bj, b, wgm, wgn, kpart, r16, g4);
 }
 
-template <typename T, int BM, int BN>
+template <typename T, int BM, int BN, bool AT = true, bool BT = true>
 static int launch_dds_pipe_t_inst(const DdsParams& p, int nnz_bound, int batch, hipStream_t st) {
     constexpr int VE = 16 / (int)sizeof(T);
     constexpr int KT = DdsPipeCfg<BM, BN>::STAGE_BYTES / (int)sizeof(T);
     constexpr int NST = DdsPipeCfg<BM, BN>::NST;
     typedef DdsWaveGrid<BM / 16, BN / 16> G;
-    size_t smem = 2 * (size_t)KT * (BM + BN + 2 * VE) * sizeof(T);
+    constexpr size_t a_part = AT ? (size_t)KT * (BM + VE) : (size_t)BM * (KT + VE);
+    constexpr size_t b_part = BT ? (size_t)KT * (BN + VE) : (size_t)BN * (KT + VE);
+    size_t smem = 2 * (a_part + b_part) * sizeof(T);
     size_t epi = (size_t)G::KS * BM * (BN + 4) * sizeof(float);
     if (epi > smem) smem = epi;
     if (smem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_pipe_t_kernel<T, BM, BN, NST>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dds_pipe_t_kernel<T, BM, BN, NST, AT, BT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(dds_pipe_t_kernel)");
     }
-    hipLaunchKernelGGL((dds_pipe_t_kernel<T, BM, BN, NST>), dim3(nnz_bound, batch, 1), dim3(256), smem, st, p);
+    hipLaunchKernelGGL((dds_pipe_t_kernel<T, BM, BN, NST, AT, BT>), dim3(nnz_bound, batch, 1), dim3(256), smem, st, p);
     SPX_LAUNCH_CHECK("dds_pipe_t_kernel");
     return 0;
 }
@@ -857,7 +886,7 @@ static int dds_pipe_ok(const DdsParams& p, int BM, int BN) {
     if (p.K % stage != 0) return 0;
     if (p.a_kcontig && p.b_kcontig) return 1;
     if (!p.a_kcontig && !p.b_kcontig) return 2;
-    return 0;
+    return p.a_kcontig ? 3 : 4;   // mixed: A k-contiguous and B [K, N], or A [K, M] and B k-contiguous
 }
 
 template <typename T, int BM, int BN>
@@ -891,12 +920,14 @@ int launch_dds_impl(const DdsParams& p, int BM, int BN, int nnz_bound, int batch
         return launch_dds_row<T>(p, BM, BN, batch, st);
     }
     if (tile_cfg == 2 && !pipe)
-        return fail(SPX_E_CONFIG, "tile config 2 needs both operands stored the same way round and K a multiple of the stage depth");
+        return fail(SPX_E_CONFIG, "tile config 2 needs K to be a multiple of the stage depth");
 #define SPX_DDS_CASE(bm, bn) \
     if (BM == bm && BN == bn) \
         return tile_cfg != 2 ? launch_dds_inst<T, bm, bn>(p, nnz_bound, batch, st) \
              : pipe == 1 ? launch_dds_pipe_inst<T, bm, bn>(p, nnz_bound, batch, st) \
-                         : launch_dds_pipe_t_inst<T, bm, bn>(p, nnz_bound, batch, st);
+             : pipe == 2 ? launch_dds_pipe_t_inst<T, bm, bn>(p, nnz_bound, batch, st) \
+             : pipe == 3 ? launch_dds_pipe_t_inst<T, bm, bn, false, true>(p, nnz_bound, batch, st) \
+                         : launch_dds_pipe_t_inst<T, bm, bn, true, false>(p, nnz_bound, batch, st);
     SPX_DDS_CASE(16, 16) SPX_DDS_CASE(16, 32) SPX_DDS_CASE(16, 64)
     SPX_DDS_CASE(32, 16) SPX_DDS_CASE(32, 32) SPX_DDS_CASE(32, 64)
     SPX_DDS_CASE(64, 16) SPX_DDS_CASE(64, 32) SPX_DDS_CASE(64, 64)
