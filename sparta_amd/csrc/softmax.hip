@@ -439,7 +439,11 @@ static int launch_softmax(int dtype, int compressed, const void* x, const void* 
     const int ve = dtype == SPX_F32 ? 4 : 8;
     const bool vec_ok = BW % ve == 0 && aligned(x, 16) && aligned(out, 16) && (!y_in || aligned(y_in, 16)) &&
                         (!mask || aligned(mask, 8)) && batch_stride % ve == 0;
-    if (tile_cfg == 0) tile_cfg = vec_ok ? (W / ve <= 16 * SMV_CACHE ? 3 : 2) : 1;
+    // Few long rows (under 8192 in all, 256 vectors wide or more) also take a wavefront each:
+    // sixteen-lane groups would leave most of the device without work (3072 rows of 4096:
+    // 3.7 against 5.8 us forward, 3.8 against 6.7 us backward).
+    const bool few_long_rows = (int64_t)H * batch < 8192 && W / ve >= 256;
+    if (tile_cfg == 0) tile_cfg = vec_ok ? (W / ve <= 16 * SMV_CACHE && !few_long_rows ? 3 : 2) : 1;
     if (tile_cfg >= 2) {
         SPX_REQUIRE(vec_ok, SPX_E_CONFIG, "tile configs 2 and 3 need BW %% %d == 0 and 16-byte aligned tensors", ve);
         const bool narrow = tile_cfg == 3;
