@@ -269,7 +269,9 @@ int launch_spmm_impl(const SpmmParams& p, int BN, int batch, int tile_cfg, hipSt
         // operands that are not both k-contiguous (input gradients, transposed layouts) have only
         // the LDS-staged kernel besides 7, which 7 beats two- to threefold at every size measured
         // (64 to 8192 rows, 10 to 99 % sparsity)
-        else if (panel7_ok && (!kcontig || (p.Mc >= 512 && fill))) tile_cfg = 7;
+        // (fp32 with an m-contiguous dense operand builds its fragments from 4-byte LDS reads and
+        // only pays on large problems: 1024^3 29.7 against 17.5 us)
+        else if (panel7_ok && ((!kcontig && (sizeof(T) == 2 || p.d_kcontig)) || (p.Mc >= 512 && fill))) tile_cfg = 7;
         // sparse blocks wider than the K-split kernel takes: the register-direct kernel only while
         // the problem is small and its block-columns short (measured 2 - 3x behind 5 otherwise)
         else if (panel_ok && !ksplit_ok && (big_tiles >= 128 || (big_tiles >= 64 && p.K / p.BK >= 64))) tile_cfg = 5;
