@@ -8,7 +8,9 @@
 //      of the tile non-zero").
 //   2. emit_kernel (one workgroup): turns the byte map into 64-block words with
 //      wavefront ballots, prefix-scans the word popcounts (which directly yields
-//      row_ptr / col_ptr and every block's rank), and writes the index arrays.
+//      row_ptr / col_ptr and every block's rank), and writes the index arrays.  With
+//      more than 256 words the same three steps run as three launches, the first and
+//      the last with one wavefront per word (emit_general_*_kernel).
 // Replaces bcs_index_1 / bcs_index_2 of the reference
 // (sparta/tesa/templates/block_compressed.cu.j2:67-170) and the cumsum + .item()
 // glue of sparta/tesa/block_compressed.py:242-309.
@@ -230,6 +232,99 @@ __global__ __launch_bounds__(1024) void emit_kernel(EmitParams p) {
         }
     }
     if (p.col_order) schedule_segments(p.col_ptr, p.Cn, p.col_order, s_bins);
+}
+
+// ---- the same work spread over the device, for block grids with many words ----------------
+// emit_kernel walks the words with the sixteen wavefronts of one workgroup, one dependent
+// load per step: a grid of 4096 row words takes it 200 us.  The three kernels below do the
+// same steps in the same order of results - word building and index writing by one
+// wavefront per word across as many workgroups as there are words, the two prefix sums,
+// the pointer arrays and the launch orders by a single workgroup in between.
+
+// wavefront g < NW: row word g (bits and popcount); NW <= g < NW + NWC: popcount of column word g - NW
+__global__ __launch_bounds__(256) void emit_general_words_kernel(EmitParams p) {
+    const int lane = lane_id();
+    const int g = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int NW = p.R * p.WPR;
+    const int NWC = p.col_ptr ? p.Cn * p.WPC : 0;
+    if (g < NW) {
+        const int r = g / p.WPR;
+        const int c = (g - r * p.WPR) * 64 + lane;
+        const bool flag = c < p.Cn && p.live[(int64_t)r * p.Cn + c] != 0;
+        const unsigned long long word = __ballot(flag);
+        if (lane == 0) {
+            p.wbits[g] = word;
+            p.wbase[g] = __popcll(word);
+        }
+    } else if (g < NW + NWC) {
+        const int gc = g - NW;
+        const int c = gc / p.WPC;
+        const int r = (gc - c * p.WPC) * 64 + lane;
+        const bool flag = r < p.R && p.live[(int64_t)r * p.Cn + c] != 0;
+        const unsigned long long word = __ballot(flag);
+        if (lane == 0) p.cbase[gc] = __popcll(word);
+    }
+}
+
+__global__ __launch_bounds__(1024) void emit_general_scan_kernel(EmitParams p) {
+    __shared__ int lds[32];
+    __shared__ int s_bins[256];
+    const int NW = p.R * p.WPR;
+    const int nnz = block_scan_inplace(p.wbase, NW, lds);
+    if (threadIdx.x == 0) p.nnz_dev[0] = nnz;
+    if (p.row_ptr) {
+        __syncthreads();   // the scanned values were written by other threads of the workgroup
+        for (int r = threadIdx.x; r < p.R; r += blockDim.x) p.row_ptr[r] = p.wbase[r * p.WPR];
+        if (threadIdx.x == 0) p.row_ptr[p.R] = nnz;
+    }
+    if (p.row_order && p.row_ptr) schedule_segments(p.row_ptr, p.R, p.row_order, s_bins);
+    if (!p.col_ptr) return;  // uniform over the workgroup
+    __syncthreads();
+    const int NWC = p.Cn * p.WPC;
+    const int nnz2 = block_scan_inplace(p.cbase, NWC, lds);
+    __syncthreads();
+    for (int c = threadIdx.x; c < p.Cn; c += blockDim.x) p.col_ptr[c] = p.cbase[c * p.WPC];
+    if (threadIdx.x == 0) p.col_ptr[p.Cn] = nnz2;
+    if (p.col_order) schedule_segments(p.col_ptr, p.Cn, p.col_order, s_bins);
+}
+
+// wavefront g < NW: the BCSR entries of row word g; NW <= g < NW + NWC: the BCSC entries of column word g - NW
+__global__ __launch_bounds__(256) void emit_general_write_kernel(EmitParams p) {
+    const int lane = lane_id();
+    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int g = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int NW = p.R * p.WPR;
+    const int NWC = p.bcsc_idx ? p.Cn * p.WPC : 0;
+    if (g < NW) {
+        if (!p.bcsr_idx) return;
+        const int r = g / p.WPR;
+        const int c = (g - r * p.WPR) * 64 + lane;
+        const unsigned long long word = p.wbits[g];
+        if ((word >> lane) & 1ull) {
+            const int pos = p.wbase[g] + __popcll(word & lt_mask);
+            if (pos < p.cap) p.bcsr_idx[pos] = (r << 16) | c;
+        }
+    } else if (g < NW + NWC) {
+        const int gc = g - NW;
+        const int c = gc / p.WPC;
+        const int r = (gc - c * p.WPC) * 64 + lane;
+        const bool flag = r < p.R && p.live[(int64_t)r * p.Cn + c] != 0;
+        const unsigned long long word = __ballot(flag);
+        if (flag) {
+            const int pos = p.cbase[gc] + __popcll(word & lt_mask);
+            if (pos < p.cap) {
+                if (p.bcsc_i64) {
+                    const int gw = r * p.WPR + (c >> 6);
+                    const int cl = c & 63;
+                    const unsigned long long below = cl == 0 ? 0ull : (p.wbits[gw] & (~0ull >> (64 - cl)));
+                    const long long bpos = p.wbase[gw] + __popcll(below);
+                    reinterpret_cast<long long*>(p.bcsc_idx)[pos] = (bpos << 32) | ((long long)c << 16) | (long long)r;
+                } else {
+                    reinterpret_cast<int32_t*>(p.bcsc_idx)[pos] = (c << 16) | r;
+                }
+            }
+        }
+    }
 }
 
 // ---- fast path: block grids of at most 2048 row words and 2048 column words ----------
@@ -719,8 +814,19 @@ static int spx::bcs_index_impl(const uint8_t* mask, int H, int W, int BH, int BW
     else if (vec == 4) hipLaunchKernelGGL(liveness_kernel<4>, grid, dim3(256), 0, st, lp);
     else hipLaunchKernelGGL(liveness_kernel<1>, grid, dim3(256), 0, st, lp);
     SPX_LAUNCH_CHECK("liveness_kernel");
-    hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
-    SPX_LAUNCH_CHECK("emit_kernel");
+    const int64_t n_words = (int64_t)ws.R * ws.WPR + (col_ptr ? (int64_t)ws.Cn * ws.WPC : 0);
+    if (n_words <= 256) {   // few words: one workgroup does all of it in one launch
+        hipLaunchKernelGGL(emit_kernel, dim3(1), dim3(1024), 0, st, ep);
+        SPX_LAUNCH_CHECK("emit_kernel");
+        return 0;
+    }
+    const unsigned word_groups = (unsigned)((n_words + 3) / 4);
+    hipLaunchKernelGGL(emit_general_words_kernel, dim3(word_groups), dim3(256), 0, st, ep);
+    SPX_LAUNCH_CHECK("emit_general_words_kernel");
+    hipLaunchKernelGGL(emit_general_scan_kernel, dim3(1), dim3(1024), 0, st, ep);
+    SPX_LAUNCH_CHECK("emit_general_scan_kernel");
+    hipLaunchKernelGGL(emit_general_write_kernel, dim3(word_groups), dim3(256), 0, st, ep);
+    SPX_LAUNCH_CHECK("emit_general_write_kernel");
     return 0;
 }
 

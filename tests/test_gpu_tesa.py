@@ -145,6 +145,8 @@ def test_index_reference_shapes(BH, BW, gpu):
     ((64, 96), (4, 4), (1, 1), 0.5),
     ((256, 8), (4, 8), (1, 1), 0.9),             # single block column
     ((8, 20), (4, 4), (1, 1), 0.3),              # row pitch not a multiple of 16
+    ((4096, 4096), (8, 8), (8, 8), 0.90),        # 4096 row words: the general path, one wavefront per word
+    ((2048, 1032), (8, 8), (1, 1), 0.999),       # the same path with 4-byte loads and a partial last word per row
 ])
 def test_index_bench_shapes(shape, block, gran, sparsity, gpu):
     _check_indexes(ops.block_mask(shape, gran, sparsity, seed=2022), block[0], block[1], gpu)
