@@ -45,61 +45,50 @@ __global__ __launch_bounds__(256) void moe_hist_kernel(const int32_t* exp_ids, i
     for (int e = threadIdx.x; e < n_exp; e += 256) partial[(int64_t)blockIdx.x * n_exp + e] = hist[e];
 }
 
-// One workgroup: exclusive scan of partial[] in (expert, chunk) order, in place;
-// also writes expert_count [n_exp - 1] and expert_offset [n_exp] (n_exp counts the
-// pseudo expert of out-of-range ids, whose tokens follow those of the real experts, so
-// expert_offset[n_exp - 1] is the number of tokens with a valid id).
-__global__ __launch_bounds__(1024) void moe_scan_kernel(int32_t* partial, int n_chunk, int n_exp,
-                                                        int32_t* expert_count, int32_t* expert_offset) {
-    __shared__ int lds[32];
+// Wavefront e: exclusive prefix of expert e's counts over the chunks, in place, and the
+// expert's total.  Every lane takes a run of consecutive chunks (sums it, then rewrites it
+// from the lane's offset), so the serial part is 1/64 of the chunks.  n_exp counts the
+// pseudo expert of out-of-range ids.
+__global__ __launch_bounds__(256) void moe_colscan_kernel(int32_t* partial, int n_chunk, int n_exp, int32_t* totals) {
     const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
-    const int n = n_chunk * n_exp;
-    int carry = 0;
-    if (n == 0)
-        for (int e = threadIdx.x; e < n_exp; e += 1024) expert_offset[e] = 0;
-    for (int base = 0; base < n; base += 1024) {
-        const int i = base + threadIdx.x;  // position in (expert, chunk) order
-        int v = 0, e = 0, c = 0;
-        if (i < n) {
-            e = i / n_chunk;
-            c = i - e * n_chunk;
-            v = partial[(int64_t)c * n_exp + e];
-        }
-        const int inc = wave_inclusive_scan(v);
-        if (lane == 63) lds[wave] = inc;
-        __syncthreads();
-        int before = 0, total = 0;
-        for (int w = 0; w < 16; ++w) {
-            const int t = lds[w];
-            if (w < wave) before += t;
-            total += t;
-        }
-        if (i < n) {
-            const int excl = carry + before + inc - v;
-            partial[(int64_t)c * n_exp + e] = excl;
-            if (c == 0) expert_offset[e] = excl;
-        }
-        carry += total;
-        __syncthreads();
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (e >= n_exp) return;
+    const int per = (n_chunk + 63) / 64;
+    const int c0 = lane * per < n_chunk ? lane * per : n_chunk;
+    const int c1 = c0 + per < n_chunk ? c0 + per : n_chunk;
+    int sum = 0;
+    for (int c = c0; c < c1; ++c) sum += partial[(int64_t)c * n_exp + e];
+    const int inc = wave_inclusive_scan(sum);
+    int run = inc - sum;
+    for (int c = c0; c < c1; ++c) {
+        const int v = partial[(int64_t)c * n_exp + e];
+        partial[(int64_t)c * n_exp + e] = run;
+        run += v;
     }
-    __syncthreads();
-    // counts from consecutive offsets (offsets were written by this workgroup)
-    for (int e = threadIdx.x; e + 1 < n_exp; e += 1024) expert_count[e] = expert_offset[e + 1] - expert_offset[e];
+    if (lane == 63) totals[e] = inc;
+}
+
+__global__ __launch_bounds__(256) void moe_zero_index_kernel(int n_exp, int32_t* expert_count, int32_t* expert_offset) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e < n_exp) expert_count[e] = 0;
+    if (e <= n_exp) expert_offset[e] = 0;
 }
 
 // Stable placement of one chunk.  Waves take 64 tokens at a time; inside a wave the
 // rank among equal experts comes from ballots, between waves from a small table.
 // FUSED: `counts` holds the raw per-chunk histograms (at most MOE_FUSED_TABLE of them);
 // every workgroup scans them in (expert, chunk) order itself and workgroup 0 also writes
-// expert_offset and expert_count.  Otherwise `counts` was scanned by moe_scan_kernel.
+// expert_offset and expert_count.  Otherwise `counts` holds every expert's prefix over the
+// chunks (moe_colscan_kernel) and `totals` the experts' token counts, which every workgroup
+// turns into the experts' offsets itself (at most MOE_MAX_EXP + 1 of them).
 template <bool FUSED>
 __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, int n_tok, int n_exp, int chunk,
-                                                        const int32_t* counts, int32_t* token_perm,
+                                                        const int32_t* counts, const int32_t* totals, int32_t* token_perm,
                                                         int32_t* expert_count, int32_t* expert_offset) {
     extern __shared__ int sm[];
     int* running = sm;               // [n_exp] tokens of expert e already placed by this chunk
     int* wavecnt = sm + n_exp;       // [4][n_exp] tokens of expert e in the current pass, per wave
+    int* ebase = sm + 5 * n_exp;     // [n_exp] first position of expert e (not FUSED)
     __shared__ int tab[FUSED ? MOE_FUSED_TABLE : 1];
     __shared__ int wave_total[4];
     const int lane = lane_id();
@@ -139,6 +128,32 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, 
             }
         }
     }
+    if constexpr (!FUSED) {
+        // experts per * tid .. per * tid + per - 1: exclusive scan of their totals
+        const int per = (n_exp + 255) / 256;
+        int sum = 0;
+        for (int j = 0; j < per; ++j) {
+            const int e = threadIdx.x * per + j;
+            if (e < n_exp) sum += totals[e];
+        }
+        const int inc = wave_inclusive_scan(sum);
+        if (lane == 63) wave_total[wave] = inc;
+        __syncthreads();
+        int excl = inc - sum;
+        for (int w = 0; w < wave; ++w) excl += wave_total[w];
+        for (int j = 0; j < per; ++j) {
+            const int e = threadIdx.x * per + j;
+            if (e < n_exp) {
+                const int t = totals[e];
+                ebase[e] = excl;
+                if (blockIdx.x == 0) {
+                    expert_offset[e] = excl;
+                    if (e + 1 < n_exp) expert_count[e] = t;
+                }
+                excl += t;
+            }
+        }
+    }
     __syncthreads();
     const int chunk0 = blockIdx.x * chunk;
     const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
@@ -169,7 +184,7 @@ __global__ __launch_bounds__(256) void moe_place_kernel(const int32_t* exp_ids, 
         if (e >= 0) {
             int before = running[e];
             for (int w = 0; w < wave; ++w) before += wavecnt[w * n_exp + e];
-            const int base = FUSED ? tab[e * gridDim.x + blockIdx.x] : counts[(int64_t)blockIdx.x * n_exp + e];
+            const int base = FUSED ? tab[e * gridDim.x + blockIdx.x] : ebase[e] + counts[(int64_t)blockIdx.x * n_exp + e];
             token_perm[base + before + rank] = t;
         }
         __syncthreads();
@@ -814,21 +829,29 @@ static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
 
 // Tokens per workgroup of the index kernels: the smallest multiple of 256 (up to MOE_CHUNK)
 // whose table of (chunk, expert) counts the placement workgroups can scan themselves;
-// MOE_CHUNK with a scan launch when there is none.
+// else 256 (more beyond 262144 tokens, so that a launch has at most 1024 chunks)
+// with a launch in between that scans every expert's column of the table.
 static int moe_index_chunk(int n_tok, int n_exp, bool* fused) {
     for (int chunk = 256; chunk <= MOE_CHUNK; chunk += 256) {
         const int64_t n_chunk = (n_tok + chunk - 1) / chunk;
         if (n_chunk * (n_exp + 1) <= MOE_FUSED_TABLE) { *fused = true; return chunk; }
     }
     *fused = false;
-    return MOE_CHUNK;
+    int chunk = 256;
+    while ((n_tok + chunk - 1) / chunk > 1024) chunk += 256;
+    return chunk;
 }
 
-static size_t moe_index_ws(int n_tok, int n_exp) {
+// [n_chunk][n_exp + 1] counts, then the n_exp + 1 totals of the experts
+static size_t moe_index_table_bytes(int n_tok, int n_exp) {
     bool fused;
     const int chunk = moe_index_chunk(n_tok, n_exp, &fused);
     const int n_chunk = (n_tok + chunk - 1) / chunk;
     return round_up((size_t)(n_chunk > 0 ? n_chunk : 1) * (n_exp + 1) * sizeof(int32_t), 256);
+}
+
+static size_t moe_index_ws(int n_tok, int n_exp) {
+    return moe_index_table_bytes(n_tok, n_exp) + round_up((size_t)(n_exp + 1) * sizeof(int32_t), 256);
 }
 
 }  // namespace spx
@@ -858,20 +881,24 @@ extern "C" int spx_moe_index(const int32_t* exp_ids, int n_tok, int n_exp,
         hipLaunchKernelGGL(moe_hist_kernel, dim3(n_chunk), dim3(256), (n_exp + 1) * sizeof(int), st, exp_ids, n_tok, n_exp + 1, chunk, partial);
         SPX_LAUNCH_CHECK("moe_hist_kernel");
     }
-    if (!fused || n_chunk == 0) {
-        hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(1024), 0, st, partial, n_chunk, n_exp + 1, expert_count, expert_offset);
-        SPX_LAUNCH_CHECK("moe_scan_kernel");
+    int32_t* totals = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) + moe_index_table_bytes(n_tok, n_exp));
+    if (n_chunk == 0) {   // no tokens: all offsets and counts are zero (a kernel, so that the call can be captured)
+        hipLaunchKernelGGL(moe_zero_index_kernel, dim3((n_exp + 1 + 255) / 256), dim3(256), 0, st, n_exp, expert_count, expert_offset);
+        SPX_LAUNCH_CHECK("moe_zero_index_kernel");
+        return 0;
     }
-    if (n_chunk > 0) {
-        const size_t smem = 5 * (n_exp + 1) * sizeof(int);
-        if (fused)
-            hipLaunchKernelGGL(moe_place_kernel<true>, dim3(n_chunk), dim3(256), smem, st, exp_ids, n_tok, n_exp + 1, chunk, partial,
-                               token_perm, expert_count, expert_offset);
-        else
-            hipLaunchKernelGGL(moe_place_kernel<false>, dim3(n_chunk), dim3(256), smem, st, exp_ids, n_tok, n_exp + 1, chunk, partial,
-                               token_perm, expert_count, expert_offset);
-        SPX_LAUNCH_CHECK("moe_place_kernel");
+    if (!fused) {
+        hipLaunchKernelGGL(moe_colscan_kernel, dim3((n_exp + 1 + 3) / 4), dim3(256), 0, st, partial, n_chunk, n_exp + 1, totals);
+        SPX_LAUNCH_CHECK("moe_colscan_kernel");
     }
+    const size_t smem = 6 * (n_exp + 1) * sizeof(int);
+    if (fused)
+        hipLaunchKernelGGL(moe_place_kernel<true>, dim3(n_chunk), dim3(256), smem, st, exp_ids, n_tok, n_exp + 1, chunk, partial,
+                           totals, token_perm, expert_count, expert_offset);
+    else
+        hipLaunchKernelGGL(moe_place_kernel<false>, dim3(n_chunk), dim3(256), smem, st, exp_ids, n_tok, n_exp + 1, chunk, partial,
+                           totals, token_perm, expert_count, expert_offset);
+    SPX_LAUNCH_CHECK("moe_place_kernel");
     return 0;
 }
 
