@@ -60,6 +60,33 @@ class KernelPlaceholder:
         return self.active_kernel().test(self.sample_inputs, num_warmups, num_iters, cuda)
 
 
+def check_shared_block_shapes(placeholders: Dict[str, KernelPlaceholder], built) -> None:
+    """Kernels that share a sparse tensor share one index object, which is rebuilt for the
+    block shape of whichever kernel was bound last: a kernel bound earlier with another
+    block shape keeps an index (and a compressed layout) that no longer matches the values
+    it will be handed.  The kernels named in `built` must therefore agree with their port
+    (AssertionError, like any other invalid combination of parameters); a kernel left
+    over from an earlier build that no longer agrees is switched off, so that calling it
+    raises instead of computing on a stale layout."""
+    for name, placeholder in placeholders.items():
+        kernel = placeholder.active_kernel()
+        if kernel is None or not kernel.ready:
+            continue
+        want = kernel.sparse_block_shape()
+        if want is None:
+            continue
+        for port in kernel.ports.values():
+            # (a port no kernel has given a block shape yet holds no index either)
+            if not port.is_sparse or not port._block_H or (port._block_H, port._block_W) == tuple(want):
+                continue
+            if name in built:
+                raise AssertionError(
+                    f'kernel {name} takes {want[0]}x{want[1]} blocks of its sparse tensor, the kernels it shares '
+                    f'that tensor with take {port._block_H}x{port._block_W}')
+            kernel.ready = False
+            placeholder.ready = False
+
+
 class SparseCtxBase(abc.ABC):
 
     def __init__(self):
@@ -105,6 +132,7 @@ class SparseCtxBase(abc.ABC):
     def build(self, config: Dict[str, Dict[str, Any]]):
         for kernel_name, kernel_config in config.items():
             self._kernels[kernel_name].build(kernel_config)
+        check_shared_block_shapes({name: k for name, k in self._kernels.items()}, config)
 
     def get_sparse_indexes(self, port_name: str):
         ports = self.sparse_ports.get(port_name)

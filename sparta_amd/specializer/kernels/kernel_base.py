@@ -194,6 +194,10 @@ class KernelBase(abc.ABC):
         returns a one-line description instead of source code."""
         return f'// {type(self).__name__}: precompiled gfx950 kernel in libsparta_hip.so'
 
+    def sparse_block_shape(self) -> Optional[Tuple[int, int]]:
+        """(block_H, block_W) this kernel assumes for its sparse tensor, None if it has none."""
+        return None
+
     def compile(self, params: Dict[str, Any]):
         self._check_parameters(params)
         self.set_parameters(params)

@@ -127,6 +127,9 @@ class SparseMatMulKernel(KernelBase):
     def get_block_shape(self):
         return tuple(self.get_parameter(f'BLOCK_SIZE_{d}_VALUE') for d in 'MKN')
 
+    def sparse_block_shape(self):
+        return self.get_parameter(self._sparse_block_H), self.get_parameter(self._sparse_block_W)
+
     def blocks_per_grid(self):
         batch_size, M, K, N = self.get_shape()
         if self._mode == 'dds':

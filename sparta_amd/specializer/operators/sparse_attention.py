@@ -18,6 +18,7 @@ from sparta_amd.specializer.operators.operator_base import OperatorBase
 from sparta_amd.specializer.operators.sparse_matmul import SparseBatchMatMul
 from sparta_amd.specializer.operators.sparse_softmax import SparseSoftmax
 from sparta_amd.specializer.kernels import KernelBase, PortConfig
+from sparta_amd.specializer.funtional.sparse_ctx_base import check_shared_block_shapes
 
 # operator-level name -> (attribute, sparse port of that operator)
 _PARTS = (('qk', '_matmul_qk', 'C'), ('sm', '_softmax', 'y'), ('out', '_matmul_out', 'A'))
@@ -343,6 +344,11 @@ class SparseAttention(OperatorBase):
             prefix = f'{name}/'
             op.build(config={k[len(prefix):]: v for k, v in config.items() if k.startswith(prefix)},
                      sample_inputs=part_inputs[name])
+        # the three parts share one index: a part built later must not have changed the block
+        # shape under a part built before it
+        for name, op, _ in self._parts():
+            prefix = f'{name}/'
+            check_shared_block_shapes(op._sparse_ctx._kernels, {k[len(prefix):] for k in config if k.startswith(prefix)})
         self.ready = True
 
     def set_sample_inputs(self, sample_inputs: List[torch.Tensor],

@@ -290,3 +290,31 @@ def test_dynamic_mode_never_fetches_nnz(gpu):
                                     transpose_B=True, mask=mask_np, dtype=np.float64)[0]
         assert_close(y, want, torch.float16, f'dynamic seed {seed}')
         assert idx.block_nnz == int(mask_np.reshape(N // 32, 32, K // 64, 64).any(axis=(1, 3)).sum())
+
+
+def test_build_rejects_kernels_that_disagree_on_a_shared_block_shape(gpu):
+    """The kernels of one operator that read the same compressed tensor share its index: a
+    configuration whose kernels want different block shapes for that tensor is refused (an
+    AssertionError, like any invalid combination), and a kernel of an earlier build that no
+    longer fits is switched off instead of running on a stale layout."""
+    _, A = randn((2, 128, 64), 71, torch.float16)
+    _, B = randn((2, 96, 64), 72, torch.float16)
+    mask = torch.from_numpy(ops.block_mask((128, 96), (32, 32), 0.5, seed=73)).to(gpu)
+    good = {k: dict(CFG32) for k in ('forward:C', 'backward:A', 'backward:B')}
+    bad = {k: dict(v) for k, v in good.items()}
+    bad['backward:B']['BLOCK_SIZE_M_VALUE'] = 16     # its tile of the sparse tensor becomes 32 x 16
+    op = sparta.nn.SparseBatchMatMul(C_mask=mask, transpose_A=False, transpose_B=True, compressed=True)
+    with pytest.raises(AssertionError, match='shares'):
+        op.build(bad, sample_inputs=[A.to(gpu), B.to(gpu)])
+    op.build(good, sample_inputs=[A.to(gpu), B.to(gpu)])
+    want = torch.matmul(A.to(gpu).float(), B.to(gpu).float().transpose(1, 2)) * mask
+    got = op.get_sparse_indexes('C').inverse(op(A.to(gpu), B.to(gpu)))
+    torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2)
+    # a forward-only rebuild with other blocks leaves the backward kernels of the first build behind
+    fwd16 = {'forward:C': {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': 16, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 16}}
+    op.build(fwd16, sample_inputs=[A.to(gpu), B.to(gpu)])
+    got = op.get_sparse_indexes('C').inverse(op(A.to(gpu), B.to(gpu)))
+    torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2)
+    Ar = A.to(gpu).requires_grad_(True)
+    with pytest.raises(ValueError, match='not compiled'):
+        op(Ar, B.to(gpu)).sum().backward()
