@@ -170,7 +170,8 @@ int spx_bcs_index_static(const uint8_t* mask, int H, int W, int BH, int BW,
  * axis 0: result [batch, H] = sum over W;  axis 1: result [batch, W] = sum
  * over H.  Every entry of `result` is written (zero where no block is live) and
  * the additions follow the index order, so the sums are bit-identical from run
- * to run (the reference adds with atomics).  idx as in spx_bcs_gather. */
+ * to run (the reference adds with atomics).  idx as in spx_bcs_gather.  `sparse`
+ * holds values of type `dtype` (f32, f16 or bf16); `result` is fp32 in every case. */
 int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
                 int nnz, int batch, int H, int W, int BH, int BW, int dtype, int axis,
                 int64_t sparse_batch_stride, spx_stream_t stream);

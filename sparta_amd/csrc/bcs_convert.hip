@@ -200,7 +200,7 @@ extern "C" int spx_bcs_sum(const void* sparse, void* result, const void* idx, in
                 "block size (%d,%d) must be a power of two in [4,256]", BH, BW);
     SPX_REQUIRE(H > 0 && W > 0 && H % BH == 0 && W % BW == 0, SPX_E_SHAPE, "bad shape");
     SPX_REQUIRE(axis == 0 || axis == 1, SPX_E_CONFIG, "axis must be 0 (sum over W) or 1 (sum over H)");
-    SPX_REQUIRE(dtype == SPX_F32, SPX_E_DTYPE, "spx_bcs_sum accumulates into an fp32 result; dtype must be f32");
+    SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(batch >= 0 && batch <= 65535 && nnz >= 0, SPX_E_SHAPE, "bad batch / nnz");
     if (batch == 0 || nnz == 0) return 0;
     SumParams p;
@@ -208,8 +208,13 @@ extern "C" int spx_bcs_sum(const void* sparse, void* result, const void* idx, in
     p.idx = idx; p.idx_kind = idx_kind; p.nnz = nnz;
     p.H = H; p.W = W; p.BH = BH; p.BW = BW; p.axis = axis;
     p.sparse_batch_stride = sparse_batch_stride;
-    hipLaunchKernelGGL(sum_kernel<float>, dim3(axis == 0 ? H / BH : W / BW, batch, 1), dim3(256), 0,
-                       reinterpret_cast<hipStream_t>(stream), p);
+    const dim3 grid(axis == 0 ? H / BH : W / BW, batch, 1);
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    switch (dtype) {   // the values are read in their own type; the result is fp32 in every case
+        case SPX_F32: hipLaunchKernelGGL(sum_kernel<float>, grid, dim3(256), 0, st, p); break;
+        case SPX_F16: hipLaunchKernelGGL(sum_kernel<_Float16>, grid, dim3(256), 0, st, p); break;
+        default: hipLaunchKernelGGL(sum_kernel<bf16_t>, grid, dim3(256), 0, st, p); break;
+    }
     SPX_LAUNCH_CHECK("sum_kernel");
     return 0;
 }

@@ -191,3 +191,20 @@ def test_convert_other_element_sizes(dtype, gpu):
                          else torch.int64).numpy()
     assert np.array_equal(raw, want)
     assert torch.equal(idx.inverse(got).cpu(), src)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_sum_of_16_bit_values(dtype, gpu):
+    """Row and column sums read 16-bit compressed values as they are (fp32 accumulate) for all
+    three index flavours."""
+    mask_np = ops.block_mask((256, 384), (16, 32), 0.7, seed=91)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    dense = (torch.randn((3, 256, 384), generator=torch.Generator().manual_seed(92)).to(gpu) * mask).to(dtype)
+    for bcsr, bcsc in ((True, False), (False, True), (True, True)):
+        idx = get_bcs_function(16, 32, bcsr, bcsc).build_indexes(mask)
+        vals = idx.convert(dense)
+        for axis in (-1, -2):
+            got = idx.sum(vals, axis=axis)
+            assert got.dtype == dtype
+            want = dense.float().sum(axis)
+            torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
