@@ -72,19 +72,18 @@ def check_shared_block_shapes(placeholders: Dict[str, KernelPlaceholder], built)
         kernel = placeholder.active_kernel()
         if kernel is None or not kernel.ready:
             continue
-        want = kernel.sparse_block_shape()
-        if want is None:
+        sized = kernel.sparse_block_shape()
+        if sized is None:
             continue
-        for port in kernel.ports.values():
-            # (a port no kernel has given a block shape yet holds no index either)
-            if not port.is_sparse or not port._block_H or (port._block_H, port._block_W) == tuple(want):
-                continue
-            if name in built:
-                raise AssertionError(
-                    f'kernel {name} takes {want[0]}x{want[1]} blocks of its sparse tensor, the kernels it shares '
-                    f'that tensor with take {port._block_H}x{port._block_W}')
-            kernel.ready = False
-            placeholder.ready = False
+        port, want = sized
+        if (port._block_H, port._block_W) == tuple(want):
+            continue
+        if name in built:
+            raise AssertionError(
+                f'kernel {name} takes {want[0]}x{want[1]} blocks of its sparse tensor, the kernels it shares '
+                f'that tensor with take {port._block_H}x{port._block_W}')
+        kernel.ready = False
+        placeholder.ready = False
 
 
 class SparseCtxBase(abc.ABC):

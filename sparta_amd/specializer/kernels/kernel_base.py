@@ -194,8 +194,9 @@ class KernelBase(abc.ABC):
         returns a one-line description instead of source code."""
         return f'// {type(self).__name__}: precompiled gfx950 kernel in libsparta_hip.so'
 
-    def sparse_block_shape(self) -> Optional[Tuple[int, int]]:
-        """(block_H, block_W) this kernel assumes for its sparse tensor, None if it has none."""
+    def sparse_block_shape(self) -> Optional[Tuple['PortConfig', Tuple[int, int]]]:
+        """(the port whose index this kernel reads, the (block_H, block_W) it assumes for it);
+        None for a kernel without a sparse tensor."""
         return None
 
     def compile(self, params: Dict[str, Any]):

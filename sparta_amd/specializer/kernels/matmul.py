@@ -128,7 +128,8 @@ class SparseMatMulKernel(KernelBase):
         return tuple(self.get_parameter(f'BLOCK_SIZE_{d}_VALUE') for d in 'MKN')
 
     def sparse_block_shape(self):
-        return self.get_parameter(self._sparse_block_H), self.get_parameter(self._sparse_block_W)
+        return (self.ports[self._sparse_port],
+                (self.get_parameter(self._sparse_block_H), self.get_parameter(self._sparse_block_W)))
 
     def blocks_per_grid(self):
         batch_size, M, K, N = self.get_shape()

@@ -47,7 +47,7 @@ class SparseSoftmaxKernel(KernelBase):
         return self.get_parameter('BLOCK_SIZE_H_VALUE'), self.get_parameter('BLOCK_SIZE_W_VALUE')
 
     def sparse_block_shape(self):
-        return self.get_block_shape()
+        return self.ports['y'], self.get_block_shape()
 
     def _launch_state(self):
         """Everything a launch closure needs, resolved once per update_func()."""
