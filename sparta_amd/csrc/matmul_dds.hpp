@@ -877,9 +877,9 @@ static int launch_dds_row(const DdsParams& p, int BM, int BN, int batch, hipStre
     return fail(SPX_E_CONFIG, "the block-row kernel takes 32 / 64-wide blocks");
 }
 
-// The pipelined kernels need both operands stored the same way round (both k-contiguous,
-// or A as [K, M] and B as [K, N]) and K a multiple of the stage depth (256 bytes of k per
-// row; 128 bytes for 64 x 64 blocks).  Returns 0 (no), 1 (k-contiguous) or 2.
+// The pipelined kernels need K to be a multiple of the stage depth (256 bytes of k per row;
+// 128 bytes for 64 x 64 blocks).  Returns 0 (no), 1 (both operands k-contiguous), 2 (A as
+// [K, M] and B as [K, N]), 3 or 4 (one of each).
 template <typename T>
 static int dds_pipe_ok(const DdsParams& p, int BM, int BN) {
     const int stage = (BM + BN == 128 ? 128 : 256) / (int)sizeof(T);
