@@ -928,27 +928,34 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
     // 2 / 3 / 4: tiles filled by LDS-direct loads - 128x128 with four wavefronts (two
     // workgroups per CU), 256x256 with eight wavefronts of 128x64, 256x256 with sixteen
     // wavefronts of 64x64 - for 16-bit types in either weight layout and fp32 with
-    // k-contiguous weights.  0 picks 4 when the problem has enough 256x256 tiles to fill
-    // the device (it moves half the bytes from L2 to the CUs, which is what bounds the
-    // 128x128 kernel), else 2; fp32 [E, in, out] weights take 1.  5 = 4 for the whole
-    // rounds of 256-row tiles plus 2 for the row tiles of a thinly filled last round
-    // (two launches, see moe_find_tile); 0 picks it in place of 4.
+    // k-contiguous weights.  256x256 tiles move half the bytes from L2 to the CUs, which is
+    // what bounds the 128x128 kernel.  5 = 4 for the whole rounds of 256-row tiles plus 2 for
+    // the row tiles of a thinly filled last round (two launches, see moe_find_tile).  0 picks
+    // between 5, 4 and 2 by the number of 256x256 tiles (below); fp32 [E, in, out] weights take 1.
     const bool direct_ok = p.w_kcontig || es == 2;
+    static int n_cu = 0;
+    if (n_cu == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n_cu = prop.multiProcessorCount;
+        if (n_cu <= 0) n_cu = 256;
+    }
     if (tile_cfg == 0) {
-        const int64_t big_tiles = (int64_t)((n_tok + 255) / 256) * ((out_dim + 255) / 256);
-        tile_cfg = !direct_ok ? 1 : (es == 2 && big_tiles >= 512 ? 5 : 2);
+        // 16-bit types: 256x256 tiles from 256 of them on (split launch, 5); from 128 on when
+        // all of them, the partly filled ones at the expert boundaries included, run in a
+        // single round (4: ten mid-size problems measured 10 - 25 % ahead of the 128x128
+        // tiles there, and behind them as soon as a second round starts); else 128x128
+        const int64_t row_tiles = (n_tok + 255) / 256, col_tiles = (out_dim + 255) / 256;
+        const int64_t big_tiles = row_tiles * col_tiles;
+        if (!direct_ok) tile_cfg = 1;
+        else if (es == 2 && big_tiles >= 256) tile_cfg = 5;
+        else if (es == 2 && big_tiles >= 128 && (row_tiles + n_exp) * col_tiles <= n_cu) tile_cfg = 4;
+        else tile_cfg = 2;
     }
     SPX_REQUIRE(tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg >= 2) {
         SPX_REQUIRE(direct_ok, SPX_E_CONFIG, "tile config %d takes fp32 weights in layout 1 only", tile_cfg);
         if (tile_cfg == 5) {
-            static int n_cu = 0;
-            if (n_cu == 0) {
-                int dev = 0;
-                hipDeviceProp_t prop;
-                if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n_cu = prop.multiProcessorCount;
-                if (n_cu <= 0) n_cu = 256;
-            }
             const int ntn = (out_dim + 255) / 256;
             p.round_rows = n_cu / ntn > 0 ? n_cu / ntn : 1;
         }
