@@ -127,7 +127,8 @@ int spx_bcs_index_scheduled(const uint8_t* mask, int H, int W, int BH, int BW,
  * W % 16 == 0 and at most 2048 words of 64 blocks per side) share one pair of launches, up to
  * four at a time - a model that rebuilds the masks of several layers per step otherwise pays
  * one pair of small dependent launches per layer; the other jobs are built one after the
- * other.  Results are those of separate calls.  No counterpart in the reference, which builds
+ * other.  Results are those of separate calls.  The workspaces of the jobs must not overlap
+ * (SPX_E_WORKSPACE otherwise).  No counterpart in the reference, which builds
  * one index per call (block_compressed.py:242-265). */
 typedef struct spx_bcs_index_job {
     const uint8_t* mask;
@@ -171,7 +172,8 @@ int spx_bcs_index_static(const uint8_t* mask, int H, int W, int BH, int BW,
  * over H.  Every entry of `result` is written (zero where no block is live) and
  * the additions follow the index order, so the sums are bit-identical from run
  * to run (the reference adds with atomics).  idx as in spx_bcs_gather.  `sparse`
- * holds values of type `dtype` (f32, f16 or bf16); `result` is fp32 in every case. */
+ * holds values of type `dtype` (f32, f16 or bf16); `result` is fp32 in every case.
+ * With nnz == 0 `sparse` and `idx` may be NULL and `result` is filled with zeros. */
 int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
                 int nnz, int batch, int H, int W, int BH, int BW, int dtype, int axis,
                 int64_t sparse_batch_stride, spx_stream_t stream);
@@ -191,7 +193,9 @@ int spx_bcs_sum(const void* sparse, void* result, const void* idx, int idx_kind,
  * compressed != 0: the sparse tensor is [batch, nnz*tileH*tileW] compressed
  * values with sparse_batch_stride elements between batches; otherwise it is
  * stored dense and the index only selects tiles (a dense DDS output must be
- * zero-filled by the caller; dead tiles are not written).
+ * zero-filled by the caller; dead tiles are not written).  A compressed sparse
+ * tensor with nnz_bound == 0 may be NULL (and idx with it) under every tile
+ * configuration, the persistent one (10) included: C is then bias (or zero).
  * ptr  row_ptr (BCSR) or col_ptr (BCSC); optional for DDS: row_ptr lets the launch
  *           group the live blocks of neighbouring block rows on one XCD (NULL = BCSR order).
  * idx / idx_kind  see spx_idx_kind.  nnz_bound / nnz_dev as in spx_bcs_gather

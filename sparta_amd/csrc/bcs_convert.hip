@@ -193,7 +193,8 @@ extern "C" int spx_bcs_sum(const void* sparse, void* result, const void* idx, in
                            int nnz, int batch, int H, int W, int BH, int BW, int dtype, int axis,
                            int64_t sparse_batch_stride, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(sparse && result, SPX_E_NULL, "sparse / result buffer is NULL");
+    SPX_REQUIRE(result, SPX_E_NULL, "result buffer is NULL");
+    SPX_REQUIRE(sparse || nnz == 0, SPX_E_NULL, "sparse buffer is NULL");
     SPX_REQUIRE(idx || nnz == 0, SPX_E_NULL, "index array is NULL");
     SPX_REQUIRE(idx_kind >= 0 && idx_kind <= 2, SPX_E_CONFIG, "unknown idx_kind %d", idx_kind);
     SPX_REQUIRE(valid_block_edge(BH) && valid_block_edge(BW), SPX_E_CONFIG,
@@ -202,7 +203,9 @@ extern "C" int spx_bcs_sum(const void* sparse, void* result, const void* idx, in
     SPX_REQUIRE(axis == 0 || axis == 1, SPX_E_CONFIG, "axis must be 0 (sum over W) or 1 (sum over H)");
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(batch >= 0 && batch <= 65535 && nnz >= 0, SPX_E_SHAPE, "bad batch / nnz");
-    if (batch == 0 || nnz == 0) return 0;
+    if (batch == 0) return 0;
+    // nnz == 0 is launched as well: every entry of `result` is written (zeros then), the
+    // kernel reads neither `sparse` nor `idx`
     SumParams p;
     p.sparse = sparse; p.result = reinterpret_cast<float*>(result);
     p.idx = idx; p.idx_kind = idx_kind; p.nnz = nnz;

@@ -840,6 +840,14 @@ extern "C" int spx_bcs_index_batch(const spx_bcs_index_job* jobs, int n_jobs, sp
         // one pair of launches, the others are built one by one
         const int last = first + INDEX_BATCH_MAX < n_jobs ? first + INDEX_BATCH_MAX : n_jobs;
         FastIndexJob prep[INDEX_BATCH_MAX];
+        // the builds of one group run in the same launches: their workspaces must be disjoint
+        for (int i = first; i < last; ++i)
+            for (int k = i + 1; k < last; ++k) {
+                const char* a = static_cast<const char*>(jobs[i].workspace);
+                const char* b = static_cast<const char*>(jobs[k].workspace);
+                SPX_REQUIRE(!a || !b || a + jobs[i].workspace_bytes <= b || b + jobs[k].workspace_bytes <= a,
+                            SPX_E_WORKSPACE, "jobs %d and %d share workspace memory", i, k);
+            }
         for (int i = first; i < last; ++i) {
             const spx_bcs_index_job& j = jobs[i];
             SPX_REQUIRE(!j.row_order || j.row_ptr, SPX_E_NULL, "row_order needs the BCSR index");

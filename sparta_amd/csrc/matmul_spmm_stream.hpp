@@ -160,7 +160,9 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN) + (p.s_kcontig ? ch * KC : ch * KC * BN)
                                      : (p.s_kcontig ? S + (int64_t)t.j * BN * p.s_ld + koff
                                                     : S + (int64_t)koff * p.s_ld + (int64_t)t.j * BN);
-        if (sh_active) sreg = *reinterpret_cast<const u32x4*>(live ? sblk + sh_toff : S);
+        // an idle step reads the first bytes of the dense operand: the sparse operand may be NULL
+        // when no block is live (every step of every tile is idle then)
+        if (sh_active) sreg = *reinterpret_cast<const u32x4*>(live ? sblk + sh_toff : D);
     };
 
     f32x4 acc[4][NT];

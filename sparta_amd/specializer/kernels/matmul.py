@@ -15,6 +15,7 @@ import torch
 from sparta_amd import _lib
 from sparta_amd.common.tuning import TunableItemCfg
 from sparta_amd.specializer.kernels.kernel_base import KernelBase, PortConfig
+from sparta_amd.specializer.kernels.operand_sizes import matmul_extent, check_matmul_operands
 
 # mode / transpose -> (sparse port, tile height param, tile width param, index format)
 _SPARSE_LAYOUT = {
@@ -180,10 +181,14 @@ class SparseMatMulKernel(KernelBase):
         # fully overwritten by the kernel.
         alloc = torch.zeros if (dds and not compressed) else torch.empty
         ptr_p, idx_p = _lib.dev_ptr(ptr), _lib.dev_ptr(idx)
+        # what this closure's kernel walks behind each pointer: a compressed operand laid out
+        # by another index (other block shape, other mask) is refused before the launch
+        extent = matmul_extent(self._mode, bool(compressed), batch_size, M, K, N, sparse_stride)
 
         def matmul_func(A: torch.Tensor, B: torch.Tensor, bias: torch.Tensor = None,
                         _keepalive=(indexes, ptr, idx, sched)):
             assert A.dtype == B.dtype, f'operand dtypes differ: {A.dtype} vs {B.dtype}'
+            check_matmul_operands(extent, A, B, bias, biased)
             C = alloc(C_shape, dtype=A.dtype, device=A.device)
             if bias is not None:
                 bias = bias.to(A.dtype).contiguous()

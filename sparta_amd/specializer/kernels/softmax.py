@@ -11,6 +11,7 @@ import torch
 from sparta_amd import _lib
 from sparta_amd.common.tuning import TunableItemCfg
 from sparta_amd.specializer.kernels.kernel_base import KernelBase, PortConfig
+from sparta_amd.specializer.kernels.operand_sizes import require_numel
 from sparta_amd.testing import sparse_softmax_forward_reference, sparse_softmax_backward_reference
 
 
@@ -98,7 +99,12 @@ class SparseSoftmaxForwardKernel(SparseSoftmaxKernel):
         row_ptr, idx = indexes.row_ptr, indexes._bcsr_buf
         lib = _lib.load()
 
+        numel = batch_size * stride
+        if mask is not None:
+            require_numel('spx_softmax_forward', 'mask', mask, stride)
+
         def softmax_forward_func(x: torch.Tensor, T: np.float32):
+            require_numel('spx_softmax_forward', 'x', x, numel)
             y = alloc(shape, dtype=x.dtype, device=x.device)
             if y.numel() == 0:  # no live block: nothing to compute
                 return y
@@ -138,7 +144,14 @@ class SparseSoftmaxBackwardKernel(SparseSoftmaxKernel):
         row_ptr, idx = indexes.row_ptr, indexes._bcsr_buf
         lib = _lib.load()
 
+        numel = batch_size * stride
+        if mask is not None:
+            require_numel('spx_softmax_backward', 'mask', mask, stride)
+
         def softmax_backward_func(grad_y: torch.Tensor, y: torch.Tensor, T: np.float32):
+            require_numel('spx_softmax_backward', 'grad_y', grad_y, numel)
+            require_numel('spx_softmax_backward', 'y', y, numel)
+            assert grad_y.dtype == y.dtype, f'operand dtypes differ: {grad_y.dtype} vs {y.dtype}'
             grad_x = alloc(shape, dtype=grad_y.dtype, device=grad_y.device)
             if grad_x.numel() == 0:
                 return grad_x

@@ -19,6 +19,7 @@ from sparta_amd.specializer.operators.sparse_matmul import SparseBatchMatMul
 from sparta_amd.specializer.operators.sparse_softmax import SparseSoftmax
 from sparta_amd.specializer.kernels import KernelBase, PortConfig
 from sparta_amd.specializer.funtional.sparse_ctx_base import check_shared_block_shapes
+from sparta_amd.specializer.kernels.operand_sizes import attention_extent, check_index_matches, require_numel
 
 # operator-level name -> (attribute, sparse port of that operator)
 _PARTS = (('qk', '_matmul_qk', 'C'), ('sm', '_softmax', 'y'), ('out', '_matmul_out', 'A'))
@@ -33,6 +34,9 @@ class _FusedAttentionFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, op: 'SparseAttention', query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
         q, k, v = query.detach(), key.detach(), value.detach()
+        # the index of this forward pass: the probabilities are laid out by it, and a mask update
+        # between forward and backward must not change what the backward kernels walk
+        ctx.indexes = op._sparse_port.indexes
         out, probs = op._fused_forward_train(q, k, v)
         ctx.save_for_backward(q, k, v, out, probs)
         ctx.op = op
@@ -46,16 +50,22 @@ class _FusedAttentionFunc(torch.autograd.Function):
         grad_out = grad_out.detach().contiguous()
         need_q, need_k, need_v = ctx.needs_input_grad[1:4]
         grad_q = grad_k = grad_v = None
-        if (need_k or need_v) and op._fused_backward_kv_supported(grad_out):
+        indexes = ctx.indexes
+        if (need_k or need_v) and op._fused_backward_kv_supported(grad_out, indexes):
             # two launches: the row side gives grad_q and the row constants, the column side
             # recomputes the score gradient from the probabilities for grad_k and grad_v
-            _, grad_q, row_dot = op._fused_backward_scores(grad_out, out, probs, k, v, store_scores=False)
-            grad_k, grad_v = op._fused_backward_kv(grad_out, q, v, probs, row_dot)
+            _, grad_q, row_dot = op._fused_backward_scores(grad_out, out, probs, k, v, store_scores=False,
+                                                           indexes=indexes)
+            grad_k, grad_v = op._fused_backward_kv(grad_out, q, v, probs, row_dot, indexes)
         else:
+            # the operator kernels are bound to the operator's current index
+            assert indexes is op._sparse_port.indexes, \
+                'the mask was updated between forward and backward of a SparseAttention call'
             if need_v:
                 grad_v = out_ctx.backward_B(grad_out, probs)
             if need_q or need_k:
-                grad_scores, grad_q, _ = op._fused_backward_scores(grad_out, out, probs, k, v, store_scores=need_k)
+                grad_scores, grad_q, _ = op._fused_backward_scores(grad_out, out, probs, k, v, store_scores=need_k,
+                                                                   indexes=indexes)
                 if need_k:
                     grad_k = qk_ctx.backward_B(grad_scores, q)
         return None, grad_q if need_q else None, grad_k if need_k else None, grad_v if need_v else None
@@ -69,6 +79,9 @@ class _RecomputeAttentionFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, op: 'SparseAttention', query: torch.Tensor, key: torch.Tensor, value: torch.Tensor):
         q, k, v = query.detach().contiguous(), key.detach().contiguous(), value.detach().contiguous()
+        # the index of this forward pass: the log-sum-exp belongs to its set of live blocks, so
+        # the backward kernels walk the same index even if the mask has been updated since
+        ctx.indexes = op._sparse_port.indexes
         out, row_lse = op._fused_forward_lse(q, k, v)
         ctx.save_for_backward(q, k, v, out, row_lse)
         ctx.op = op
@@ -80,10 +93,10 @@ class _RecomputeAttentionFunc(torch.autograd.Function):
         op = ctx.op
         grad_out = grad_out.detach().contiguous()
         need_q, need_k, need_v = ctx.needs_input_grad[1:4]
-        grad_q, row_dot = op._recompute_backward_q(grad_out, out, q, k, v, row_lse)
+        grad_q, row_dot = op._recompute_backward_q(grad_out, out, q, k, v, row_lse, ctx.indexes)
         grad_k = grad_v = None
         if need_k or need_v:
-            grad_k, grad_v = op._recompute_backward_kv(grad_out, q, k, v, row_lse, row_dot)
+            grad_k, grad_v = op._recompute_backward_kv(grad_out, q, k, v, row_lse, row_dot, ctx.indexes)
         return None, grad_q if need_q else None, grad_k if need_k else None, grad_v if need_v else None
 
 
@@ -117,6 +130,7 @@ class SparseAttention(OperatorBase):
         self._fused_mask_key = None   # index object the cached element mask belongs to
         self._fused_mask = None
         self._inv_temperature = 1.0
+        self._warned_unfused = False
         self.ready = False
 
     def _parts(self):
@@ -132,6 +146,14 @@ class SparseAttention(OperatorBase):
                 return _RecomputeAttentionFunc.apply(self, query, key, value)
             if self._fused_train_supported(query):
                 return _FusedAttentionFunc.apply(self, query, key, value)
+        if self.ready and self._fused and not self._warned_unfused and torch.is_grad_enabled() and (
+                query.requires_grad or key.requires_grad or value.requires_grad):
+            self._warned_unfused = True
+            indexes = self._sparse_port.indexes
+            warnings.warn(
+                f'SparseAttention: no fused training kernel for {query.dtype} inputs of head dim {query.shape[-1]} '
+                f'with {indexes.block_H}x{indexes.block_W} score blocks (16-bit types, head dims 64 / 128 and '
+                'blocks of 32 / 64 / 128 are covered); this step runs as three forward and six backward launches')
         scores = self._matmul_qk.forward(query, key)
         probs = self._softmax.forward(scores)
         return self._matmul_out.forward(probs, value)
@@ -156,12 +178,26 @@ class SparseAttention(OperatorBase):
                 and getattr(indexes, 'col_ptr', None) is not None and getattr(indexes, 'row_ptr', None) is not None
                 and self._element_mask() is None)
 
+    def _check_operands(self, what: str, indexes, batch: int, E: int, q_like=(), kv_like=(), rows=(),
+                        probs=(), nnz=None):
+        """Sizes of the tensors behind the pointers of one fused-kernel call, against what the
+        kernel walks for `batch` entries of the index's mask; AssertionError before any launch."""
+        check_index_matches(what, indexes, self._Nt, self._Ns)
+        want = attention_extent(batch, self._Nt, self._Ns, E, indexes.block_nnz if nnz is None else nnz,
+                                indexes.block_H, indexes.block_W)
+        for group, numel in ((q_like, want.q), (kv_like, want.kv), (rows, want.rows), (probs, want.probs)):
+            for name, tensor in group:
+                if tensor is not None:
+                    require_numel(what, name, tensor, numel)
+
     def _fused_forward_lse(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
         """(output, log-sum-exp per query) from spx_attention_forward_lse."""
         indexes = self._sparse_port.indexes
         batch, _, E = q.shape
         out = torch.empty_like(q)
         row_lse = torch.empty((batch, self._Nt), dtype=torch.float32, device=q.device)
+        self._check_operands('spx_attention_forward_lse', indexes, batch, E, q_like=[('q', q)],
+                             kv_like=[('k', k), ('v', v)], nnz=0)
         rc = _lib.load().spx_attention_forward_lse(
             _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
             _lib.dev_ptr(row_lse), _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), None,
@@ -170,12 +206,15 @@ class SparseAttention(OperatorBase):
         _lib.check(rc, 'spx_attention_forward_lse')
         return out, row_lse
 
-    def _recompute_backward_q(self, grad_out, out, q, k, v, row_lse):
+    def _recompute_backward_q(self, grad_out, out, q, k, v, row_lse, indexes=None):
         """(query gradient, row constants) from spx_attention_backward_q."""
-        indexes = self._sparse_port.indexes
+        indexes = self._sparse_port.indexes if indexes is None else indexes
         batch, _, E = grad_out.shape
         grad_q = torch.empty_like(q)
         row_dot = torch.empty((batch, self._Nt), dtype=torch.float32, device=q.device)
+        self._check_operands('spx_attention_backward_q', indexes, batch, E,
+                             q_like=[('grad_out', grad_out), ('out', out), ('q', q)],
+                             kv_like=[('k', k), ('v', v)], rows=[('row_lse', row_lse)], nnz=0)
         rc = _lib.load().spx_attention_backward_q(
             _lib.dtype_code(q.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(out), _lib.dev_ptr(q), _lib.dev_ptr(k),
             _lib.dev_ptr(v), _lib.dev_ptr(row_lse), _lib.dev_ptr(grad_q), _lib.dev_ptr(row_dot),
@@ -184,14 +223,17 @@ class SparseAttention(OperatorBase):
         _lib.check(rc, 'spx_attention_backward_q')
         return grad_q, row_dot
 
-    def _recompute_backward_kv(self, grad_out, q, k, v, row_lse, row_dot):
+    def _recompute_backward_kv(self, grad_out, q, k, v, row_lse, row_dot, indexes=None):
         """(key gradient, value gradient) from spx_attention_backward_kv_recompute."""
-        indexes = self._sparse_port.indexes
+        indexes = self._sparse_port.indexes if indexes is None else indexes
         batch, _, E = grad_out.shape
         grad_k = torch.empty_like(k)
         grad_v = torch.empty_like(v)
         idx = indexes._bcsc_buf
         kind = _lib.IDX_BCSC_I64 if idx.dtype == torch.int64 else _lib.IDX_BCSC_I32
+        self._check_operands('spx_attention_backward_kv_recompute', indexes, batch, E,
+                             q_like=[('grad_out', grad_out), ('q', q)], kv_like=[('k', k), ('v', v)],
+                             rows=[('row_lse', row_lse), ('row_dot', row_dot)], nnz=0)
         rc = _lib.load().spx_attention_backward_kv_recompute(
             _lib.dtype_code(q.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v),
             _lib.dev_ptr(row_lse), _lib.dev_ptr(row_dot), _lib.dev_ptr(grad_k), _lib.dev_ptr(grad_v),
@@ -218,6 +260,8 @@ class SparseAttention(OperatorBase):
         q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
         out = torch.empty_like(q)
         probs = torch.empty((batch, indexes.block_nnz * indexes.block_H * indexes.block_W), dtype=q.dtype, device=q.device)
+        self._check_operands('spx_attention_forward_train', indexes, batch, E, q_like=[('q', q)],
+                             kv_like=[('k', k), ('v', v)])
         rc = _lib.load().spx_attention_forward_train(
             _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
             _lib.dev_ptr(probs), probs.shape[1], _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf),
@@ -226,15 +270,18 @@ class SparseAttention(OperatorBase):
         _lib.check(rc, 'spx_attention_forward_train')
         return out, probs
 
-    def _fused_backward_scores(self, grad_out, out, probs, key, value, store_scores=True):
+    def _fused_backward_scores(self, grad_out, out, probs, key, value, store_scores=True, indexes=None):
         """(compressed score gradient or None, query gradient, row constants) from
         spx_attention_backward_scores."""
-        indexes = self._sparse_port.indexes
+        indexes = self._sparse_port.indexes if indexes is None else indexes
         batch, _, E = grad_out.shape
         k, v = key.contiguous(), value.contiguous()
         grad_scores = torch.empty_like(probs) if store_scores else None
         grad_q = torch.empty_like(grad_out)
         row_dot = torch.empty((batch, self._Nt), dtype=torch.float32, device=grad_out.device)
+        self._check_operands('spx_attention_backward_scores', indexes, batch, E,
+                             q_like=[('grad_out', grad_out), ('out', out)], kv_like=[('k', k), ('v', v)],
+                             probs=[('probs', probs)])
         rc = _lib.load().spx_attention_backward_scores(
             _lib.dtype_code(grad_out.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(out), _lib.dev_ptr(probs),
             _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(grad_scores), _lib.dev_ptr(grad_q), _lib.dev_ptr(row_dot),
@@ -244,23 +291,26 @@ class SparseAttention(OperatorBase):
         _lib.check(rc, 'spx_attention_backward_scores')
         return grad_scores, grad_q, row_dot
 
-    def _fused_backward_kv_supported(self, grad_out: torch.Tensor) -> bool:
+    def _fused_backward_kv_supported(self, grad_out: torch.Tensor, indexes=None) -> bool:
         """The column-side kernel needs the BCSC index next to the BCSR one (the probabilities
         are stored in BCSR order) and the block shapes it covers."""
-        indexes = self._sparse_port.indexes
+        indexes = self._sparse_port.indexes if indexes is None else indexes
         BH, BW, E = indexes.block_H, indexes.block_W, grad_out.shape[-1]
         return (getattr(indexes, 'col_ptr', None) is not None and getattr(indexes, 'row_ptr', None) is not None
                 and BH in (32, 64, 128) and BW in (32, 64, 128) and E in (64, 128) and BH * E >= 32 * BW)
 
-    def _fused_backward_kv(self, grad_out, query, value, probs, row_dot):
+    def _fused_backward_kv(self, grad_out, query, value, probs, row_dot, indexes=None):
         """(key gradient, value gradient) from spx_attention_backward_kv."""
-        indexes = self._sparse_port.indexes
+        indexes = self._sparse_port.indexes if indexes is None else indexes
         batch, _, E = grad_out.shape
         q, v = query.contiguous(), value.contiguous()
         grad_k = torch.empty_like(v)
         grad_v = torch.empty_like(v)
         idx = indexes._bcsc_buf
         kind = _lib.IDX_BCSC_I64 if idx.dtype == torch.int64 else _lib.IDX_BCSC_I32
+        self._check_operands('spx_attention_backward_kv', indexes, batch, E,
+                             q_like=[('grad_out', grad_out), ('q', q)], kv_like=[('v', v)],
+                             rows=[('row_dot', row_dot)], probs=[('probs', probs)])
         rc = _lib.load().spx_attention_backward_kv(
             _lib.dtype_code(grad_out.dtype), _lib.dev_ptr(grad_out), _lib.dev_ptr(q), _lib.dev_ptr(v),
             _lib.dev_ptr(probs), _lib.dev_ptr(row_dot), _lib.dev_ptr(grad_k), _lib.dev_ptr(grad_v), probs.shape[1],
@@ -284,6 +334,8 @@ class SparseAttention(OperatorBase):
         batch = int(np.prod(lead)) if len(lead) else 1
         q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
         out = torch.empty_like(q)
+        self._check_operands('spx_attention_forward', indexes, batch, E, q_like=[('q', q)],
+                             kv_like=[('k', k), ('v', v)], nnz=0)
         rc = _lib.load().spx_attention_forward(
             _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
             _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(self._fused_mask),

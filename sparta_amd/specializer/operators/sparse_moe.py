@@ -38,10 +38,13 @@ class DynamicSparseMoE(torch.nn.Module):
         self.sparse_index = torch.zeros(0, **i32)  # token permutation, sized at first call
 
     def forward(self, tokens: torch.Tensor, exp_ids: torch.Tensor):
-        n_tok = tokens.shape[0]
-        assert tokens.shape[1] == self.in_hidden, \
+        assert tokens.dim() == 2 and tokens.shape[1] == self.in_hidden, \
             f'expected tokens of width {self.in_hidden}, got {tuple(tokens.shape)}'
-        assert exp_ids.shape[0] == n_tok, 'one expert id per token is required'
+        n_tok = tokens.shape[0]
+        assert exp_ids.numel() == n_tok, 'one expert id per token is required'
+        # the kernel walks num_exps matrices of in_hidden x out_hidden behind the weight pointer
+        assert self.weight.numel() == self.num_exps * self.in_hidden * self.out_hidden, \
+            f'the weight has shape {tuple(self.weight.shape)}, expected ({self.num_exps}, {self.in_hidden}, {self.out_hidden})'
         if exp_ids.dtype != torch.int32:
             exp_ids = exp_ids.to(torch.int32)
         if self.sparse_index.numel() < n_tok:

@@ -308,6 +308,10 @@ class BCSFunctionContext(TeSAFunctionContext):
         """axis 0: [..., H] sums over W; axis 1: [..., W] sums over H (fp32 accumulate)."""
         lead = tuple(sparse_val.shape[:-1])
         batch = int(np.prod(lead)) if lead else 1
+        # values kept at index capacity (dynamic masks) are longer than the live blocks
+        stride = sparse_val.shape[-1]
+        assert stride >= block_nnz * self._block_size, \
+            f'expected at least (..., {block_nnz * self._block_size}) values, got {tuple(sparse_val.shape)}'
         vals = sparse_val.contiguous()
         if vals.dtype not in (torch.float32, torch.float16, torch.bfloat16):
             vals = vals.to(torch.float32)
@@ -317,7 +321,7 @@ class BCSFunctionContext(TeSAFunctionContext):
             rc = _lib.load().spx_bcs_sum(
                 _lib.dev_ptr(vals), _lib.dev_ptr(result), _lib.dev_ptr(index), idx_kind, block_nnz,
                 batch, H, W, self._block_H, self._block_W, _lib.dtype_code(vals.dtype), axis,
-                block_nnz * self._block_size, _lib.current_stream(vals.device))
+                stride, _lib.current_stream(vals.device))
         _lib.check(rc, 'spx_bcs_sum')
         return result.to(sparse_val.dtype).reshape(lead + (n_out,))
 

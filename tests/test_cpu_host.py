@@ -122,6 +122,10 @@ def test_host_validation_of_recompute_batch_and_moe_entry_points():
     assert lib.spx_bcs_index_batch(jobs, 2, None) == _lib.E_CONFIG
     jobs[0].H, jobs[0].W, jobs[0].BH, jobs[0].BW = 64, 60, 32, 32
     assert lib.spx_bcs_index_batch(jobs, 1, None) == _lib.E_SHAPE
+    # two jobs of one group must not share workspace memory (they run in the same launches)
+    jobs[0].workspace, jobs[0].workspace_bytes = 4096, 1024
+    jobs[1].workspace, jobs[1].workspace_bytes = 4096 + 512, 1024
+    assert lib.spx_bcs_index_batch(jobs, 2, None) == _lib.E_WORKSPACE and 'share workspace' in _lib.last_error()
     # index build on the library's own scratch: limits are checked before the array is looked up
     assert lib.spx_bcs_index_static_max_bytes() == 1 << 20
     rc = lib.spx_bcs_index_static(None, 64, 64, 3, 32, None, None, None, None, 0, None, 0, None)

@@ -76,6 +76,55 @@ def test_c3_attention_all_96_heads(gpu):
     assert_close(piped[heads], want, torch.float16, 'C3 three-operator pipeline, sampled heads')
 
 
+def _attention_train_config(bh, bw):
+    mm = lambda m, k, n: {'_impl': 'sparta', 'BLOCK_SIZE_M_VALUE': m, 'BLOCK_SIZE_K_VALUE': k, 'BLOCK_SIZE_N_VALUE': n}
+    sm = {'_impl': 'sparta', 'BLOCK_SIZE_H_VALUE': bh, 'BLOCK_SIZE_W_VALUE': bw, 'ROW_TILE_VALUE': 4}
+    return {'qk/forward:C': mm(bh, 32, bw), 'qk/backward:A': mm(bh, bw, 32), 'qk/backward:B': mm(bw, bh, 32),
+            'sm/forward:y': dict(sm), 'sm/backward:x': dict(sm),
+            'out/forward:C': mm(bh, bw, 32), 'out/backward:A': mm(bh, 32, bw), 'out/backward:B': mm(bw, bh, 32)}
+
+
+@pytest.mark.parametrize('bh,bw', [(32, 32), (32, 64)])
+def test_c3_training_step_with_other_block_shapes(bh, bw, gpu):
+    """A well-formed SparseAttention training step at the full C3 size (96 heads x 4096 x 64
+    fp16, the C3 mask) with score blocks other than 64x64, through its three paths - the
+    kernels that recompute the probabilities, the kernels that store them, and the three
+    operators with their six backward kernels - each against dense fp32 autograd on a sample of
+    heads.  Every kernel of the step agrees on one block shape (build() refuses anything else)
+    and every closure checks the size of its operands before it launches."""
+    BH, N, E = 96, 4096, 64
+    mask_np = np.kron(attention_grid(), np.ones((64, 64), dtype=np.uint8))
+    mask = torch.from_numpy(mask_np).to(gpu)
+    g = torch.Generator().manual_seed(2023)
+    q, k, v, go = (torch.randn((BH, N, E), generator=g).half().to(gpu) for _ in range(4))
+    heads = [0, 41, 95]
+    # dense fp32 autograd on the sampled heads
+    ref = [t[heads].float().requires_grad_(True) for t in (q, k, v)]
+    scores = ref[0] @ ref[1].transpose(1, 2) / math.sqrt(E)
+    scores = scores.masked_fill(mask == 0, float('-inf'))
+    ref_out = torch.softmax(scores, -1) @ ref[2]
+    ref_out.backward(go[heads].float())
+    want = [ref_out.detach()] + [t.grad for t in ref]
+    del scores
+
+    for path, recompute, fused in (('recompute', True, True), ('stored probabilities', False, True),
+                                   ('three operators', True, False)):
+        print(f'C3 training step, blocks {bh}x{bw}, path: {path}', flush=True)
+        att = sparta.nn.SparseAttention(mask=mask, recompute=recompute, fused=fused)
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        att.build(_attention_train_config(bh, bw), sample_inputs=[t.detach() for t in leaves])
+        idx = att._sparse_port.indexes
+        assert (idx.block_H, idx.block_W) == (bh, bw)
+        assert idx.block_nnz * bh * bw == int(attention_grid().sum()) * 64 * 64
+        out = att(*leaves)
+        out.backward(go)
+        torch.cuda.synchronize()
+        got = [out.detach()[heads].float()] + [t.grad[heads].float() for t in leaves]
+        for name, a, b in zip(('out', 'grad_q', 'grad_k', 'grad_v'), got, want):
+            torch.testing.assert_close(a, b, rtol=2e-2, atol=2e-2, msg=lambda m: f'{path}, {name}: {m}')
+        del att, leaves, out, got
+
+
 # ------------------------------------------------------------------------------- C4
 def topk_block_mask(shape, seed, block=(32, 64), keep_frac=0.1):
     """Keeps the ceil(10%) blocks with the largest |score| (score ~ N(0,1), seeded)."""

@@ -253,6 +253,27 @@ def test_matmul_empty_mask_gives_zero_or_bias(gpu):
     assert_close(C, np.broadcast_to(bias_np[:, None, :], (1, 128, 64)), torch.float16)
 
 
+@pytest.mark.parametrize('tile_cfg', [0, 10])
+def test_matmul_empty_mask_through_the_persistent_kernel(tile_cfg, gpu):
+    """A fully pruned compressed weight at a shape that the dispatcher sends to the persistent
+    kernel (tile config 10: batch 1, N / BN >= 128, M >= 4096, K / BK >= 32): the compressed
+    operand is an empty tensor (a NULL pointer), every step of every tile is idle, and the
+    output equals the bias."""
+    M = K = N = 4096
+    _, a = randn((1, M, K), 1, torch.float16)
+    bias_np, bias = randn((1, N), 3, torch.float16)
+    mask = torch.zeros((N, K), dtype=torch.uint8, device=gpu)
+    kernel = SparTASparseMatMulKernel(mode='dsd', biased=True, transpose_A=False, transpose_B=True, compressed=True)
+    kernel.ports['B'].set_mask(mask)
+    kernel.set_shape(1, M, K, N)
+    kernel.compile({'BLOCK_SIZE_M_VALUE': 32, 'BLOCK_SIZE_K_VALUE': 32, 'BLOCK_SIZE_N_VALUE': 32, 'TILE_CFG': tile_cfg})
+    w = kernel.ports['B'].indexes.convert(torch.zeros((1, N, K), dtype=torch.float16, device=gpu))
+    assert w.shape == (1, 0)
+    C = kernel(a.to(gpu), w, bias.to(gpu))
+    want = torch.from_numpy(bias_np).to(gpu).half().expand(M, N)
+    assert torch.equal(C[0], want)
+
+
 def test_matmul_ragged_m(gpu):
     """M that is not a multiple of the workgroup tile (dense dimension of 'dsd')."""
     for M in (16, 48, 200):

@@ -208,3 +208,32 @@ def test_sum_of_16_bit_values(dtype, gpu):
             assert got.dtype == dtype
             want = dense.float().sum(axis)
             torch.testing.assert_close(got.float(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
+
+
+@pytest.mark.parametrize('at_capacity', [False, True])
+def test_sum_over_an_empty_index_is_zero(at_capacity, gpu):
+    """No live block: every entry of the result is written as zero, whether the values are an
+    empty tensor (static storage) or a buffer kept at index capacity (dynamic masks)."""
+    mask = torch.zeros((128, 192), dtype=torch.uint8, device=gpu)
+    dense = torch.randn((2, 128, 192), generator=torch.Generator().manual_seed(5)).to(gpu).half()
+    for bcsr, bcsc in ((True, False), (False, True), (True, True)):
+        idx = get_bcs_function(32, 32, bcsr, bcsc).build_indexes(mask)
+        vals = idx.convert(dense, at_capacity=at_capacity)
+        assert vals.shape == (2, (idx.capacity if at_capacity else 0) * 32 * 32)
+        for axis, n_out in ((-1, 128), (-2, 192)):
+            got = idx.sum(vals, axis=axis)
+            assert got.shape == (2, n_out)
+            assert torch.count_nonzero(got).item() == 0
+
+
+def test_sum_of_values_kept_at_capacity(gpu):
+    """Values stored at index capacity (dynamic masks) have a longer batch stride than the live
+    blocks; the sums must follow the stride of the tensor they are given."""
+    mask_np = ops.block_mask((128, 192), (32, 32), 0.6, seed=17)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    dense = (torch.randn((3, 128, 192), generator=torch.Generator().manual_seed(18)).to(gpu) * mask).half()
+    idx = get_bcs_function(32, 32, True, True).build_indexes(mask)
+    vals = idx.convert(dense, at_capacity=True)
+    assert vals.shape[-1] == idx.capacity * 32 * 32 > idx.block_nnz * 32 * 32
+    for axis in (-1, -2):
+        assert torch.equal(idx.sum(vals, axis=axis), idx.sum(idx.convert(dense), axis=axis))
