@@ -73,10 +73,13 @@ def _tuner_class(algo: str):
 def tune_sparse_module(module: OperatorBase, name: str, sample_inputs: List[torch.Tensor],
                        sample_grads: Optional[List[torch.Tensor]] = None, algo: str = 'grid',
                        max_trials: int = sys.maxsize, backward_weight: float = 0,
-                       debug_func: Optional[Callable[[int, Dict[Any, Any]], float]] = None):
+                       debug_func: Optional[Callable[[int, Dict[Any, Any]], float]] = None,
+                       refine_tiles: bool = False):
     """Tune one sparse operator and build it with the best configuration found.
     Returns that configuration ({kernel: {'_impl': ..., PARAM: ...}}), or None if
-    every trial failed or `debug_func` replaced the measurement."""
+    every trial failed or `debug_func` replaced the measurement.  With `refine_tiles`
+    every kernel of the best configuration then tries each gfx950 tile configuration
+    with its block sizes kept (see refine_tile_configs)."""
     tuner_cls = _tuner_class(algo)
     with_backward = backward_weight > 0
     module.set_sample_inputs(sample_inputs, sample_grads)
@@ -143,9 +146,46 @@ def tune_sparse_module(module: OperatorBase, name: str, sample_inputs: List[torc
         _logger.warning(f'[{name}] All trials failed.')
         return None
     best_config = best_lower[str(upper_tuner.best_config)]
+    if refine_tiles:
+        best_config = refine_tile_configs(module, name, best_config, with_backward)
     _logger.info(f'[{name}] Best config:\n{best_config}')
     module.build(best_config, sample_inputs)
     return best_config
+
+
+def refine_tile_configs(module: OperatorBase, name: str, config: Dict[str, Dict[str, Any]],
+                        with_backward: bool = False) -> Dict[str, Dict[str, Any]]:
+    """Second stage of a search that keeps the block sizes of `config`: every kernel that has
+    a table of gfx950 tile configurations is built and timed with each of its entries (the
+    costs add to those of the block-size search instead of multiplying them).  Returns
+    `config` with 'TILE_CFG' set where an entry other than the library's own choice (0) was
+    the fastest.  Needs the sample inputs of `module` to be set (tune_sparse_module does)."""
+    from sparta_amd import _lib
+    refined = {kernel_name: dict(params) for kernel_name, params in config.items() if params is not None}
+    for kernel_name, placeholder in module.get_kernel_placeholders(with_backward).items():
+        params = refined.get(kernel_name)
+        if params is None:
+            continue
+        placeholder.select_impl(params['_impl'])
+        op = placeholder.active_kernel()._tile_op()
+        if op is None:
+            continue
+        best_id, best_latency = 0, math.inf
+        for tile in _lib.tile_configs(op):
+            trial = {k: v for k, v in params.items() if k != 'TILE_CFG'}
+            trial['TILE_CFG'] = tile['id']
+            try:
+                placeholder.build(trial)
+                latency = placeholder.test()
+            except AssertionError:
+                latency = math.inf
+            _logger.info(f'[{name}][Kernel: {kernel_name}] tile config {tile["id"]} ({tile["name"]}) => {latency} ms')
+            if latency < best_latency:
+                best_id, best_latency = tile['id'], latency
+        params.pop('TILE_CFG', None)
+        if best_id:
+            params['TILE_CFG'] = best_id
+    return refined
 
 
 def iter_sparse_modules(module: torch.nn.Module, module_name: str,
@@ -157,6 +197,20 @@ def iter_sparse_modules(module: torch.nn.Module, module_name: str,
         return
     for child_name, child in module.named_children():
         iter_sparse_modules(child, f'{module_name}/{child_name}', func)
+
+
+def iter_tile_modules(module: torch.nn.Module, module_name: str,
+                      func: Callable[[torch.nn.Module, str], None]):
+    """Apply `func(op, name)` to every module below `module` that chooses a tile configuration
+    for a kernel of its own through `tune_tile_config` / `set_tile_config` (the fused
+    attention kernel, the gathered MoE product); such a module is a leaf of the walk."""
+    if hasattr(module, 'tune_tile_config'):
+        func(module, module_name)
+        return
+    if isinstance(module, OperatorBase):
+        return
+    for child_name, child in module.named_children():
+        iter_tile_modules(child, f'{module_name}/{child_name}', func)
 
 
 def get_input_hook(input_dict: Dict[str, List], module_name: str):
@@ -180,12 +234,13 @@ def _capture_samples(module: torch.nn.Module, sample_inputs, sample_grads, with_
     grads = {'root': sample_grads}
     handles = []
 
-    def register(op: OperatorBase, name: str):
+    def register(op: torch.nn.Module, name: str):
         handles.append(op.register_forward_hook(get_input_hook(inputs, name)))
-        if with_backward:
+        if with_backward and isinstance(op, OperatorBase):
             handles.append(op.register_full_backward_hook(get_grad_hook(grads, name)))
 
     iter_sparse_modules(module, 'root', register)
+    iter_tile_modules(module, 'root', lambda op, name: None if isinstance(op, OperatorBase) else register(op, name))
     try:
         with warnings.catch_warnings():
             warnings.simplefilter('ignore')
@@ -210,7 +265,7 @@ def tune_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Tens
                          sample_grads: Optional[List[torch.Tensor]] = None, algo: str = 'grid',
                          max_trials: int = sys.maxsize, backward_weight: float = 0,
                          verbose: bool = False, debug_func: Optional[Callable] = None,
-                         tile_configs: bool = False):
+                         tile_configs=False):
     """Find, tune and build every sparse operator inside `module`.
 
     Args:
@@ -222,9 +277,13 @@ def tune_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Tens
         backward_weight: weight of backward latencies; 0 tunes forward kernels only.
         verbose: log every trial.
         debug_func: replaces build + measurement of a trial (for tests).
-        tile_configs: also search the gfx950 tile configurations of the matmul
-            kernels (parameter TILE_CFG); off by default, which leaves exactly the
-            reference's search space.
+        tile_configs: also search the gfx950 tile configurations (parameter TILE_CFG of
+            the matmul and softmax kernels, and the kernels that SparseAttention and
+            DynamicSparseMoE launch themselves).  False (default) leaves exactly the
+            reference's search space and trial counts.  True adds TILE_CFG to the lower
+            space of every kernel (a joint search: the trial budget is spent on block
+            sizes x tile configurations).  'refine' searches the reference's space first
+            and then tries every tile configuration with the best block sizes kept.
 
     Returns:
         {operator name: best config}; names are 'root' or 'root/child/...'.
@@ -234,8 +293,7 @@ def tune_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Tens
     def set_tile_search(op: OperatorBase, name: str):
         for placeholder in op.get_kernel_placeholders(backward=True).values():
             for kernel in placeholder.possible_kernels.values():
-                if hasattr(kernel, 'enable_tile_search'):
-                    kernel.enable_tile_search(tile_configs)
+                kernel.enable_tile_search(tile_configs is True)
 
     iter_sparse_modules(module, 'root', set_tile_search)
     _logger.setLevel(logging.DEBUG if verbose else logging.WARNING)
@@ -244,9 +302,22 @@ def tune_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Tens
     def tune_one(op: OperatorBase, name: str):
         best_configs[name] = tune_sparse_module(
             module=op, name=name, sample_inputs=inputs[name], sample_grads=grads.get(name),
-            algo=algo, max_trials=max_trials, backward_weight=backward_weight, debug_func=debug_func)
+            algo=algo, max_trials=max_trials, backward_weight=backward_weight, debug_func=debug_func,
+            refine_tiles=tile_configs == 'refine')
 
     iter_sparse_modules(module, 'root', tune_one)
+
+    def tune_own_kernel(op: torch.nn.Module, name: str):
+        # kernels that a module launches itself, outside the kernel placeholders
+        if isinstance(op, OperatorBase) and best_configs.get(name) is None:
+            return
+        own = op.tune_tile_config(inputs[name])
+        if own:
+            best_configs[name] = {**(best_configs.get(name) or {}), **own}
+        _logger.info(f'[{name}] tile configuration of its own kernel: {own}')
+
+    if tile_configs and debug_func is None:
+        iter_tile_modules(module, 'root', tune_own_kernel)
     return best_configs
 
 
@@ -256,3 +327,5 @@ def build_combined_module(module: torch.nn.Module, sample_inputs: List[torch.Ten
     (as returned by tune)."""
     inputs, _ = _capture_samples(module, sample_inputs, None, False)
     iter_sparse_modules(module, 'root', lambda op, name: op.build(configs[name], sample_inputs=inputs[name]))
+    iter_tile_modules(module, 'root', lambda op, name: None if isinstance(op, OperatorBase) or name not in configs
+                      else op.set_tile_config(configs[name]))

@@ -199,8 +199,34 @@ class KernelBase(abc.ABC):
         None for a kernel without a sparse tensor."""
         return None
 
+    # ---- gfx950 tile configurations ----------------------------------------------------
+    def _tile_op(self) -> Optional[int]:
+        """Which tile-config table of the library (spx_tile_cfg_info's `op`) lists this kernel's
+        variants; None for a kernel without a TILE_CFG parameter."""
+        return None
+
+    def enable_tile_search(self, enabled: bool = True):
+        """Add (or remove) the gfx950 tile configuration to the tunable parameters.
+        Off by default so that the search space equals the reference's; tune(...,
+        tile_configs=True) switches it on.  A configuration that does not fit the operand
+        layout, block shape or dtype is rejected by the library with an AssertionError,
+        which the tuner counts as an infinitely slow trial."""
+        op = self._tile_op()
+        if op is None:
+            return
+        from sparta_amd import _lib
+        param = self._parameters['TILE_CFG']
+        if enabled:
+            param.is_tunable = True
+            param.search_space = TunableItemCfg('choice', [cfg['id'] for cfg in _lib.tile_configs(op)])
+        else:
+            param.is_tunable = False
+            param.search_space = None
+
     def compile(self, params: Dict[str, Any]):
         self._check_parameters(params)
+        if 'TILE_CFG' in self._parameters and 'TILE_CFG' not in params:
+            self.set_parameter('TILE_CFG', 0)   # not the choice of an earlier configuration
         self.set_parameters(params)
         self.update_func()
         self.ready = True

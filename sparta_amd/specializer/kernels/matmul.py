@@ -87,21 +87,8 @@ class SparseMatMulKernel(KernelBase):
         # default search space so that reference configs and trial counts carry over.
         self._add_parameter('TILE_CFG', value=0)
 
-    def enable_tile_search(self, enabled: bool = True):
-        """Add (or remove) the gfx950 tile configuration to the tunable parameters.
-        Off by default so that the search space equals the reference's; tune(...,
-        tile_configs=True) switches it on.  Configurations that do not fit the
-        operand layout are rejected by the library with an AssertionError, which the
-        tuner counts as an infinitely slow trial."""
-        param = self._parameters['TILE_CFG']
-        if enabled:
-            op = _lib.OP_DDS if self._mode == 'dds' else _lib.OP_SPMM
-            ids = [cfg['id'] for cfg in _lib.tile_configs(op)]
-            param.is_tunable = True
-            param.search_space = TunableItemCfg('choice', ids)
-        else:
-            param.is_tunable = False
-            param.search_space = None
+    def _tile_op(self):
+        return _lib.OP_DDS if self._mode == 'dds' else _lib.OP_SPMM
 
     def set_parameters(self, params: Dict[str, Any]):
         super().set_parameters(params)

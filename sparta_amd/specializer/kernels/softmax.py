@@ -29,8 +29,11 @@ class SparseSoftmaxKernel(KernelBase):
         for name in ('BATCH_SIZE', 'GLOBAL_H_VALUE', 'GLOBAL_W_VALUE'):
             self._add_parameter(name)
         self._add_parameter('COMPRESSED', value=self._compressed)
-        # gfx950 kernel variant (0 = chosen by the library); outside the search space
+        # gfx950 kernel variant (0 = chosen by the library); outside the default search space
         self._add_parameter('TILE_CFG', value=0)
+
+    def _tile_op(self):
+        return _lib.OP_SOFTMAX
 
     def set_parameters(self, params: Dict[str, Any]):
         super().set_parameters(params)

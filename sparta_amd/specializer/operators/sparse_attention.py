@@ -401,7 +401,35 @@ class SparseAttention(OperatorBase):
         for name, op, _ in self._parts():
             prefix = f'{name}/'
             check_shared_block_shapes(op._sparse_ctx._kernels, {k[len(prefix):] for k in config if k.startswith(prefix)})
+        if 'fused/forward' in config:   # written by tune(..., tile_configs=...)
+            self._fused_tile_cfg = int(config['fused/forward'].get('TILE_CFG', 0) or 0)
         self.ready = True
+
+    def tune_tile_config(self, sample_inputs: List[torch.Tensor], num_warmups: int = 10, num_iters: int = 10):
+        """Time the fused forward kernel under every tile configuration of the library's
+        attention table on `sample_inputs` (device time), keep the fastest one whose output
+        agrees with the three-operator pipeline, and return it as a configuration entry
+        ({'fused/forward': {'TILE_CFG': id}}, accepted by build()); None when the fused kernel
+        does not take these inputs.  The operator must be built."""
+        from sparta_amd.testing import profile
+        query, key, value = (t.detach() for t in sample_inputs)
+        if not (self.ready and self._fused and self._fused_supported(query)):
+            return None
+        with torch.no_grad():
+            scores = self._matmul_qk.forward(query, key)
+            want = self._matmul_out.forward(self._softmax.forward(scores), value)
+            del scores
+            best_id, best_latency = 0, float('inf')
+            for tile in _lib.tile_configs(_lib.OP_ATTENTION):
+                self._fused_tile_cfg = tile['id']
+                try:
+                    latency = profile(self._fused_forward, [query, key, value], [want], num_warmups, num_iters, cuda=True)
+                except AssertionError:   # the configuration does not take this block shape / head dim
+                    latency = float('inf')
+                if latency < best_latency:
+                    best_id, best_latency = tile['id'], latency
+        self._fused_tile_cfg = best_id
+        return {'fused/forward': {'TILE_CFG': best_id}}
 
     def set_sample_inputs(self, sample_inputs: List[torch.Tensor],
                           sample_grads: Optional[List[torch.Tensor]] = None):

@@ -18,12 +18,16 @@ class DynamicSparseMoE(torch.nn.Module):
     """Args:
         exp_modules: one bias-free torch.nn.Linear per expert, all of one shape.
 
+        tile_cfg: tile configuration of the gathered product (0 = the library's choice from
+            the problem size; see spx_tile_cfg_info, table SPX_OP_MOE).
+
     forward(tokens [n_tok, in], exp_ids int32 [n_tok]) -> [n_tok, out].
     """
 
-    def __init__(self, exp_modules: List[torch.nn.Linear]):
+    def __init__(self, exp_modules: List[torch.nn.Linear], tile_cfg: int = 0):
         super().__init__()
         _lib.load()
+        self.tile_cfg = int(tile_cfg)
         self.num_exps = len(exp_modules)
         self.out_hidden, self.in_hidden = exp_modules[0].weight.shape
         self.device = exp_modules[0].weight.device
@@ -69,6 +73,35 @@ class DynamicSparseMoE(torch.nn.Module):
         rc = lib.spx_moe_forward(_lib.dtype_code(tokens.dtype), _lib.dev_ptr(tokens),
                                  _lib.dev_ptr(weight.contiguous()), 0, _lib.dev_ptr(out),
                                  _lib.dev_ptr(self.expert_offset), _lib.dev_ptr(self.sparse_index),
-                                 n_tok, self.in_hidden, self.out_hidden, self.num_exps, 0, stream)
+                                 n_tok, self.in_hidden, self.out_hidden, self.num_exps, self.tile_cfg, stream)
         _lib.check(rc, 'spx_moe_forward')
         return out
+
+    # ---- tile configuration (sparta.nn.tune(..., tile_configs=...)) ---------------------
+    def set_tile_config(self, config):
+        """Accepts what tune_tile_config returns: {'forward': {'TILE_CFG': id}}."""
+        self.tile_cfg = int((config or {}).get('forward', {}).get('TILE_CFG', 0) or 0)
+
+    def tune_tile_config(self, sample_inputs, num_warmups: int = 5, num_iters: int = 5):
+        """Time the forward pass on `sample_inputs` = [tokens, exp_ids] (device time) under
+        every tile configuration of the library's MoE table, keep the fastest one whose
+        output agrees with the per-expert dense products, and return it as
+        {'forward': {'TILE_CFG': id}}."""
+        from sparta_amd.testing import profile
+        tokens, exp_ids = (t.detach() for t in sample_inputs)
+        with torch.no_grad():
+            want = torch.zeros((tokens.shape[0], self.out_hidden), dtype=tokens.dtype, device=tokens.device)
+            for e in range(self.num_exps):
+                rows = exp_ids == e
+                want[rows] = torch.matmul(tokens[rows].float(), self.weight[e].float()).to(tokens.dtype)
+            best_id, best_latency = 0, float('inf')
+            for tile in _lib.tile_configs(_lib.OP_MOE):
+                self.tile_cfg = tile['id']
+                try:
+                    latency = profile(self.forward, [tokens, exp_ids], [want], num_warmups, num_iters, cuda=True)
+                except AssertionError:   # the configuration does not take this dtype / layout
+                    latency = float('inf')
+                if latency < best_latency:
+                    best_id, best_latency = tile['id'], latency
+        self.tile_cfg = best_id
+        return {'forward': {'TILE_CFG': best_id}}

@@ -238,6 +238,131 @@ def test_tune_grid_builds_best_config(gpu):
     assert_close(op2(x.to(gpu)), want, torch.float32, 'built op')
 
 
+def _tuner_log():
+    """Collects the tuner's trial lines ('... => <latency> ms')."""
+    import logging
+    from sparta_amd.nn import module_tuner
+    lines = []
+
+    class Collect(logging.Handler):
+        def emit(self, record):
+            lines.append(record.getMessage())
+
+    handler = Collect()
+    module_tuner._logger.addHandler(handler)
+    return lines, lambda: module_tuner._logger.removeHandler(handler)
+
+
+@pytest.mark.parametrize('tile_configs', [True, 'refine'])
+def test_tune_searches_the_tile_configurations(tile_configs, gpu):
+    """tune(tile_configs=...) really enumerates the library's tile table, on device time:
+    every configuration id shows up as a trial, configurations the library refuses for this
+    layout count as infinitely slow trials, the winner is written as TILE_CFG into a config
+    that build() accepts, and the tuned operator still matches the oracle (forward and the
+    gradient of the input)."""
+    from sparta_amd import _lib
+    M, K, N = 512, 256, 256
+    x_np, x = randn((M, K), 15, torch.float16)
+    w_np, w = randn((N, K), 16, torch.float16)
+    g_np, g = randn((M, N), 18, torch.float16)
+    mask_np = ops.block_mask((N, K), (32, 32), 0.7, seed=17)
+    mask = torch.from_numpy(mask_np).to(gpu)
+    lin = dense_linear(K, N, w * torch.from_numpy(mask_np), None, gpu, torch.float16)
+    op = sparta.nn.SparseLinear(lin, weight_mask=mask)
+    lines, stop = _tuner_log()
+    try:
+        best = sparta.nn.tune(op, sample_inputs=[x.to(gpu)], sample_grads=[g.to(gpu)], algo='grid', max_trials=10 ** 6,
+                              backward_weight=1.0, tile_configs=tile_configs, verbose=True)
+    finally:
+        stop()
+    config = best['root']
+    assert set(config) == {'forward:C', 'backward:A', 'backward:B'}
+    trials = [l for l in lines if '=> ' in l]
+    failed = [l for l in trials if '=> inf' in l]
+    n_spmm, n_dds = (len(_lib.tile_configs(op_id)) for op_id in (_lib.OP_SPMM, _lib.OP_DDS))
+    # the reference's space per kernel: 3 x 3 upper points (the two tile dims are shared) x one
+    # free block size, + the single point of the 'openai' slot (test/unit/test_tuners.py:58-61)
+    if tile_configs is True:
+        # joint search: every lower space is multiplied by the kernel's tile table
+        assert len(trials) == (9 * 3 + 1) * (n_spmm + n_spmm + n_dds)
+    else:
+        # the reference's space first, then the tile table once per kernel
+        assert len(trials) == (9 * 3 + 1) * 3 + (n_spmm + n_spmm + n_dds)
+    # the thin-operand kernel (tile config 9) takes 64 / 128 rows of m only: refused for M = 512
+    assert failed and len(failed) < len(trials)
+    chosen = {name: cfg.get('TILE_CFG', 0) for name, cfg in config.items()}
+    assert all(0 <= c < n_spmm for c in chosen.values())
+    # reference configs carry no TILE_CFG: building one resets the kernels to the library's choice
+    want = ops.matmul_reference(x_np[None], w_np[None], None, mode='dsd', transpose_A=False, transpose_B=True,
+                                mask=mask_np, dtype=np.float64)[0]
+    for name, cfg in config.items():
+        kernel = op._sparse_ctx._kernels[name].active_kernel()
+        assert int(kernel.get_parameter('TILE_CFG') or 0) == chosen[name]
+    xg = x.to(gpu).requires_grad_(True)
+    y = op(xg)
+    assert_close(y, want, torch.float16, f'tuned op, tile configs {chosen}')
+    y.backward(g.to(gpu))
+    want_gx = g_np @ (w_np * mask_np)
+    assert_close(xg.grad, want_gx, torch.float16, 'tuned op, input gradient', scale=float(np.abs(want_gx).max()))
+    op2 = sparta.nn.SparseLinear(dense_linear(K, N, w * torch.from_numpy(mask_np), None, gpu, torch.float16), weight_mask=mask)
+    sparta.nn.build(op2, [x.to(gpu)], best)
+    assert_close(op2(x.to(gpu)), want, torch.float16, 'built from the tuned config')
+    plain = {name: {k: v for k, v in cfg.items() if k != 'TILE_CFG'} for name, cfg in config.items()}
+    op2.build(plain, sample_inputs=[x.to(gpu)])
+    assert all(int(op2._sparse_ctx._kernels[n].active_kernel().get_parameter('TILE_CFG') or 0) == 0 for n in plain)
+
+
+def test_tune_tile_configurations_of_softmax_attention_and_moe(gpu):
+    """The softmax kernels' TILE_CFG, the fused attention kernel's and the MoE product's tile
+    configuration are search entries too; the tuned modules match their references."""
+    from sparta_amd import _lib
+    H, Nt, Ns, E = 2, 256, 256, 64
+    _, q = randn((H, Nt, E), 21, torch.float16)
+    _, k = randn((H, Ns, E), 22, torch.float16)
+    _, v = randn((H, Ns, E), 23, torch.float16)
+    mask_np = ops.block_mask((Nt, Ns), (32, 32), 0.6, seed=24)
+    att = sparta.nn.SparseAttention(mask=torch.from_numpy(mask_np).to(gpu))
+    lines, stop = _tuner_log()
+    try:
+        best = sparta.nn.tune(att, sample_inputs=[q.to(gpu), k.to(gpu), v.to(gpu)], algo='rand', max_trials=3,
+                              tile_configs='refine', verbose=True)
+    finally:
+        stop()
+    config = best['root']
+    assert 'fused/forward' in config and 0 <= config['fused/forward']['TILE_CFG'] < len(_lib.tile_configs(_lib.OP_ATTENTION))
+    n_sm = len(_lib.tile_configs(_lib.OP_SOFTMAX))
+    assert sum('[Kernel: sm/forward:y] tile config' in l for l in lines) == n_sm
+    want = ops.attention_reference(*(t.double().numpy() for t in (q, k, v)), mask_np)
+    with torch.no_grad():
+        assert_close(att(q.to(gpu), k.to(gpu), v.to(gpu)), want, torch.float16, 'tuned attention (fused)')
+        att._fused = False
+        assert_close(att(q.to(gpu), k.to(gpu), v.to(gpu)), want, torch.float16, 'tuned attention (three operators)')
+    att2 = sparta.nn.SparseAttention(mask=torch.from_numpy(mask_np).to(gpu))
+    sparta.nn.build(att2, [q.to(gpu), k.to(gpu), v.to(gpu)], best)
+    assert att2._fused_tile_cfg == config['fused/forward']['TILE_CFG']
+
+    class Net(torch.nn.Module):
+        def __init__(self, moe):
+            super().__init__()
+            self.moe = moe
+
+        def forward(self, tokens, ids):
+            return self.moe(tokens, ids)
+
+    torch.manual_seed(3)
+    experts = [torch.nn.Linear(128, 256, bias=False, device=gpu, dtype=torch.float16) for _ in range(4)]
+    tokens = torch.randn((512, 128), device=gpu, dtype=torch.float16)
+    ids = torch.randint(0, 4, (512,), device=gpu, dtype=torch.int32)
+    net = Net(sparta.nn.DynamicSparseMoE(experts))
+    best = sparta.nn.tune(net, sample_inputs=[tokens, ids], tile_configs=True)
+    assert set(best) == {'root/moe'} and net.moe.tile_cfg == best['root/moe']['forward']['TILE_CFG']
+    want = torch.stack([experts[int(e)](t) for t, e in zip(tokens, ids.cpu())])
+    torch.testing.assert_close(net(tokens, ids).float(), want.float(), rtol=1e-2, atol=1e-2)
+    net2 = Net(sparta.nn.DynamicSparseMoE(experts))
+    sparta.nn.build(net2, [tokens, ids], best)
+    assert net2.moe.tile_cfg == net.moe.tile_cfg
+
+
 def test_tune_inside_a_combined_module(gpu):
     class Net(torch.nn.Module):
         def __init__(self, a, b):
