@@ -45,7 +45,8 @@ def time_graph(torch, fn, steps, warmup, repeats=1, min_total=0.0):
     bracketed by events on the replay stream.  Returns seconds for all steps (the
     shortest of the timed replays: at least `repeats` of them, and as many more as
     it takes to spend `min_total` seconds of device time, so that a short graph is
-    also timed at settled clocks)."""
+    also timed at settled clocks).  `time_graph.last` keeps the shortest and the mean
+    replay and their number."""
     for _ in range(max(warmup, 1)):
         fn()
     torch.cuda.synchronize()
@@ -71,7 +72,11 @@ def time_graph(torch, fn, steps, warmup, repeats=1, min_total=0.0):
             best = took if best is None else min(best, took)
             total += took
             done += 1
+    time_graph.last = {'steps': steps, 'replays': done, 'min_s': best, 'mean_s': total / done}
     return best
+
+
+time_graph.last = None
 
 
 def time_eager(torch, fn, steps, warmup):
@@ -266,13 +271,15 @@ def main():
     if not args.no_secondary:
         import bench_configs
         try:
-            rows = bench_configs.run(['c1', 'c2', 'c3', 'c4', 'c5'], min(args.steps, 50), min(args.warmup, 10), time_graph,
+            sec_steps = min(args.steps, 50)
+            rows = bench_configs.run(['c1', 'c2', 'c3', 'c4', 'c5'], sec_steps, min(args.warmup, 10), time_graph,
                                      time_eager, brief=True, verbose=False)
             out['secondary'] = {
                 'note': 'other benchmark configurations; each result was compared with the dense fp32 torch '
-                        'computation of the same inputs before it was timed; times are the shortest graph '
-                        'replay of 50 steps out of at least three and at least 50 ms of replays (the first short '
-                        'replays right after the checks run at ramping clocks)',
+                        f'computation of the same inputs before it was timed; a replay is one graph of {sec_steps} '
+                        'steps, replayed at least three times and for at least 50 ms: "ms" is the shortest replay '
+                        '(the first short replays right after the checks run at ramping clocks), "ms_mean" the '
+                        'mean over all "replays" (the statistic of the reference\'s profile())',
                 'results': [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in r.items()
                              if k != 'expert_counts'} for r in rows],
             }

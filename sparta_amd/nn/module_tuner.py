@@ -20,8 +20,12 @@ import torch
 from sparta_amd.common.tuning import TunableItemCfg
 from sparta_amd.specializer import OperatorBase
 
-_logger = logging.Logger(__name__)
-_logger.addHandler(logging.StreamHandler())
+# A logger of the logging module's registry (a bare logging.Logger(...) keeps its cache of
+# enabled levels across setLevel, so `verbose` would stick to its first value).
+_logger = logging.getLogger(__name__)
+_logger.propagate = False
+if not _logger.handlers:
+    _logger.addHandler(logging.StreamHandler())
 
 
 class Tuner:

@@ -150,10 +150,14 @@ class SparseAttention(OperatorBase):
                 query.requires_grad or key.requires_grad or value.requires_grad):
             self._warned_unfused = True
             indexes = self._sparse_port.indexes
-            warnings.warn(
-                f'SparseAttention: no fused training kernel for {query.dtype} inputs of head dim {query.shape[-1]} '
-                f'with {indexes.block_H}x{indexes.block_W} score blocks (16-bit types, head dims 64 / 128 and '
-                'blocks of 32 / 64 / 128 are covered); this step runs as three forward and six backward launches')
+            ctxs = (self._matmul_qk._sparse_ctx, self._matmul_out._sparse_ctx)
+            if all(hasattr(c, 'backward_B') for c in ctxs):
+                why = (f'no fused training kernel for {query.dtype} inputs of head dim {query.shape[-1]} with '
+                       f'{indexes.block_H}x{indexes.block_W} score blocks (16-bit types, head dims 64 / 128 and '
+                       'blocks of 32 / 64 / 128 are covered)')
+            else:
+                why = 'the backward kernels of the operator were not built (no backward:* entries in its configuration)'
+            warnings.warn(f'SparseAttention: {why}; this step runs as three forward launches and six backward launches')
         scores = self._matmul_qk.forward(query, key)
         probs = self._softmax.forward(scores)
         return self._matmul_out.forward(probs, value)
