@@ -15,7 +15,10 @@ method and point; the Triton competitors are left out).
 Operator configurations come from the tuned-config tables shipped in
 sparta_amd/params/<op>/ (`<device name>.csv`, else `default.csv`; the format of the
 reference's test/bench/*/params/default.csv).  With --tune the tables are
-regenerated on this GPU into --out.  Results go to <out>/sweep_<op>_<dtype>.csv.
+regenerated on this GPU into --out: block sizes by the tuner's search over the reference's
+space, then the gfx950 tile configuration of every kernel with those block sizes kept
+(tune(..., tile_configs='refine'); every trial is timed on the device).  Results go to
+<out>/sweep_<op>_<dtype>.csv.
 """
 import argparse
 import os
@@ -123,7 +126,7 @@ def sweep_matmul(args, torch, sparta, table_dir, device_name):
             sample = [data['A'], data['B']]
             if args.tune:
                 best = sparta.nn.tune(op, sample_inputs=sample, sample_grads=[data['grad_C']], algo=args.algo,
-                                      max_trials=args.tune, backward_weight=1.0, tile_configs=False)
+                                      max_trials=args.tune, backward_weight=1.0, tile_configs='refine')
                 config = best['root']
                 if config is None:
                     config = MATMUL_FALLBACK
@@ -180,7 +183,7 @@ def sweep_attention(args, torch, sparta, table_dir, device_name):
             op = sparta.nn.SparseAttention(mask=mask)
             if args.tune:
                 best = sparta.nn.tune(op, sample_inputs=[q, k, v], sample_grads=[grad], algo=args.algo,
-                                      max_trials=args.tune, backward_weight=1.0)
+                                      max_trials=args.tune, backward_weight=1.0, tile_configs='refine')
                 config = best['root']
                 if config is None:  # every random trial hit an invalid combination: use the fallback
                     config = ATTENTION_FALLBACK

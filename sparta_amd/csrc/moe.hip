@@ -536,9 +536,11 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeParams p) {
 // stage.  The loads are issued through inline assembly, which keeps the compiler from
 // serialising them against the fragment reads of the other buffers.
 
-template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN>
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN, bool XS>
 __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 : 2) void moe_gemm_direct_kernel(MoeParams p) {
     static_assert(!BKN || sizeof(T) == 2, "the [K, N] weight layout is read with 16-bit LDS transpose loads");
+    static_assert(!XS || (HasMma32<T>::value && NBUF >= 3 && NBUF <= 4 && (KTB / (int)sizeof(T) / 16) % 2 == 0),
+                  "the cross-stage pipeline needs 32x32 MFMAs, three or four buffers and an even number of k-steps per stage");
     constexpr int NTH = 64 * WAVES;
     constexpr int WGN = WAVES / WGM;
     constexpr int MT = TM / WGM / 16;   // 16-row tiles per wave
@@ -659,6 +661,76 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
     for (int s0 = 0; s0 < NBUF - 1; ++s0)
         if (s0 < n_st) issue_stage(s0);
 
+    // wait until at most `newer` stages of this thread's loads are still in flight
+    auto wait_stages = [&](int newer) {
+        if (NBUF > 3 && newer >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L) : "memory");
+        else if (NBUF > 2 && newer == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+
+    if constexpr (XS) {
+        // Cross-stage pipeline: shallow stages (KTB bytes of k) in a ring of NBUF buffers, and the
+        // barrier that publishes stage s + 1 sits ahead of the LAST k-step of stage s, whose MFMAs
+        // then run over the first fragment reads of stage s + 1.  The wait for the loads, the
+        // barrier and the LDS latency of a stage's first fragments - about 800 clocks that a
+        // barrier at the top of the stage leaves the matrix cores idle - are covered by MFMAs
+        // that are already queued.  Loads run NBUF - 1 stages ahead, so the wait is short.
+        constexpr int KSTEPS = KT / 16;
+        typename MmaW<T>::frag af[2][MTW], bf[2][NTW];
+        auto read_frags = [&](const char* As, const char* Bs, int c, int slot) {
+#pragma unroll
+            for (int i = 0; i < MTW; ++i)
+                af[slot][i] = *reinterpret_cast<const typename MmaW<T>::frag*>(As + lds_off(wrow + i * 32 + l32, c * 2 + h2));
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) {
+                if constexpr (BKN) {
+                    typedef short s16x8_t __attribute__((ext_vector_type(8)));
+                    typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
+                    const int kr = c * 16 + 8 * h2 + (r16 >> 2);             // and kr + 4
+                    const int unit = (wcol + t * 32 + 16 * ((lane >> 4) & 1)) >> 4;
+                    const char* at = Bs + kr * RB + ((unit ^ ((kr & 3) << 1)) << 5) + ((r16 & 3) << 3);
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(at + 4 * RB));
+                    bf[slot][t] = __builtin_bit_cast(typename MmaW<T>::frag,
+                                                     (s16x8_t)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                } else {
+                    bf[slot][t] = *reinterpret_cast<const typename MmaW<T>::frag*>(Bs + lds_off(wcol + t * 32 + l32, c * 2 + h2));
+                }
+            }
+        };
+        wait_stages(n_st - 1 < NBUF - 2 ? n_st - 1 : NBUF - 2);
+        __syncthreads();
+        read_frags(smem, smem + A_BYTES, 0, 0);
+        for (int s = 0; s < n_st; ++s) {
+            const char* cur = smem + (s % NBUF) * BUF;
+            const char* nxt = smem + ((s + 1) % NBUF) * BUF;
+            const bool more = s + NBUF - 1 < n_st;
+#pragma unroll
+            for (int c = 0; c < KSTEPS; ++c) {
+                if (c + 1 < KSTEPS) {
+                    read_frags(cur, cur + A_BYTES, c + 1, (c + 1) & 1);
+                } else if (s + 1 < n_st) {
+                    // stage s + 1 has landed once only the stages after it are in flight; every
+                    // fragment read of stage s has been issued by now, and is complete before
+                    // the barrier lets anyone's loads into that buffer
+                    const int last = s + NBUF - 1 < n_st - 1 ? s + NBUF - 1 : n_st - 1;
+                    wait_stages(last - (s + 1));
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    read_frags(nxt, nxt + A_BYTES, 0, 0);
+                }
+                // the loads of stage s + NBUF - 1 reuse the buffer of stage s - 1, which the
+                // barrier inside stage s - 1 has freed
+                // (all of them in the first k-step, so that the wait above counts whole stages)
+                if (more && c == 0) issue_stage(s + NBUF - 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < MTW; ++i)
+#pragma unroll
+                    for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
+            }
+        }
+    } else
     for (int s = 0; s < n_st; ++s) {
         // stage s has landed once at most the loads of the stages after it are outstanding
         // (NBUF - 2 of them, fewer at the end of the walk)
@@ -804,7 +876,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
     }
 }
 
-template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN>
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool BKN, bool XS>
 static int launch_moe_direct_inst(const MoeParams& p, hipStream_t st) {
     // split 2 covers at most one round of 256-row tiles, as 128-row halves
     const int tiles = p.split == 2 ? 2 * p.round_rows : (p.n_tok + TM - 1) / TM + p.n_exp + 1;
@@ -812,19 +884,23 @@ static int launch_moe_direct_inst(const MoeParams& p, hipStream_t st) {
     // the epilogue stages every wavefront's (TM / WGM) x 64 output tile as rows of 128 bytes
     const int epi = sizeof(T) == 2 ? WAVES * (TM / WGM) * 128 : 0;
     const int smem = NBUF * (TM + TN) * KTB > epi ? NBUF * (TM + TN) * KTB : epi;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF, KTB, BKN>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF, KTB, BKN, XS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(moe_gemm_direct_kernel)");
-    hipLaunchKernelGGL((moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF, KTB, BKN>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
+    hipLaunchKernelGGL((moe_gemm_direct_kernel<T, TM, TN, WAVES, WGM, NBUF, KTB, BKN, XS>), dim3((p.N + TN - 1) / TN, tiles, 1), dim3(64 * WAVES), smem, st, p);
     SPX_LAUNCH_CHECK("moe_gemm_direct_kernel");
     return 0;
 }
 
-template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB>
+template <typename T, int TM, int TN, int WAVES, int WGM, int NBUF, int KTB, bool XS = false>
 static int launch_moe_direct(const MoeParams& p, hipStream_t st) {
-    if (p.w_kcontig) return launch_moe_direct_inst<T, TM, TN, WAVES, WGM, NBUF, KTB, false>(p, st);
-    if constexpr (sizeof(T) == 2) return launch_moe_direct_inst<T, TM, TN, WAVES, WGM, NBUF, KTB, true>(p, st);
-    else return fail(SPX_E_CONFIG, "fp32 weights stored [E, in, out] run through tile config 1");
+    if constexpr (XS && sizeof(T) != 2) {
+        return fail(SPX_E_CONFIG, "the cross-stage pipelined tile configurations take 16-bit types");
+    } else {
+        if (p.w_kcontig) return launch_moe_direct_inst<T, TM, TN, WAVES, WGM, NBUF, KTB, false, XS>(p, st);
+        if constexpr (sizeof(T) == 2) return launch_moe_direct_inst<T, TM, TN, WAVES, WGM, NBUF, KTB, true, XS>(p, st);
+        else return fail(SPX_E_CONFIG, "fp32 weights stored [E, in, out] run through tile config 1");
+    }
 }
 
 // Tokens per workgroup of the index kernels: the smallest multiple of 256 (up to MOE_CHUNK)
@@ -907,7 +983,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
                                int n_tok, int in_dim, int out_dim, int n_exp,
                                int tile_cfg, spx_stream_t stream) {
     using namespace spx;
-    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
+    SPX_REQUIRE(tile_cfg >= 0 && tile_cfg <= 6, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     SPX_REQUIRE(dtype == SPX_F32 || dtype == SPX_F16 || dtype == SPX_BF16, SPX_E_DTYPE, "unknown dtype %d", dtype);
     SPX_REQUIRE(n_tok >= 0 && in_dim > 0 && out_dim > 0 && n_exp > 0, SPX_E_SHAPE, "bad sizes");
     SPX_REQUIRE(weight_layout == 0 || weight_layout == 1, SPX_E_CONFIG, "weight_layout must be 0 ([E,in,out]) or 1 ([E,out,in])");
@@ -952,7 +1028,6 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
         else if (es == 2 && big_tiles >= 128 && (row_tiles + n_exp) * col_tiles <= n_cu) tile_cfg = 4;
         else tile_cfg = 2;
     }
-    SPX_REQUIRE(tile_cfg <= 5, SPX_E_CONFIG, "unknown tile config %d", tile_cfg);
     if (tile_cfg >= 2) {
         SPX_REQUIRE(direct_ok, SPX_E_CONFIG, "tile config %d takes fp32 weights in layout 1 only", tile_cfg);
         if (tile_cfg == 5) {
@@ -967,6 +1042,7 @@ extern "C" int spx_moe_forward(int dtype, const void* tokens, const void* weight
             p.split = 2;                                                                   \
             return launch_moe_direct<T, 128, 128, 4, 2, 2, 128>(p, st);                    \
         }                                                                                  \
+        if (tile_cfg == 6) return launch_moe_direct<T, 256, 256, 16, 4, 4, 64, true>(p, st); \
         if (tile_cfg == 2) return launch_moe_direct<T, 128, 128, 4, 2, 2, 128>(p, st);     \
         if (tile_cfg == 3) return launch_moe_direct<T, 256, 256, 8, 2, 2, 128>(p, st);     \
         return launch_moe_direct<T, 256, 256, 16, 4, 2, 128>(p, st);

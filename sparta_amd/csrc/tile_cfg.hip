@@ -48,6 +48,7 @@ static const spx_tile_cfg kMoeCfgs[] = {
     {3, 256, 256, 8, 2, 0, 7, "gather-256x256-lds-direct"},
     {4, 256, 256, 16, 2, 0, 7, "gather-256x256-direct-16-waves"},
     {5, 256, 256, 16, 2, 0, 7, "gather-256x256-plus-128-tail"},
+    {6, 256, 256, 16, 4, 0, 6, "gather-256x256-cross-stage"},
 };
 
 static const spx_tile_cfg* table(int op, int* n) {
