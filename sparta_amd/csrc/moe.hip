@@ -221,9 +221,78 @@ struct MoeParams {
 // split 2 = the remaining row tiles cut into 128-row halves for the small-tile kernel,
 // which fills the device with them.  Both launches derive the same boundary from the
 // device-side expert counts.
+// Single launch (split == 0): the row tiles are numbered with every expert's full tiles first
+// and the partly filled last tiles of the experts behind them (longest first).  Workgroups start in the order
+// of their tile numbers, so the short tiles (a partly filled tile skips the work of its empty
+// 64-row groups) fill the end of the launch, where the long ones would leave most CUs idle.
+template <int TM>
+__device__ __forceinline__ void moe_find_tile_sorted(const MoeParams& p, int y, int lane,
+                                                     int& found_e, int& found_row0, int& found_rows) {
+    int total_full = 0;
+    for (int e0 = 0; e0 <= p.n_exp; e0 += 64) {
+        const int e = e0 + lane;
+        int cnt = 0;
+        if (e <= p.n_exp) cnt = (e < p.n_exp ? p.expert_offset[e + 1] : p.n_tok) - p.expert_offset[e];
+        total_full += __shfl(wave_inclusive_scan(cnt / TM), 63, 64);
+    }
+    const bool part = y >= total_full;   // looking for a partly filled tile
+    const int want = part ? y - total_full : y;
+    int before = 0;
+    found_e = -1; found_row0 = 0; found_rows = 0;
+    if (part && p.n_exp < 64) {
+        // at most 64 candidates: the partly filled tiles go out longest first (rank = number of
+        // experts whose last tile holds more rows, ties in expert order)
+        int cnt = 0, off = 0;
+        if (lane <= p.n_exp) {
+            off = p.expert_offset[lane];
+            cnt = (lane < p.n_exp ? p.expert_offset[lane + 1] : p.n_tok) - off;
+        }
+        const int full = cnt / TM, rest = cnt - full * TM;
+        int rank = 0;
+        for (int o = 0; o <= p.n_exp; ++o) {
+            const int r = __shfl(rest, o, 64);
+            rank += (r > rest || (r == rest && o < lane)) ? 1 : 0;
+        }
+        const unsigned long long hit = __ballot(rest > 0 && rank == want);
+        if (hit) {
+            const int src = __ffsll((long long)hit) - 1;
+            found_e = src;
+            found_row0 = __shfl(off, src, 64) + __shfl(full, src, 64) * TM;
+            found_rows = __shfl(rest, src, 64);
+        }
+        return;
+    }
+    for (int e0 = 0; e0 <= p.n_exp; e0 += 64) {
+        const int e = e0 + lane;
+        int cnt = 0, off = 0;
+        if (e <= p.n_exp) {
+            off = p.expert_offset[e];
+            cnt = (e < p.n_exp ? p.expert_offset[e + 1] : p.n_tok) - off;
+        }
+        const int full = cnt / TM, rest = cnt - full * TM;
+        const int tiles = part ? (rest ? 1 : 0) : full;
+        const int inc = wave_inclusive_scan(tiles);
+        const int excl = before + inc - tiles;
+        const unsigned long long hit = __ballot(want >= excl && want < excl + tiles);
+        if (hit) {
+            const int src = __ffsll((long long)hit) - 1;
+            const int lt = want - __shfl(excl, src, 64);
+            found_e = e0 + src;
+            found_row0 = __shfl(off, src, 64) + (part ? __shfl(full, src, 64) : lt) * TM;
+            found_rows = part ? __shfl(rest, src, 64) : TM;
+            return;
+        }
+        before += __shfl(inc, 63, 64);
+    }
+}
+
 template <int TM>
 __device__ __forceinline__ void moe_find_tile(const MoeParams& p, int y, int lane,
                                               int& found_e, int& found_row0, int& found_rows) {
+    if (p.split == 0) {
+        moe_find_tile_sorted<TM>(p, y, lane, found_e, found_row0, found_rows);
+        return;
+    }
     const int TS = p.split ? 256 : TM;      // tile height the row tiles are counted in
     int half = 0;
     if (p.split == 2) { half = y & 1; y >>= 1; }
@@ -583,6 +652,9 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
     const int r16 = lane & 15, g4 = lane >> 4;
     const int wm = wave / WGN, wn = wave % WGN;
     const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
+    // a partly filled tile: wavefronts whose rows are all past its end load their share of the
+    // stages and meet the barriers, but read no fragments, issue no MFMAs and store nothing
+    const bool active = wrow < rows;
 
     const T* X = reinterpret_cast<const T*>(p.tokens);
     const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
@@ -700,7 +772,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
         };
         wait_stages(n_st - 1 < NBUF - 2 ? n_st - 1 : NBUF - 2);
         __syncthreads();
-        read_frags(smem, smem + A_BYTES, 0, 0);
+        if (active) read_frags(smem, smem + A_BYTES, 0, 0);
         for (int s = 0; s < n_st; ++s) {
             const char* cur = smem + (s % NBUF) * BUF;
             const char* nxt = smem + ((s + 1) % NBUF) * BUF;
@@ -708,7 +780,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
 #pragma unroll
             for (int c = 0; c < KSTEPS; ++c) {
                 if (c + 1 < KSTEPS) {
-                    read_frags(cur, cur + A_BYTES, c + 1, (c + 1) & 1);
+                    if (active) read_frags(cur, cur + A_BYTES, c + 1, (c + 1) & 1);
                 } else if (s + 1 < n_st) {
                     // stage s + 1 has landed once only the stages after it are in flight; every
                     // fragment read of stage s has been issued by now, and is complete before
@@ -717,17 +789,19 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                     wait_stages(last - (s + 1));
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                     __syncthreads();
-                    read_frags(nxt, nxt + A_BYTES, 0, 0);
+                    if (active) read_frags(nxt, nxt + A_BYTES, 0, 0);
                 }
                 // the loads of stage s + NBUF - 1 reuse the buffer of stage s - 1, which the
                 // barrier inside stage s - 1 has freed
                 // (all of them in the first k-step, so that the wait above counts whole stages)
                 if (more && c == 0) issue_stage(s + NBUF - 1);
                 __builtin_amdgcn_sched_barrier(0);
+                if (active) {
 #pragma unroll
-                for (int i = 0; i < MTW; ++i)
+                    for (int i = 0; i < MTW; ++i)
 #pragma unroll
-                    for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
+                        for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
+                }
             }
         }
     } else
@@ -774,21 +848,23 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                 }
             };
             constexpr int LPS = (L + KSTEPS - 1) / KSTEPS;  // loads per k-step
-            read_frags(0, 0);
+            if (active) read_frags(0, 0);
 #pragma unroll
             for (int c = 0; c < KSTEPS; ++c) {
-                if (c + 1 < KSTEPS) read_frags(c + 1, (c + 1) & 1);
+                if (active && c + 1 < KSTEPS) read_frags(c + 1, (c + 1) & 1);
                 if (more) {
 #pragma unroll
                     for (int q = c * LPS; q < (c + 1) * LPS && q < L; ++q) issue_one(s + NBUF - 1, q);
                 }
                 __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of this step's MFMAs
+                if (active) {
 #pragma unroll
-                for (int i = 0; i < MTW; ++i)
+                    for (int i = 0; i < MTW; ++i)
 #pragma unroll
-                    for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
+                        for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
+                }
             }
-        } else {
+        } else if (active) {
 #pragma unroll
             for (int kc = 0; kc < KT; kc += 16) {
                 typename Mma16<T>::frag af[MT], bf[NTT];
@@ -806,6 +882,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
         }
     }
     __syncthreads();   // the epilogue reuses the LDS buffers
+    if (!active) return;   // no barrier follows
 
     T* out = reinterpret_cast<T*>(p.out);
     if constexpr (WIDE) {

@@ -236,8 +236,8 @@ def test_attention_training_forward_kernel(dtype, bh, bw, E, gran, recompute, gp
     ref_out.backward(g.to(gpu).float())
     want = [ref_out.detach()] + [t.grad for t in ref_leaves]
     for name, a, b, c in zip(('out', 'grad_q', 'grad_k', 'grad_v'), got, piped, want):
-        torch.testing.assert_close(a, c, rtol=2e-2, atol=2e-2, msg=lambda m: f'{name} vs dense autograd: {m}')
-        torch.testing.assert_close(a, b, rtol=2e-2, atol=2e-2, msg=lambda m: f'{name} vs pipeline: {m}')
+        torch.testing.assert_close(a, c, rtol=1e-2, atol=1e-2, msg=lambda m: f'{name} vs dense autograd: {m}')
+        torch.testing.assert_close(a, b, rtol=1e-2, atol=1e-2, msg=lambda m: f'{name} vs pipeline: {m}')
     assert float(got[0][:, :bh].abs().max()) == 0.0 and (block_level or float(got[0][:, bh + 3].abs().max()) == 0.0)
 
 
@@ -296,7 +296,7 @@ def test_attention_backward_scores_kernel(dtype, BH, BW, E, element_mask, gpu, b
     masked = (scores * inv_t).masked_fill(mask == 0, float('-inf'))
     p_ref = torch.softmax(masked, -1).nan_to_num(0.0)
     (p_ref @ vf).backward(g.float())
-    tol = dict(rtol=2e-2, atol=2e-2)
+    tol = dict(rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(row_dot, (g.float() * out.float()).sum(-1) * inv_t, rtol=1e-3, atol=1e-3)
     if BH * E >= 32 * BW:
         grad_k = torch.full_like(k, float('nan'))
@@ -360,7 +360,7 @@ def test_attention_recompute_kernels(dtype, BH, BW, E, gpu, batch=3, Nt=256, Ns=
     p_ref = torch.softmax(masked, -1).nan_to_num(0.0)
     o_ref = p_ref @ vf
     o_ref.backward(g.float())
-    tol = dict(rtol=2e-2, atol=2e-2)
+    tol = dict(rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(out.float(), o_ref.detach(), **tol)
     # natural-log log-sum-exp of the live scores = row_lse * ln 2; +inf where nothing is live
     lse_ref = torch.logsumexp(masked.detach(), -1)
@@ -410,7 +410,7 @@ def test_attention_training_partial_gradients(needs, gpu, H=2, Nt=256, Ns=256, E
     (torch.softmax(scores, -1) @ ref[2]).backward(g.to(gpu).float())
     for t, r, n in zip(leaves, ref, needs):
         if n:
-            torch.testing.assert_close(t.grad.float(), r.grad, rtol=2e-2, atol=2e-2)
+            torch.testing.assert_close(t.grad.float(), r.grad, rtol=1e-2, atol=1e-2)
         else:
             assert t.grad is None
 
@@ -440,6 +440,6 @@ def test_attention_training_after_mask_update(gpu, H=3, Nt=256, Ns=256, E=64, bh
         scores = (ref[0] @ ref[1].transpose(1, 2) / float(np.sqrt(E))).masked_fill(mask == 0, float('-inf'))
         ref_out = torch.softmax(scores, -1).nan_to_num(0.0) @ ref[2]
         ref_out.backward(g.to(gpu).float())
-        torch.testing.assert_close(out.detach().float(), ref_out.detach(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(out.detach().float(), ref_out.detach(), rtol=1e-2, atol=1e-2)
         for t, r in zip(leaves, ref):
-            torch.testing.assert_close(t.grad.float(), r.grad, rtol=2e-2, atol=2e-2)
+            torch.testing.assert_close(t.grad.float(), r.grad, rtol=1e-2, atol=1e-2)

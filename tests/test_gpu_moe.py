@@ -200,7 +200,7 @@ def test_moe_out_of_range_ids_give_zero_rows(gpu):
 
 
 @pytest.mark.parametrize('layout', [0, 1])
-@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5])
+@pytest.mark.parametrize('tile_cfg', [1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize('dtype,n_tok,in_dims,out_dims', [
     (torch.float16, 3000, 256, 520), (torch.bfloat16, 1500, 128, 256), (torch.float32, 700, 96, 136),
     (torch.float16, 5, 64, 64), (torch.float16, 2500, 192, 776)])
@@ -211,6 +211,8 @@ def test_moe_tile_configs(layout, tile_cfg, dtype, n_tok, in_dims, out_dims, gpu
     from sparta_amd import _lib
     if dtype == torch.float32 and layout == 0 and tile_cfg != 1:
         pytest.skip('fp32 weights stored [E, in, out] run through tile config 1')
+    if dtype == torch.float32 and tile_cfg == 6:
+        pytest.skip('the cross-stage pipelined configuration takes 16-bit types')
     n_exp = 5
     moe, w = make_moe(n_exp, in_dims, out_dims, dtype, gpu)
     ids_np = np.random.default_rng(n_tok).choice([0, 1, 2, 4], size=n_tok, p=[0.6, 0.2, 0.15, 0.05]).astype(np.int32)
