@@ -27,6 +27,7 @@ M = K = N = 4096
 BLOCK = (32, 32)
 SPARSITY = 0.95
 SEED = 2022
+SETTLE_S = 0.1   # untimed replays before the timed region (seconds of device time)
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0  # dense fp16
 
@@ -40,13 +41,15 @@ def make_inputs(torch, device):
     return x, w, mask
 
 
-def time_graph(torch, fn, steps, warmup, repeats=1, min_total=0.0):
+def time_graph(torch, fn, steps, warmup, repeats=1, min_total=0.0, settle=0.0):
     """Device time of `steps` calls of fn(), replayed from one captured graph and
     bracketed by events on the replay stream.  Returns seconds for all steps (the
     shortest of the timed replays: at least `repeats` of them, and as many more as
     it takes to spend `min_total` seconds of device time, so that a short graph is
-    also timed at settled clocks).  `time_graph.last` keeps the shortest and the mean
-    replay and their number."""
+    also timed at settled clocks).  `settle` > 0 replays the graph untimed for that many
+    seconds of device time first: the clocks of an idle GPU ramp for tens of milliseconds,
+    longer than a short timed region lasts.  `time_graph.last` keeps the shortest and the
+    mean replay and their number."""
     for _ in range(max(warmup, 1)):
         fn()
     torch.cuda.synchronize()
@@ -60,6 +63,17 @@ def time_graph(torch, fn, steps, warmup, repeats=1, min_total=0.0):
                 fn()
         graph.replay()  # untimed replay: page in the graph
         stream.synchronize()
+        spent, rolls = 0.0, 0
+        while spent < settle and rolls < 100000:
+            begin = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            begin.record(stream)
+            for _ in range(8):
+                graph.replay()
+            end.record(stream)
+            stream.synchronize()
+            spent += begin.elapsed_time(end) / 1e3
+            rolls += 8
         best, total, done = None, 0.0, 0
         while done < max(repeats, 1) or (total < min_total and done < 1000):
             begin = torch.cuda.Event(enable_timing=True)
@@ -194,14 +208,15 @@ def main():
 
         step = lambda: op(x)
         try:
-            total = time_graph(torch, step, args.steps, args.warmup)
-            timing = 'hip graph replay of the timed steps, events on the replay stream'
+            total = time_graph(torch, step, args.steps, args.warmup, settle=SETTLE_S)
+            timing = (f'hip graph replay of the timed steps, events on the replay stream, after the warm-up steps and '
+                      f'{SETTLE_S} s of untimed replays of the same graph (an idle GPU ramps its clocks for tens of ms)')
         except Exception as exc:  # capture unsupported: fall back to the eager loop
             total = time_eager(torch, step, args.steps, args.warmup)
             timing = f'eager loop (graph capture failed: {type(exc).__name__})'
         eager = time_eager(torch, step, args.steps, args.warmup)
         w_dense = dense.weight
-        dense_total = time_graph(torch, lambda: torch.matmul(x, w_dense.t()), min(args.steps, 100), 5)
+        dense_total = time_graph(torch, lambda: torch.matmul(x, w_dense.t()), min(args.steps, 100), 5, settle=SETTLE_S)
         dense_ms = dense_total / min(args.steps, 100) * 1e3
 
         cold = None
@@ -220,7 +235,7 @@ def main():
 
             cold_steps = max(ring * 4, (args.steps // ring) * ring)
             try:
-                cold = time_graph(torch, cold_step, cold_steps, args.warmup) / cold_steps
+                cold = time_graph(torch, cold_step, cold_steps, args.warmup, settle=SETTLE_S) / cold_steps
             except Exception:
                 cold = time_eager(torch, cold_step, cold_steps, args.warmup) / cold_steps
             torch.testing.assert_close(ys[ring - 1].float(), torch.matmul(xs[ring - 1].float(), dense.weight.float().t()),

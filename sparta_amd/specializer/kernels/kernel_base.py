@@ -104,6 +104,10 @@ class KernelBase(abc.ABC):
         self._func: Optional[Callable] = None
         self.ports: Dict[str, PortConfig] = {}
         self.ready = False
+        # A TILE_CFG that the library refuses for the shapes of a call (a tuned table entry used
+        # on other shapes) gives way to the library's own choice - except inside test(), where
+        # the tuner must see the refusal as a failed trial.
+        self._tile_strict = False
         self._add_parameters()
         self._set_ports()
 
@@ -239,7 +243,11 @@ class KernelBase(abc.ABC):
         target = self.reference(*sample)
         targets = list(target) if isinstance(target, tuple) else [target]
         self._convert_data(sample, targets)
-        return profile(self, sample, targets, num_warmups, num_iters, cuda)
+        self._tile_strict = True
+        try:
+            return profile(self, sample, targets, num_warmups, num_iters, cuda)
+        finally:
+            self._tile_strict = False
 
     def __call__(self, *args) -> torch.Tensor:
         if not self.ready:

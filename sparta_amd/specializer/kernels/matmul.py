@@ -171,6 +171,7 @@ class SparseMatMulKernel(KernelBase):
         # what this closure's kernel walks behind each pointer: a compressed operand laid out
         # by another index (other block shape, other mask) is refused before the launch
         extent = matmul_extent(self._mode, bool(compressed), batch_size, M, K, N, sparse_stride)
+        tile = [tile_cfg]   # tile variant (low 16 bits) | epilogue flags; see the retry below
 
         def matmul_func(A: torch.Tensor, B: torch.Tensor, bias: torch.Tensor = None,
                         _keepalive=(indexes, ptr, idx, sched)):
@@ -179,11 +180,20 @@ class SparseMatMulKernel(KernelBase):
             C = alloc(C_shape, dtype=A.dtype, device=A.device)
             if bias is not None:
                 bias = bias.to(A.dtype).contiguous()
-            rc = lib.spx_matmul(
-                mode_code, _lib.dtype_code(A.dtype), tA, tB, compressed,
-                _lib.dev_ptr(A.contiguous()), _lib.dev_ptr(B.contiguous()), _lib.dev_ptr(bias), _lib.dev_ptr(C),
-                ptr_p, idx_p, idx_kind, sched_p, nnz, nnz_dev_p, sparse_stride,
-                batch_size, M, K, N, BM, BK, BN, tile_cfg, _lib.current_stream(A.device))
+            A, B = A.contiguous(), B.contiguous()
+            cfg = tile[0]
+            while True:
+                rc = lib.spx_matmul(
+                    mode_code, _lib.dtype_code(A.dtype), tA, tB, compressed,
+                    _lib.dev_ptr(A), _lib.dev_ptr(B), _lib.dev_ptr(bias), _lib.dev_ptr(C),
+                    ptr_p, idx_p, idx_kind, sched_p, nnz, nnz_dev_p, sparse_stride,
+                    batch_size, M, K, N, BM, BK, BN, cfg, _lib.current_stream(A.device))
+                if rc == _lib.E_CONFIG and cfg & 0xffff and not self._tile_strict:
+                    # the configured tile variant does not take these shapes (nothing was
+                    # launched): the library's own choice from here on
+                    cfg = tile[0] = cfg & ~0xffff
+                    continue
+                break
             _lib.check(rc, 'spx_matmul')
             return C
 

@@ -103,6 +103,7 @@ class SparseSoftmaxForwardKernel(SparseSoftmaxKernel):
         lib = _lib.load()
 
         numel = batch_size * stride
+        tile = [tile_cfg]
         if mask is not None:
             require_numel('spx_softmax_forward', 'mask', mask, stride)
 
@@ -111,10 +112,16 @@ class SparseSoftmaxForwardKernel(SparseSoftmaxKernel):
             y = alloc(shape, dtype=x.dtype, device=x.device)
             if y.numel() == 0:  # no live block: nothing to compute
                 return y
-            rc = lib.spx_softmax_forward(
-                _lib.dtype_code(x.dtype), compressed, _lib.dev_ptr(x.contiguous()), _lib.dev_ptr(y),
-                _lib.dev_ptr(row_ptr), _lib.dev_ptr(idx), _lib.dev_ptr(mask), float(T),
-                batch_size, H, W, BH, BW, stride, tile_cfg, _lib.current_stream(x.device))
+            x = x.contiguous()
+            while True:
+                rc = lib.spx_softmax_forward(
+                    _lib.dtype_code(x.dtype), compressed, _lib.dev_ptr(x), _lib.dev_ptr(y),
+                    _lib.dev_ptr(row_ptr), _lib.dev_ptr(idx), _lib.dev_ptr(mask), float(T),
+                    batch_size, H, W, BH, BW, stride, tile[0], _lib.current_stream(x.device))
+                if rc == _lib.E_CONFIG and tile[0] and not self._tile_strict:
+                    tile[0] = 0   # the configured variant does not take this dtype / block width
+                    continue
+                break
             _lib.check(rc, 'spx_softmax_forward')
             return y
 
@@ -148,6 +155,7 @@ class SparseSoftmaxBackwardKernel(SparseSoftmaxKernel):
         lib = _lib.load()
 
         numel = batch_size * stride
+        tile = [tile_cfg]
         if mask is not None:
             require_numel('spx_softmax_backward', 'mask', mask, stride)
 
@@ -158,11 +166,16 @@ class SparseSoftmaxBackwardKernel(SparseSoftmaxKernel):
             grad_x = alloc(shape, dtype=grad_y.dtype, device=grad_y.device)
             if grad_x.numel() == 0:
                 return grad_x
-            rc = lib.spx_softmax_backward(
-                _lib.dtype_code(grad_y.dtype), compressed, _lib.dev_ptr(grad_y.contiguous()),
-                _lib.dev_ptr(y.contiguous()), _lib.dev_ptr(grad_x),
-                _lib.dev_ptr(row_ptr), _lib.dev_ptr(idx), _lib.dev_ptr(mask), float(T),
-                batch_size, H, W, BH, BW, stride, tile_cfg, _lib.current_stream(grad_y.device))
+            grad_y, y = grad_y.contiguous(), y.contiguous()
+            while True:
+                rc = lib.spx_softmax_backward(
+                    _lib.dtype_code(grad_y.dtype), compressed, _lib.dev_ptr(grad_y), _lib.dev_ptr(y), _lib.dev_ptr(grad_x),
+                    _lib.dev_ptr(row_ptr), _lib.dev_ptr(idx), _lib.dev_ptr(mask), float(T),
+                    batch_size, H, W, BH, BW, stride, tile[0], _lib.current_stream(grad_y.device))
+                if rc == _lib.E_CONFIG and tile[0] and not self._tile_strict:
+                    tile[0] = 0
+                    continue
+                break
             _lib.check(rc, 'spx_softmax_backward')
             return grad_x
 

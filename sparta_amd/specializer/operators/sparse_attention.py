@@ -131,6 +131,7 @@ class SparseAttention(OperatorBase):
         self._fused_mask = None
         self._inv_temperature = 1.0
         self._warned_unfused = False
+        self._tile_strict = False   # True while tune_tile_config times a variant: a refusal must show
         self.ready = False
 
     def _parts(self):
@@ -340,11 +341,16 @@ class SparseAttention(OperatorBase):
         out = torch.empty_like(q)
         self._check_operands('spx_attention_forward', indexes, batch, E, q_like=[('q', q)],
                              kv_like=[('k', k), ('v', v)], nnz=0)
-        rc = _lib.load().spx_attention_forward(
-            _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
-            _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(self._fused_mask),
-            float(self._inv_temperature), batch, self._Nt, self._Ns, E,
-            indexes.block_H, indexes.block_W, self._fused_tile_cfg, _lib.current_stream(q.device))
+        while True:
+            rc = _lib.load().spx_attention_forward(
+                _lib.dtype_code(q.dtype), _lib.dev_ptr(q), _lib.dev_ptr(k), _lib.dev_ptr(v), _lib.dev_ptr(out),
+                _lib.dev_ptr(indexes.row_ptr), _lib.dev_ptr(indexes._bcsr_buf), _lib.dev_ptr(self._fused_mask),
+                float(self._inv_temperature), batch, self._Nt, self._Ns, E,
+                indexes.block_H, indexes.block_W, self._fused_tile_cfg, _lib.current_stream(q.device))
+            if rc == _lib.E_CONFIG and self._fused_tile_cfg and not self._tile_strict:
+                self._fused_tile_cfg = 0   # a tuned variant that does not take these shapes: the library's choice
+                continue
+            break
         _lib.check(rc, 'spx_attention_forward')
         return out
 
@@ -424,14 +430,18 @@ class SparseAttention(OperatorBase):
             want = self._matmul_out.forward(self._softmax.forward(scores), value)
             del scores
             best_id, best_latency = 0, float('inf')
-            for tile in _lib.tile_configs(_lib.OP_ATTENTION):
-                self._fused_tile_cfg = tile['id']
-                try:
-                    latency = profile(self._fused_forward, [query, key, value], [want], num_warmups, num_iters, cuda=True)
-                except AssertionError:   # the configuration does not take this block shape / head dim
-                    latency = float('inf')
-                if latency < best_latency:
-                    best_id, best_latency = tile['id'], latency
+            self._tile_strict = True
+            try:
+                for tile in _lib.tile_configs(_lib.OP_ATTENTION):
+                    self._fused_tile_cfg = tile['id']
+                    try:
+                        latency = profile(self._fused_forward, [query, key, value], [want], num_warmups, num_iters, cuda=True)
+                    except AssertionError:   # the configuration does not take this block shape / head dim
+                        latency = float('inf')
+                    if latency < best_latency:
+                        best_id, best_latency = tile['id'], latency
+            finally:
+                self._tile_strict = False
         self._fused_tile_cfg = best_id
         return {'fused/forward': {'TILE_CFG': best_id}}
 

@@ -28,6 +28,7 @@ class DynamicSparseMoE(torch.nn.Module):
         super().__init__()
         _lib.load()
         self.tile_cfg = int(tile_cfg)
+        self._tile_strict = False   # True while tune_tile_config times a variant
         self.num_exps = len(exp_modules)
         self.out_hidden, self.in_hidden = exp_modules[0].weight.shape
         self.device = exp_modules[0].weight.device
@@ -70,10 +71,16 @@ class DynamicSparseMoE(torch.nn.Module):
         weight = self.weight.detach()
         if weight.dtype != tokens.dtype:
             weight = weight.to(tokens.dtype)
-        rc = lib.spx_moe_forward(_lib.dtype_code(tokens.dtype), _lib.dev_ptr(tokens),
-                                 _lib.dev_ptr(weight.contiguous()), 0, _lib.dev_ptr(out),
-                                 _lib.dev_ptr(self.expert_offset), _lib.dev_ptr(self.sparse_index),
-                                 n_tok, self.in_hidden, self.out_hidden, self.num_exps, self.tile_cfg, stream)
+        weight = weight.contiguous()
+        while True:
+            rc = lib.spx_moe_forward(_lib.dtype_code(tokens.dtype), _lib.dev_ptr(tokens),
+                                     _lib.dev_ptr(weight), 0, _lib.dev_ptr(out),
+                                     _lib.dev_ptr(self.expert_offset), _lib.dev_ptr(self.sparse_index),
+                                     n_tok, self.in_hidden, self.out_hidden, self.num_exps, self.tile_cfg, stream)
+            if rc == _lib.E_CONFIG and self.tile_cfg and not self._tile_strict:
+                self.tile_cfg = 0   # a tuned variant that does not take this dtype: the library's choice
+                continue
+            break
         _lib.check(rc, 'spx_moe_forward')
         return out
 
@@ -95,13 +102,17 @@ class DynamicSparseMoE(torch.nn.Module):
                 rows = exp_ids == e
                 want[rows] = torch.matmul(tokens[rows].float(), self.weight[e].float()).to(tokens.dtype)
             best_id, best_latency = 0, float('inf')
-            for tile in _lib.tile_configs(_lib.OP_MOE):
-                self.tile_cfg = tile['id']
-                try:
-                    latency = profile(self.forward, [tokens, exp_ids], [want], num_warmups, num_iters, cuda=True)
-                except AssertionError:   # the configuration does not take this dtype / layout
-                    latency = float('inf')
-                if latency < best_latency:
-                    best_id, best_latency = tile['id'], latency
+            self._tile_strict = True
+            try:
+                for tile in _lib.tile_configs(_lib.OP_MOE):
+                    self.tile_cfg = tile['id']
+                    try:
+                        latency = profile(self.forward, [tokens, exp_ids], [want], num_warmups, num_iters, cuda=True)
+                    except AssertionError:   # the configuration does not take this dtype / layout
+                        latency = float('inf')
+                    if latency < best_latency:
+                        best_id, best_latency = tile['id'], latency
+            finally:
+                self._tile_strict = False
         self.tile_cfg = best_id
         return {'forward': {'TILE_CFG': best_id}}
