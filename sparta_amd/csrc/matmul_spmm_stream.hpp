@@ -94,12 +94,35 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         int mt, j, e_begin, n_it;   // uniform
         int kb_vec, slot_vec;       // lane l: k-block and value slot of index entry l (first 64)
     };
+    // Up to 128 block-columns: the launch order and the column pointers sit in lane vectors,
+    // fetched by one round of independent loads at kernel start, so that a tile's look-up
+    // (order -> pointer pair) costs no memory round trip; the chain ahead of a slot's first
+    // operand loads is then two trips (these vectors, the index entries) instead of three.
+    const bool small_nb = nb <= 128;
+    int sv0 = 0, sv1 = 0, pv0 = 0, pv1 = 0, pv2 = 0;
+    if (small_nb) {
+        if (p.sched) {
+            if (lane < nb) sv0 = p.sched[lane];
+            if (64 + lane < nb) sv1 = p.sched[64 + lane];
+        }
+        if (lane <= nb) pv0 = p.ptr[lane];
+        if (64 + lane <= nb) pv1 = p.ptr[64 + lane];
+        if (nb == 128) pv2 = p.ptr[128];
+    }
+    auto ptr_at = [&](int i) {
+        return i < 64 ? __builtin_amdgcn_readlane(pv0, i) : (i < 128 ? __builtin_amdgcn_readlane(pv1, i - 64) : __builtin_amdgcn_readfirstlane(pv2));
+    };
     auto load_tile = [&](int g, Tile& t) {
         t.mt = g * kPanelXcd + xcd;
         const int o = (g & 1) ? nb - 1 - pos : pos;
-        t.j = p.sched ? p.sched[o] : o;
-        t.e_begin = p.ptr[t.j];
-        const int n_blk = p.ptr[t.j + 1] - t.e_begin;
+        if (small_nb) {
+            t.j = p.sched ? (o < 64 ? __builtin_amdgcn_readlane(sv0, o) : __builtin_amdgcn_readlane(sv1, o - 64)) : o;
+            t.e_begin = ptr_at(t.j);
+        } else {
+            t.j = p.sched ? p.sched[o] : o;
+            t.e_begin = p.ptr[t.j];
+        }
+        const int n_blk = (small_nb ? ptr_at(t.j + 1) : p.ptr[t.j + 1]) - t.e_begin;
         t.n_it = n_blk * CH;
         t.kb_vec = 0;
         t.slot_vec = 0;

@@ -157,6 +157,9 @@ def tune_sparse_module(module: OperatorBase, name: str, sample_inputs: List[torc
     return best_config
 
 
+_TILE_MARGIN = 0.97
+
+
 def refine_tile_configs(module: OperatorBase, name: str, config: Dict[str, Dict[str, Any]],
                         with_backward: bool = False) -> Dict[str, Dict[str, Any]]:
     """Second stage of a search that keeps the block sizes of `config`: every kernel that has
@@ -174,7 +177,7 @@ def refine_tile_configs(module: OperatorBase, name: str, config: Dict[str, Dict[
         op = placeholder.active_kernel()._tile_op()
         if op is None:
             continue
-        best_id, best_latency = 0, math.inf
+        best_id, best_latency, own_choice = 0, math.inf, math.inf
         for tile in _lib.tile_configs(op):
             trial = {k: v for k, v in params.items() if k != 'TILE_CFG'}
             trial['TILE_CFG'] = tile['id']
@@ -184,10 +187,22 @@ def refine_tile_configs(module: OperatorBase, name: str, config: Dict[str, Dict[
             except AssertionError:
                 latency = math.inf
             _logger.info(f'[{name}][Kernel: {kernel_name}] tile config {tile["id"]} ({tile["name"]}) => {latency} ms')
+            if tile['id'] == 0:
+                own_choice = latency
             if latency < best_latency:
                 best_id, best_latency = tile['id'], latency
         params.pop('TILE_CFG', None)
+        # A variant is only recorded when it beats the library's own choice by more than the
+        # noise of two timings of one kernel (the choice usually IS one of the variants).  The
+        # choice is timed once more at the end: it was the first trial after the block sizes
+        # changed, which the later trials were not.
         if best_id:
+            try:
+                placeholder.build({k: v for k, v in params.items()})
+                own_choice = min(own_choice, placeholder.test())
+            except AssertionError:
+                pass
+        if best_id and best_latency < _TILE_MARGIN * own_choice:
             params['TILE_CFG'] = best_id
     return refined
 
