@@ -16,6 +16,7 @@
 // Replaces convert_sparse_index / BATCH_BLOCK_SPARSE_MATMUL[_FP16] of the
 // reference (csrc/moe_sparse_forward_kernel.cu.j2:58-71,120-325,363-483), whose
 // grid is sized by the largest expert and whose fp16 path accumulates in fp16.
+#include <type_traits>
 #include "common.hpp"
 #include "mma.hpp"
 
@@ -654,7 +655,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
     const int wrow = wm * (TM / WGM), wcol = wn * (TN / WGN);
     // a partly filled tile: wavefronts whose rows are all past its end load their share of the
     // stages and meet the barriers, but read no fragments, issue no MFMAs and store nothing
-    const bool active = wrow < rows;
+    const bool active = __builtin_amdgcn_readfirstlane(wrow) < rows;
 
     const T* X = reinterpret_cast<const T*>(p.tokens);
     const T* W = reinterpret_cast<const T*>(p.weight) + (int64_t)expert * p.K * p.N;
@@ -770,9 +771,15 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                 }
             }
         };
+        // The walk exists twice, with and without the fragment reads and MFMAs, chosen once per
+        // wavefront: a test of `active` inside the k-steps splits them into basic blocks, and the
+        // compiler then waits for ALL fragment reads in flight ahead of a step's MFMAs instead of
+        // the older ones only - the reads of step c + 1 no longer run under the MFMAs of step c.
+        auto walk = [&](auto act) {
+        constexpr bool ACT = decltype(act)::value;
         wait_stages(n_st - 1 < NBUF - 2 ? n_st - 1 : NBUF - 2);
         __syncthreads();
-        if (active) read_frags(smem, smem + A_BYTES, 0, 0);
+        if constexpr (ACT) read_frags(smem, smem + A_BYTES, 0, 0);
         for (int s = 0; s < n_st; ++s) {
             const char* cur = smem + (s % NBUF) * BUF;
             const char* nxt = smem + ((s + 1) % NBUF) * BUF;
@@ -780,7 +787,7 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
 #pragma unroll
             for (int c = 0; c < KSTEPS; ++c) {
                 if (c + 1 < KSTEPS) {
-                    if (active) read_frags(cur, cur + A_BYTES, c + 1, (c + 1) & 1);
+                    if constexpr (ACT) read_frags(cur, cur + A_BYTES, c + 1, (c + 1) & 1);
                 } else if (s + 1 < n_st) {
                     // stage s + 1 has landed once only the stages after it are in flight; every
                     // fragment read of stage s has been issued by now, and is complete before
@@ -789,14 +796,14 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                     wait_stages(last - (s + 1));
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                     __syncthreads();
-                    if (active) read_frags(nxt, nxt + A_BYTES, 0, 0);
+                    if constexpr (ACT) read_frags(nxt, nxt + A_BYTES, 0, 0);
                 }
                 // the loads of stage s + NBUF - 1 reuse the buffer of stage s - 1, which the
                 // barrier inside stage s - 1 has freed
                 // (all of them in the first k-step, so that the wait above counts whole stages)
                 if (more && c == 0) issue_stage(s + NBUF - 1);
                 __builtin_amdgcn_sched_barrier(0);
-                if (active) {
+                if constexpr (ACT) {
 #pragma unroll
                     for (int i = 0; i < MTW; ++i)
 #pragma unroll
@@ -804,7 +811,12 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                 }
             }
         }
-    } else
+        };
+        if (active) walk(std::true_type{}); else walk(std::false_type{});
+    } else {
+    // (two copies of the walk, as above)
+    auto walk = [&](auto act) {
+    constexpr bool ACT = decltype(act)::value;
     for (int s = 0; s < n_st; ++s) {
         // stage s has landed once at most the loads of the stages after it are outstanding
         // (NBUF - 2 of them, fewer at the end of the walk)
@@ -848,23 +860,23 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                 }
             };
             constexpr int LPS = (L + KSTEPS - 1) / KSTEPS;  // loads per k-step
-            if (active) read_frags(0, 0);
+            if constexpr (ACT) read_frags(0, 0);
 #pragma unroll
             for (int c = 0; c < KSTEPS; ++c) {
-                if (active && c + 1 < KSTEPS) read_frags(c + 1, (c + 1) & 1);
+                if constexpr (ACT) if (c + 1 < KSTEPS) read_frags(c + 1, (c + 1) & 1);
                 if (more) {
 #pragma unroll
                     for (int q = c * LPS; q < (c + 1) * LPS && q < L; ++q) issue_one(s + NBUF - 1, q);
                 }
                 __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of this step's MFMAs
-                if (active) {
+                if constexpr (ACT) {
 #pragma unroll
                     for (int i = 0; i < MTW; ++i)
 #pragma unroll
                         for (int t = 0; t < NTW; ++t) accw[i][t] = MmaW<T>::mma(bf[c & 1][t], af[c & 1][i], accw[i][t]);
                 }
             }
-        } else if (active) {
+        } else if constexpr (ACT) {
 #pragma unroll
             for (int kc = 0; kc < KT; kc += 16) {
                 typename Mma16<T>::frag af[MT], bf[NTT];
@@ -880,6 +892,9 @@ __global__ __launch_bounds__(64 * WAVES, (TM + TN) * NBUF * KTB > 80 * 1024 ? 1 
                     for (int t = 0; t < NTT; ++t) acc[i][t] = Mma16<T>::mma(bf[t], af[i], acc[i][t]);
             }
         }
+    }
+    };
+    if (active) walk(std::true_type{}); else walk(std::false_type{});
     }
     __syncthreads();   // the epilogue reuses the LDS buffers
     if (!active) return;   // no barrier follows
