@@ -32,6 +32,8 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     constexpr int SH_BYTES = 2 * BN * 64;  // shared, double-buffered S tile
     constexpr int E16 = 16 / (int)sizeof(T);
     static_assert(BK % KC == 0, "block depth must be a multiple of the step");
+    // store instructions of one full tile's epilogue, per wavefront
+    constexpr int kTileStores = SWAP ? 4 * ((16 * (BN / E16) + 63) / 64) : NT * ((16 * (64 / E16) + 63) / 64);
 
     __shared__ __align__(16) char lds_all[4 * ROWS * 64 + SH_BYTES];
 
@@ -70,7 +72,10 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     // shared S tile: this wave stages chunks wave*BN .. wave*BN+BN-1 of the BN*4 chunks
     // (k-contiguous S: chunk = (n row, 16-byte piece of its 64 bytes of k); otherwise a chunk
     // is 16 bytes of n at one k and is transposed on its way into LDS)
-    const int sh_chunk = wave * BN + lane;
+    // (lanes past BN fetch the chunk of lane % BN once more - the same cache lines - and do not
+    // write it to LDS: every load instruction below is then issued by every wavefront on every
+    // path, which the explicit wait counts rely on)
+    const int sh_chunk = wave * BN + (lane & (BN - 1));
     const int sh_row = sh_chunk >> 2, sh_chk = sh_chunk & 3;
     const bool sh_active = lane < BN;
     const int sh_k = sh_chunk / (BN / E16), sh_n0 = (sh_chunk % (BN / E16)) * E16;
@@ -87,7 +92,7 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         bofs[t] = row * 64 + ((g4 ^ ((row >> 2) & 3)) << 4);
     }
     const int64_t sld = p.compressed ? (p.s_kcontig ? BK : BN) : p.s_ld;
-    const int64_t sh_toff = p.s_kcontig ? (int64_t)sh_row * sld + sh_chk * E16 : (int64_t)sh_k * sld + sh_n0;
+    const int sh_boff = (int)((p.s_kcontig ? (int64_t)sh_row * sld + sh_chk * E16 : (int64_t)sh_k * sld + sh_n0) * (int64_t)sizeof(T));
 
     // ---- per-tile state: the tile being computed and the one after it -------------------
     struct Tile {
@@ -143,8 +148,21 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
 
     // Loads of one step of tile t into a stage (dreg: 4 x 16 bytes of D per lane, sreg: this
     // lane's piece of the shared S block).  A step past the end (live == false) loads one
-    // fixed line per instruction and is never accumulated: the number of loads in flight is
-    // the same on every path, so each wait covers only the oldest stage.
+    // fixed line per instruction and is never accumulated: every call issues exactly
+    // kStageLoads load instructions, on every path.
+    //
+    // The loads go out through inline assembly and are waited for with explicit counts.  Left to
+    // the compiler, the wait counts of the two stages are merged at the loop header and every
+    // second step drains ALL loads in flight - the lead of the second stage, which is there to
+    // cover a load that takes longer than one step, is lost.  Each load takes a scalar base (the
+    // tile's first row plus the k offset, or the S block) and a 32-bit lane offset.
+    constexpr int kStageLoads = 5;
+    auto uniform_base = [](const void* ptr) {
+        const uint64_t v = (uint64_t)ptr;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return ((uint64_t)hi << 32) | lo;
+    };
     auto issue = [&](const Tile& t, int it, bool live, u32x4 (&dreg)[4], u32x4& sreg) {
         const int er = it / CH;
         const int ch = it % CH;
@@ -162,30 +180,41 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
             slot = t.e_begin + er;
         }
         const int koff = kb * BK + ch * KC;
-        // buffer loads: the tile's first row is the (scalar) base, the k offset a scalar
-        // offset and the lane's place in the tile a 32-bit register - no 64-bit address
-        // arithmetic per load.  A step that is not live reads the tile's first bytes.
-        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<T*>(D + (int64_t)(live ? t.mt : 0) * 256 * p.d_ld), 0, 0x7fffffff, 0x00020000);
-        const int soff = live ? koff * (int)sizeof(T) : 0;
+        // A step that is not live reads the first bytes of the dense operand.
+        const uint64_t dbase = uniform_base(live ? D + (int64_t)t.mt * 256 * p.d_ld + koff : D);
+        int voff[4];
         if (live && t.mt == n_mtiles - 1 && last_rows < 256) {
             // partial last m-tile: rows past the end re-read its last row
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int row = wave * 64 + q * 16 + lrow;
-                const int voff = ((row < last_rows ? row : last_rows - 1) * (int)p.d_ld + lchk * E16) * (int)sizeof(T);
-                dreg[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+                voff[q] = ((row < last_rows ? row : last_rows - 1) * (int)p.d_ld + lchk * E16) * (int)sizeof(T);
             }
         } else {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) dreg[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live ? roff[q] : 0, soff, 0);
+            for (int q = 0; q < 4; ++q) voff[q] = live ? roff[q] : 0;
         }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dreg[q]) : "v"(voff[q]), "s"(dbase) : "memory");
         const T* sblk = p.compressed ? S + slot * (int64_t)(BK * BN) + (p.s_kcontig ? ch * KC : ch * KC * BN)
                                      : (p.s_kcontig ? S + (int64_t)t.j * BN * p.s_ld + koff
                                                     : S + (int64_t)koff * p.s_ld + (int64_t)t.j * BN);
         // an idle step reads the first bytes of the dense operand: the sparse operand may be NULL
         // when no block is live (every step of every tile is idle then)
-        if (sh_active) sreg = *reinterpret_cast<const u32x4*>(live ? sblk + sh_toff : D);
+        const uint64_t sbase = uniform_base(live ? (const void*)sblk : (const void*)D);
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sreg) : "v"(live ? sh_boff : 0), "s"(sbase) : "memory");
+    };
+    // Wait until at most `newer` vector-memory instructions issued after this stage's loads are
+    // still outstanding (they retire in order); the stage's registers pass through the statement
+    // so that no use is scheduled ahead of it.  `newer` may undercount (a stricter wait), never
+    // overcount.
+    auto wait_stage = [&](u32x4 (&dreg)[4], u32x4& sreg, bool behind_stores) {
+        if (behind_stores) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads + kTileStores) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads) : "memory");
+#pragma unroll
+        for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(dreg[q]));
+        asm volatile("" : "+v"(sreg));
     };
 
     f32x4 acc[4][NT];
@@ -194,7 +223,10 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
 
     // One step: stage -> LDS, refill the stage with the step two ahead (which may belong to
     // the next tile), barrier for the shared S tile, MFMAs.
-    auto step = [&](int it, int n_pad, bool have_next, u32x4 (&dreg)[4], u32x4& sreg) {
+    auto step = [&](int it, int n_pad, bool have_next, bool behind_stores, u32x4 (&dreg)[4], u32x4& sreg) {
+        // the other stage's loads are newer than this one's - and, in the first two steps of a
+        // tile, the stores of the tile before it (all of them issued if that tile was a full one)
+        wait_stage(dreg, sreg, behind_stores && it < 2);
 #pragma unroll
         for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(lds + wofs[q]) = dreg[q];
         char* sdst = wsh + (it & 1) * (BN * 64);
@@ -213,15 +245,20 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
             }
         }
         {
+            // one call site: the compiler must not end up with two copies of the loads on
+            // different paths, so the tile is selected first
             const int ahead = it + 2;
-            if (ahead < n_pad) {
-                const bool live = ahead < cur.n_it;
-                issue(cur, live ? ahead : 0, live, dreg, sreg);
-            } else {
-                const int nit = ahead - n_pad;
-                const bool live = have_next && nit < nxt.n_it;
-                issue(nxt, live ? nit : 0, live, dreg, sreg);
-            }
+            const bool in_cur = ahead < n_pad;
+            const int ait = in_cur ? ahead : ahead - n_pad;
+            Tile t;
+            t.mt = in_cur ? cur.mt : nxt.mt;
+            t.j = in_cur ? cur.j : nxt.j;
+            t.e_begin = in_cur ? cur.e_begin : nxt.e_begin;
+            t.n_it = in_cur ? cur.n_it : nxt.n_it;
+            t.kb_vec = in_cur ? cur.kb_vec : nxt.kb_vec;
+            t.slot_vec = in_cur ? cur.slot_vec : nxt.slot_vec;
+            const bool live = (in_cur || have_next) && ait < t.n_it;
+            issue(t, live ? ait : 0, live, dreg, sreg);
         }
         __syncthreads();  // the S tile of this step is complete
         if (it < cur.n_it) {
@@ -245,6 +282,7 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     T* out = reinterpret_cast<T*>(p.out) + b * p.o_batch;
     T* eT = reinterpret_cast<T*>(lds);
 
+    bool behind_stores = false;
     for (int g = 0; g < n_tiles; ++g) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -255,9 +293,11 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         const int n_pad = cur.n_it < 2 ? 2 : (cur.n_it + 1) & ~1;
         const bool have_next = g + 1 < n_tiles;
         for (int it = 0; it < n_pad; it += 2) {
-            step(it, n_pad, have_next, d0, s0);
-            step(it + 1, n_pad, have_next, d1, s1);
+            step(it, n_pad, have_next, behind_stores, d0, s0);
+            step(it + 1, n_pad, have_next, behind_stores, d1, s1);
         }
+        // a partial last m-tile stores from some of its wavefronts only
+        behind_stores = !(cur.mt == n_mtiles - 1 && last_rows < 256);
 
         // ---- epilogue of tile g: registers -> private LDS -> 16-byte row-contiguous stores
         // (LDS instructions of one wave execute in order, so the region can be reused
@@ -376,8 +416,10 @@ template <typename T>
 bool spmm_stream_supported(const SpmmParams& p, int BN) {
     const int kc = 64 / (int)sizeof(T);
     // element offsets inside a 256-row tile are kept in 32 bits
+    // (and so is a lane's byte offset inside the rows of an uncompressed sparse operand)
     return p.d_kcontig && p.BK % kc == 0 && (BN == 16 || BN == 32 || BN == 64) &&
-           p.d_ld * 256 + 64 < (int64_t)0x7fffffff / (int)sizeof(T);
+           p.d_ld * 256 + 64 < (int64_t)0x7fffffff / (int)sizeof(T) &&
+           (p.compressed || p.s_ld * 64 + 64 < (int64_t)0x7fffffff / (int)sizeof(T));
 }
 
 template <typename T, int BN, int BK, bool SWAP>
