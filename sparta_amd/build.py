@@ -63,7 +63,7 @@ def _registers(token: str) -> set:
     return {int(m.group(1))} if m else set()
 
 
-def check_inflight_registers(asm: str) -> list:
+def check_inflight_registers_in_text_order(asm: str) -> list:
     """Scan device assembly for compiler-generated instructions that touch a VGPR between the
     inline-assembly load that targets it and the inline-assembly wait that covers it.
 
@@ -91,8 +91,9 @@ def check_inflight_registers(asm: str) -> list:
             in_asm = False
             continue
         if in_asm:
-            if text.startswith(('global_load_', 'buffer_load_')) and 'lds' not in text.split()[0]:
-                pending.append(_registers(text.split()[1].rstrip(',')))
+            if text.startswith(('global_load_', 'buffer_load_')):
+                # (a load that lands in LDS writes no register but takes its place in the queue)
+                pending.append(set() if 'lds' in text.split()[0] else _registers(text.split()[1].rstrip(',')))
             elif text.startswith('s_waitcnt') and 'vmcnt' in text:
                 n = int(re.search(r'vmcnt\((\d+)\)', text).group(1))
                 pending = pending[len(pending) - n:] if n else []
@@ -118,6 +119,146 @@ def check_inflight_registers(asm: str) -> list:
         if used & set().union(*pending):
             findings.append((kernel, number, text))
     return findings
+
+
+
+STRICT_MARKER = 'spx-uniform-waits'
+_LABEL, _WAIT, _ASM_LOAD, _END, _BRANCH, _CBRANCH, _MEM, _OTHER = range(8)
+
+
+def _parse_kernels(asm: str) -> list:
+    """[(kernel, [(line number, kind, payload, registers named)])] with inline-assembly text
+    reduced to its loads and waits.  Only kernels that carry the marker comment
+    ``spx-uniform-waits`` (emitted by the kernel source through an inline-assembly comment) are
+    returned."""
+    kernels, body, in_asm, marked = [], None, False, set()
+    for number, line in enumerate(asm.split('\n'), 1):
+        m = re.match(r'^(_Z\w+):', line)
+        if m:
+            body, in_asm = [], False
+            kernels.append((m.group(1), body))
+            continue
+        if body is None:
+            continue
+        label = re.match(r'^(\.L\w+):', line)
+        if label:
+            body.append((number, _LABEL, label.group(1), None))
+            continue
+        text = line.strip()
+        if STRICT_MARKER in text:
+            marked.add(id(body))
+            continue
+        if text.startswith(';;#ASMSTART'):
+            in_asm = True
+            continue
+        if text.startswith(';;#ASMEND'):
+            in_asm = False
+            continue
+        if not text or text[0] in '.;':
+            continue
+        text = text.split(';')[0].strip()
+        wait = re.search(r'vmcnt\((\d+)\)', text) if text.startswith('s_waitcnt') else None
+        if wait:
+            body.append((number, _WAIT, int(wait.group(1)), None))
+        elif in_asm:
+            if text.startswith(('global_load_', 'buffer_load_')):
+                # a load that lands in LDS writes no register but takes its place in the queue
+                to_lds = 'lds' in text.split()[0]
+                body.append((number, _ASM_LOAD, frozenset() if to_lds else frozenset(_registers(text.split()[1].rstrip(','))), None))
+            elif text.startswith(('global_store_', 'buffer_store_')):
+                body.append((number, _ASM_LOAD, frozenset(), None))
+        elif text.startswith(('s_endpgm', 's_setpc')):
+            body.append((number, _END, text, None))
+            if text.startswith('s_endpgm'):
+                body = None
+        else:
+            target = re.match(r's_(c?branch)\w*\s+(\.L\w+)', text)
+            if target:
+                body.append((number, _BRANCH if target.group(1) == 'branch' else _CBRANCH, target.group(2), None))
+                continue
+            used = set()
+            for token in re.findall(r'v\[\d+:\d+\]|v\d+', text):
+                used |= _registers(token)
+            kind = _MEM if text.startswith(('global_', 'buffer_', 'scratch_', 'flat_')) else _OTHER
+            if used or kind == _MEM:
+                body.append((number, kind, text, frozenset(used)))
+    return [(name, items) for name, items in kernels if id(items) in marked]
+
+
+def check_inflight_registers_along_control_flow(asm: str, max_states: int = 500000) -> list:
+    """The stricter check, for kernels that declare (marker comment ``spx-uniform-waits``) that
+    every path issues the same loads and waits with one fixed count per wait: compiler-generated
+    instructions that touch a VGPR between the inline-assembly load that targets it and the
+    wait that covers it, on ANY path - feasible or not, the walk does not evaluate conditions,
+    which is why a kernel has to be written for it.
+
+    Every kernel is walked along its control flow, not in text order: labels start blocks, a
+    conditional branch continues on both sides, an unconditional one only at its target, and a
+    (block, queue) pair is walked once.  The queue holds the vector-memory operations in
+    flight, oldest first: an inline ``global_load_*`` / ``buffer_load_*`` enters with its
+    destination registers, a memory instruction of the compiler's own with none;
+    ``s_waitcnt vmcnt(N)``, inline or not, leaves the N newest entries (vector memory
+    operations retire in order).  An instruction outside inline assembly that names a register
+    of a queued load is a finding - in particular code after a loop that reuses the registers
+    of loads the loop left in flight.  Returns a list of (kernel, line number, instruction).
+    """
+    findings, seen_findings = [], set()
+    for kernel, body in _parse_kernels(asm):
+        if not any(item[1] == _ASM_LOAD and item[2] for item in body):
+            continue
+        labels = {item[2]: i for i, item in enumerate(body) if item[1] == _LABEL}
+        work, visited = [(0, ())], set()
+        while work:
+            if len(visited) > max_states:
+                raise RuntimeError(f'{kernel}: too many (block, queue) states while checking the register prefetch')
+            pos, pending = work.pop()
+            pending = list(pending)
+            busy = frozenset().union(*pending) if pending else frozenset()
+            while pos < len(body):
+                number, kind, payload, used = body[pos]
+                pos += 1
+                if kind == _OTHER:
+                    if busy and used & busy and (kernel, number) not in seen_findings:
+                        seen_findings.add((kernel, number))
+                        findings.append((kernel, number, payload))
+                elif kind == _LABEL:
+                    # entries older than the oldest pending load carry no information
+                    # (and the counter itself holds 63: older operations have retired)
+                    pending = pending[-63:]
+                    while pending and not pending[0]:
+                        pending.pop(0)
+                    key = (payload, tuple(pending))
+                    if key in visited:
+                        break
+                    visited.add(key)
+                elif kind == _WAIT:
+                    pending = pending[len(pending) - payload:] if payload else []
+                    busy = frozenset().union(*pending) if pending else frozenset()
+                elif kind == _ASM_LOAD:
+                    pending.append(payload)
+                    busy = busy | payload
+                elif kind == _MEM:
+                    if busy:
+                        if used & busy and (kernel, number) not in seen_findings:
+                            seen_findings.add((kernel, number))
+                            findings.append((kernel, number, payload))
+                        pending.append(frozenset())   # takes a place in the same queue
+                elif kind == _CBRANCH:
+                    if payload in labels:
+                        work.append((labels[payload], tuple(pending)))
+                elif kind == _BRANCH:
+                    if payload in labels:
+                        work.append((labels[payload], tuple(pending)))
+                    break
+                else:   # _END
+                    break
+    return findings
+
+
+def check_inflight_registers(asm: str) -> list:
+    """Both checks of the register prefetch: every kernel in text order, and the kernels that
+    declare uniform wait counts (the marker comment) along their control flow as well."""
+    return check_inflight_registers_in_text_order(asm) + check_inflight_registers_along_control_flow(asm)
 
 
 def _compile_checked(src: str, obj: str) -> None:

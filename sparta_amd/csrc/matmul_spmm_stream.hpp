@@ -17,6 +17,7 @@
 // Step, LDS layout, fragment mapping and epilogue are those of the panel kernel with the
 // sparse block shared by the four wavefronts (one barrier per step).
 #pragma once
+#include <type_traits>
 #include "matmul_spmm_panel.hpp"
 
 namespace spx {
@@ -32,8 +33,6 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     constexpr int SH_BYTES = 2 * BN * 64;  // shared, double-buffered S tile
     constexpr int E16 = 16 / (int)sizeof(T);
     static_assert(BK % KC == 0, "block depth must be a multiple of the step");
-    // store instructions of one full tile's epilogue, per wavefront
-    constexpr int kTileStores = SWAP ? 4 * ((16 * (BN / E16) + 63) / 64) : NT * ((16 * (64 / E16) + 63) / 64);
 
     __shared__ __align__(16) char lds_all[4 * ROWS * 64 + SH_BYTES];
 
@@ -157,6 +156,9 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     // cover a load that takes longer than one step, is lost.  Each load takes a scalar base (the
     // tile's first row plus the k offset, or the S block) and a 32-bit lane offset.
     constexpr int kStageLoads = 5;
+    // (marker for the build's check of the assembly: this kernel's waits are to be verified along
+    // every path of its control flow, not only in text order)
+    asm volatile("; spx-uniform-waits");
     auto uniform_base = [](const void* ptr) {
         const uint64_t v = (uint64_t)ptr;
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
@@ -205,13 +207,14 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         const uint64_t sbase = uniform_base(live ? (const void*)sblk : (const void*)D);
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sreg) : "v"(live ? sh_boff : 0), "s"(sbase) : "memory");
     };
-    // Wait until at most `newer` vector-memory instructions issued after this stage's loads are
+    // Wait until at most NEWER vector-memory instructions issued after this stage's loads are
     // still outstanding (they retire in order); the stage's registers pass through the statement
-    // so that no use is scheduled ahead of it.  `newer` may undercount (a stricter wait), never
-    // overcount.
-    auto wait_stage = [&](u32x4 (&dreg)[4], u32x4& sreg, bool behind_stores) {
-        if (behind_stores) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads + kTileStores) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kStageLoads) : "memory");
+    // so that no use is scheduled ahead of it.  NEWER may undercount (a stricter wait), never
+    // overcount.  The count is a compile-time property of the call site - a run-time choice
+    // between two counts would put them on two paths of which a reader of the code (and the
+    // build's check of the assembly) cannot tell which one ran.
+    auto wait_stage = [&](auto newer, u32x4 (&dreg)[4], u32x4& sreg) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(newer)::value) : "memory");
 #pragma unroll
         for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(dreg[q]));
         asm volatile("" : "+v"(sreg));
@@ -223,10 +226,8 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
 
     // One step: stage -> LDS, refill the stage with the step two ahead (which may belong to
     // the next tile), barrier for the shared S tile, MFMAs.
-    auto step = [&](int it, int n_pad, bool have_next, bool behind_stores, u32x4 (&dreg)[4], u32x4& sreg) {
-        // the other stage's loads are newer than this one's - and, in the first two steps of a
-        // tile, the stores of the tile before it (all of them issued if that tile was a full one)
-        wait_stage(dreg, sreg, behind_stores && it < 2);
+    auto step = [&](auto newer, int it, int n_pad, bool have_next, u32x4 (&dreg)[4], u32x4& sreg) {
+        wait_stage(newer, dreg, sreg);
 #pragma unroll
         for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(lds + wofs[q]) = dreg[q];
         char* sdst = wsh + (it & 1) * (BN * 64);
@@ -282,7 +283,11 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     T* out = reinterpret_cast<T*>(p.out) + b * p.o_batch;
     T* eT = reinterpret_cast<T*>(lds);
 
-    bool behind_stores = false;
+    // The other stage's kStageLoads loads are newer than the ones a step waits for.  In the first
+    // two steps of a tile so are the stores of the tile before it, a number that varies (a
+    // partial last m-tile stores from some of its wavefronts only): the count leaves them out,
+    // which only makes those two waits stricter.
+    typedef std::integral_constant<int, kStageLoads> InTile;
     for (int g = 0; g < n_tiles; ++g) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -293,11 +298,9 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         const int n_pad = cur.n_it < 2 ? 2 : (cur.n_it + 1) & ~1;
         const bool have_next = g + 1 < n_tiles;
         for (int it = 0; it < n_pad; it += 2) {
-            step(it, n_pad, have_next, behind_stores, d0, s0);
-            step(it + 1, n_pad, have_next, behind_stores, d1, s1);
+            step(InTile{}, it, n_pad, have_next, d0, s0);
+            step(InTile{}, it + 1, n_pad, have_next, d1, s1);
         }
-        // a partial last m-tile stores from some of its wavefronts only
-        behind_stores = !(cur.mt == n_mtiles - 1 && last_rows < 256);
 
         // ---- epilogue of tile g: registers -> private LDS -> 16-byte row-contiguous stores
         // (LDS instructions of one wave execute in order, so the region can be reused

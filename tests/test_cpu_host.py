@@ -424,3 +424,43 @@ def test_build_check_finds_registers_touched_while_loads_are_in_flight():
     assert check_inflight_registers(_listing(load_a + '\ts_branch .LBB0_2\n.LBB0_1:\n\tv_mov_b32_e32 v2, 0\n')) == []
     # a new kernel starts clean
     assert check_inflight_registers(_listing(load_a) + '_Z6otherv:\n\tv_mov_b32_e32 v2, 0\n\ts_endpgm\n') == []
+
+
+def test_build_check_follows_the_control_flow_of_kernels_that_ask_for_it():
+    """A kernel that carries the marker comment is also walked along its branches.  The case
+    the text-order scan cannot see: a loop leaves loads in flight, and the code behind the loop
+    (reached through the loop's branch, not by falling through) reuses their registers."""
+    from sparta_amd.build import (STRICT_MARKER, check_inflight_registers,
+                                  check_inflight_registers_along_control_flow,
+                                  check_inflight_registers_in_text_order)
+    marker = _asm(f'; {STRICT_MARKER}')
+    load = _asm('global_load_dwordx4 v[2:5], v[10:11], off')
+    wait1 = _asm('s_waitcnt vmcnt(1)')
+    loop = (load +                                   # two stages in flight ahead of the loop
+            _asm('global_load_dwordx4 v[6:9], v[12:13], off') +
+            '.LBB0_1:\n' +
+            wait1 + '\tds_write_b128 v30, v[2:5]\n' + load +
+            wait1 + '\tds_write_b128 v30, v[6:9]\n' + _asm('global_load_dwordx4 v[6:9], v[12:13], off') +
+            '\ts_cbranch_scc1 .LBB0_3\n'
+            '\ts_branch .LBB0_1\n'
+            '.LBB0_2:\n'
+            '\tv_mov_b32_e32 v40, 0\n'
+            '.LBB0_3:\n')
+    reuse = '\tv_lshlrev_b32_e32 v6, 4, v39\n'       # the epilogue takes a ring register
+    drain = _asm('s_waitcnt vmcnt(0)')
+    bad, good = _listing(marker + loop + reuse), _listing(marker + loop + drain + reuse)
+    assert check_inflight_registers_in_text_order(bad) == []
+    found = check_inflight_registers_along_control_flow(bad)
+    assert [t for _, _, t in found] == ['v_lshlrev_b32_e32 v6, 4, v39']
+    assert check_inflight_registers(good) == []
+    # without the marker the kernel is only scanned in text order
+    assert check_inflight_registers(_listing(loop + reuse)) == []
+    # a load that lands in LDS writes no register but counts: behind it vmcnt(1) still covers v[2:5]
+    lds = _asm('s_mov_b32 m0, s4', 'global_load_lds_dwordx4 v[14:15], off')
+    assert check_inflight_registers(_listing(marker + load + lds + wait1 + '\tds_write_b128 v30, v[2:5]\n')) == []
+    # two waits on two sides of a branch: the walk takes both sides, also the one that skips the wait
+    skipped = _listing(marker + load + '\ts_cbranch_scc1 .LBB0_5\n' + drain + '.LBB0_5:\n\tds_write_b128 v30, v[2:5]\n')
+    assert len(check_inflight_registers_along_control_flow(skipped)) == 1
+    # the walk ends: a loop without any wait keeps at most the 63 operations the counter holds
+    endless = _listing(marker + '.LBB0_1:\n' + load + '\ts_branch .LBB0_1\n')
+    assert check_inflight_registers_along_control_flow(endless) == []
