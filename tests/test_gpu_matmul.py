@@ -155,6 +155,22 @@ def test_matmul_persistent_kernel_walks_several_tiles(mode, compressed, dtype, b
              gran=blocks[:2] if mode == 'sdd' else (blocks[2], blocks[1]), sparsity=0.75, seed=17, tile_cfg=10)
 
 
+@pytest.mark.parametrize('mode', ['sdd', 'dsd'])
+@pytest.mark.parametrize('case', ['long columns', 'many columns'])
+def test_matmul_persistent_kernel_index_paths(mode, case, gpu):
+    """Tile config 10 off its common path: block columns of more than 64 live blocks (the entries
+    past the 64 that sit in a lane vector are read from the index at their step), and more than
+    128 block columns (launch order and column pointers are read per tile instead of sitting in
+    lane vectors)."""
+    if case == 'long columns':
+        blocks, sparse_rows, K, sparsity = (16, 32, 16), 64, 32 * 88, 0.12
+    else:
+        blocks, sparse_rows, K, sparsity = (16, 32, 16), 16 * 150, 128, 0.6
+    M, N = (600, sparse_rows) if mode == 'dsd' else (sparse_rows, 600)
+    run_case(gpu, mode, False, True, True, True, torch.float16, blocks, batch=1, M=M, K=K, N=N,
+             gran=(16, blocks[1]), sparsity=sparsity, seed=23, tile_cfg=10)
+
+
 @pytest.mark.parametrize('tile_cfg', [1, 2])
 @pytest.mark.parametrize('K', [128, 640])
 @pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (64, 32, 64)),
