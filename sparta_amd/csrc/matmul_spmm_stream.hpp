@@ -425,13 +425,30 @@ bool spmm_stream_supported(const SpmmParams& p, int BN) {
            (p.compressed || p.s_ld * 64 + 64 < (int64_t)0x7fffffff / (int)sizeof(T));
 }
 
+// 256-row tiles of the dense operand per launch.  The slots of an XCD drift apart as they walk
+// their tiles (block columns differ in length), and once they are spread over more than two row
+// panels of 2 MB the panels no longer share the XCD's 4 MB L2 with the sparse operand: measured
+// on the 4096 x 4096 weight of the headline shape, 4 tiles per slot cost 12.7 us each, 8 tiles
+// 16.3 and 16 tiles 21.6.  Longer operands are therefore walked in several launches.
+constexpr int kStreamTilesPerLaunch = 4 * kPanelXcd;
+
 template <typename T, int BN, int BK, bool SWAP>
-static int launch_spmm_stream_inst(const SpmmParams& p, int batch, hipStream_t st) {
-    const int n_mtiles = (p.Mc + 255) / 256;
-    const int64_t nblocks = (int64_t)kPanelXcd * (p.Nc / BN);
+static int launch_spmm_stream_inst(const SpmmParams& p0, int batch, hipStream_t st) {
+    const int64_t nblocks = (int64_t)kPanelXcd * (p0.Nc / BN);
     if (nblocks > 0x7fffffffLL) return fail(SPX_E_SHAPE, "problem too large for one launch");
-    hipLaunchKernelGGL((spmm_stream_kernel<T, BN, BK, SWAP>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st, p, n_mtiles);
-    SPX_LAUNCH_CHECK("spmm_stream_kernel");
+    const int total_tiles = (p0.Mc + 255) / 256;
+    for (int t0 = 0; t0 < total_tiles || t0 == 0; t0 += kStreamTilesPerLaunch) {
+        SpmmParams p = p0;
+        const int64_t m_begin = (int64_t)t0 * 256;
+        p.Mc = (int)(p0.Mc - m_begin < (int64_t)kStreamTilesPerLaunch * 256 ? p0.Mc - m_begin : (int64_t)kStreamTilesPerLaunch * 256);
+        // the chunk's first row of the dense operand, of the result, and of a bias along m
+        p.D = reinterpret_cast<const T*>(p0.D) + m_begin * p0.d_ld;
+        p.out = reinterpret_cast<T*>(p0.out) + (p0.out_ncontig ? m_begin * p0.o_ld : m_begin);
+        if (p0.bias && p0.bias_on_m) p.bias = reinterpret_cast<const T*>(p0.bias) + m_begin;
+        const int n_mtiles = (p.Mc + 255) / 256;
+        hipLaunchKernelGGL((spmm_stream_kernel<T, BN, BK, SWAP>), dim3((unsigned)nblocks, batch, 1), dim3(256), 0, st, p, n_mtiles);
+        SPX_LAUNCH_CHECK("spmm_stream_kernel");
+    }
     return 0;
 }
 

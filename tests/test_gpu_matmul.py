@@ -156,6 +156,18 @@ def test_matmul_persistent_kernel_walks_several_tiles(mode, compressed, dtype, b
 
 
 @pytest.mark.parametrize('mode', ['sdd', 'dsd'])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.float32])
+def test_matmul_persistent_kernel_long_operand_in_several_launches(mode, dtype, gpu):
+    """Tile config 10 walks a dense operand of more than thirty-two 256-row tiles in several
+    launches: thirty-four tiles here, the last one partial, with a bias (which runs along the
+    chunked dimension in one of the two modes)."""
+    dense_rows = 33 * 256 + 40
+    M, N = (dense_rows, 64) if mode == 'dsd' else (64, dense_rows)
+    run_case(gpu, mode, False, True, True, True, dtype, (32, 32, 32), batch=2, M=M, K=128, N=N,
+             gran=(32, 32), sparsity=0.5, seed=37, tile_cfg=10)
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd'])
 @pytest.mark.parametrize('case', ['long columns', 'many columns'])
 def test_matmul_persistent_kernel_index_paths(mode, case, gpu):
     """Tile config 10 off its common path: block columns of more than 64 live blocks (the entries
