@@ -152,6 +152,21 @@ def run(which, steps, warmup, time_graph, time_eager, attention_tile_cfg=0, brie
                 _emit(f'c2 {mode} 4096^3 fp16 32x32@95%', sec, flops=nnz * 2.0 * 4096 * 1024,
                       bytes_alg=2 * 4096 * 4096 * 2 + nnz * 2048, extra={'nnz_blocks': nnz})
             if not brief:
+                # the same product with the weight stored [K, N] (transpose_B = False)
+                k = SparTASparseMatMulKernel(mode='dsd', biased=False, transpose_A=False, transpose_B=False, compressed=True)
+                mask_kn = mask.t().contiguous()
+                k.ports['B'].set_mask(mask_kn)
+                k.set_shape(1, M, K, N)
+                k.compile(dict(cfg32))
+                idx = k.ports['B'].indexes
+                B_kn = B[0].t().contiguous()[None]
+                args = (A, idx.convert(B_kn))
+                want = torch.matmul(A[0].float(), B_kn[0].float() * mask_kn.float())
+                _close(torch, k(*args).reshape(want.shape), want, 'c2 dsd [K, N]')
+                del want
+                sec = timed(lambda: k(*args))
+                _emit('c2 dsd 4096^3 fp16 32x32@95%, weight stored [K, N]', sec, flops=idx.block_nnz * 2.0 * 4096 * 1024,
+                      bytes_alg=2 * 4096 * 4096 * 2 + idx.block_nnz * 2048, extra={'nnz_blocks': idx.block_nnz})
                 sec = timed(lambda: torch.matmul(A[0], B[0].t()))
                 _emit('c2 dense torch.matmul fp16 4096^3', sec, flops=2.0 * 4096 ** 3)
             from oracle import bcs

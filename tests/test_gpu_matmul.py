@@ -155,6 +155,20 @@ def test_matmul_persistent_kernel_walks_several_tiles(mode, compressed, dtype, b
              gran=blocks[:2] if mode == 'sdd' else (blocks[2], blocks[1]), sparsity=0.75, seed=17, tile_cfg=10)
 
 
+@pytest.mark.parametrize('compressed', [False, True])
+@pytest.mark.parametrize('dtype,blocks', [(torch.float16, (32, 32, 32)), (torch.bfloat16, (16, 32, 64)),
+                                          (torch.float32, (32, 16, 16))])
+def test_matmul_persistent_kernel_sparse_operand_stored_the_other_way(compressed, dtype, blocks, gpu):
+    """Tile config 10 with the sparse operand stored with its non-reduced dimension contiguous
+    (weight [K, N], transpose_B = False; sparse input [K, M], transpose_A = True): its blocks
+    are turned on their way into LDS."""
+    rows = 3 * 256 + 72
+    run_case(gpu, 'dsd', False, False, True, compressed, dtype, blocks, batch=2, M=rows, K=256, N=192,
+             gran=(blocks[1], blocks[2]), sparsity=0.7, seed=41, tile_cfg=10)
+    run_case(gpu, 'sdd', True, True, True, compressed, dtype, blocks, batch=2, M=192, K=256, N=rows,
+             gran=(blocks[1], blocks[0]), sparsity=0.7, seed=43, tile_cfg=10)
+
+
 @pytest.mark.parametrize('mode', ['sdd', 'dsd'])
 @pytest.mark.parametrize('dtype', [torch.float16, torch.float32])
 def test_matmul_persistent_kernel_long_operand_in_several_launches(mode, dtype, gpu):
