@@ -116,17 +116,22 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
     auto ptr_at = [&](int i) {
         return i < 64 ? __builtin_amdgcn_readlane(pv0, i) : (i < 128 ? __builtin_amdgcn_readlane(pv1, i - 64) : __builtin_amdgcn_readfirstlane(pv2));
     };
-    auto load_tile = [&](int g, Tile& t) {
+    // (The lane vectors serve the two tiles that are looked up at kernel start, where the round
+    // trip matters.  Later tiles are looked up a whole tile ahead and read the two arrays
+    // directly: the vectors do not have to stay in registers - or, as it turned out in one of
+    // the two output layouts, in scratch memory, each load waited for so that it could be
+    // spilled - for the rest of the kernel.)
+    auto load_tile = [&](int g, Tile& t, bool from_vectors) {
         t.mt = g * kPanelXcd + xcd;
         const int o = (g & 1) ? nb - 1 - pos : pos;
-        if (small_nb) {
+        if (from_vectors) {
             t.j = p.sched ? (o < 64 ? __builtin_amdgcn_readlane(sv0, o) : __builtin_amdgcn_readlane(sv1, o - 64)) : o;
             t.e_begin = ptr_at(t.j);
         } else {
             t.j = p.sched ? p.sched[o] : o;
             t.e_begin = p.ptr[t.j];
         }
-        const int n_blk = (small_nb ? ptr_at(t.j + 1) : p.ptr[t.j + 1]) - t.e_begin;
+        const int n_blk = (from_vectors ? ptr_at(t.j + 1) : p.ptr[t.j + 1]) - t.e_begin;
         t.n_it = n_blk * CH;
         t.kb_vec = 0;
         t.slot_vec = 0;
@@ -142,8 +147,8 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
         }
     };
     Tile cur, nxt;
-    load_tile(0, cur);
-    if (n_tiles > 1) load_tile(1, nxt); else nxt = cur;
+    load_tile(0, cur, small_nb);
+    if (n_tiles > 1) load_tile(1, nxt, small_nb); else nxt = cur;
 
     // Loads of one step of tile t into a stage (dreg: 4 x 16 bytes of D per lane, sreg: this
     // lane's piece of the shared S block).  A step past the end (live == false) loads one
@@ -411,7 +416,7 @@ __global__ __launch_bounds__(256, BN <= 32 ? 4 : 2) void spmm_stream_kernel(Spmm
 
         // ---- move on: tile g+1 becomes current, the index entries of tile g+2 are fetched --
         cur = nxt;
-        if (g + 2 < n_tiles) load_tile(g + 2, nxt);
+        if (g + 2 < n_tiles) load_tile(g + 2, nxt, false);
     }
 }
 
